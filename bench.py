@@ -1,0 +1,268 @@
+#!/usr/bin/env python3
+"""Benchmark of the reproducible-operator hot path on one MI355X.
+
+Headline (BASELINE.json `metric`): bit-exact fp32 `mm` GFLOP/s at 8192^3 -- the
+`repdl.nn.Linear` forward shape x[8192,8192] . W[8192,8192]^T (transB).  A "step"
+is one such product with the operands resident in HBM.  The same JSON line also
+carries, under "also", the HBM-bound operators of the metric (row-wise and 1-D
+sequential sums, exp, log, sqrt, div on 2^28 values), each with its own roofline
+entry, and under "parity" the SHA-256 comparison of the GPU outputs with the CPU
+checker on the same input bytes.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick] [--only mm]
+
+The CPU baseline is RepDL's own C++ CPU backend (compiled into oracle/_ref from
+the reference sources; kind "reference") when that build is present, otherwise
+the plain-C restatement (kind "port"), timed on a bounded sample of the same
+workload on the host cores.  Only the baseline and parity legs touch oracle/.
+"""
+from __future__ import annotations
+
+import argparse
+import hashlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FP32_PEAK_TFLOPS = 157.3  # MI355X vendor fp32 figure (256 CU x 2.4 GHz x 256 flop/clk)
+HBM_PEAK_GBS = 8000.0
+
+
+def sha(t) -> str:
+    return hashlib.sha256(t.detach().cpu().contiguous().numpy().tobytes()).hexdigest()
+
+
+def time_gpu(fn, steps: int, warmup: int):
+    """Returns (wall ms per step, mean kernel ms from events on the launch stream)."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        fn()
+        stops[i].record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    ev = [s.elapsed_time(e) for s, e in zip(starts, stops)]
+    return wall, sum(ev) / len(ev), min(ev)
+
+
+def hbm_entry(name, workload, algo_bytes, fn, steps, warmup, parity=None, cpu=None):
+    wall, ev_mean, ev_min = time_gpu(fn, steps, warmup)
+    gbs = algo_bytes / (ev_mean * 1e-3) / 1e9
+    out = {
+        "op": name,
+        "workload": workload,
+        "value": round(gbs, 2),
+        "unit": "GB/s",
+        "ms_per_step": round(ev_mean, 4),
+        "ms_min": round(ev_min, 4),
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+    }
+    if parity is not None:
+        out["parity"] = parity
+    if cpu is not None:
+        out["cpu_baseline"] = cpu
+    return out
+
+
+def cpu_time(fn, reps=1):
+    best = None
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        r = fn()
+        dt = time.perf_counter() - t0
+        best = dt if best is None or dt < best else best
+    return best, r
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--quick", action="store_true", help="headline only, no secondary operators, no full parity")
+    ap.add_argument("--only", default="", help="comma list of secondary ops to run (sum2d,sum1d,exp,log,sqrt,div)")
+    ap.add_argument("--size", type=int, default=8192, help="mm size (M=N=K); the metric is quoted at 8192")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (every operator shards by outputs with no "
+              "cross-device arithmetic; see DESIGN.md); run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    import repdl_amd
+    from repdl_amd import ops
+
+    from oracle import api as oracle  # checker / baseline legs only
+    from oracle import ref as oracle_ref
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    props = torch.cuda.get_device_properties(dev)
+    S = args.size
+    only = set(x for x in args.only.split(",") if x)
+
+    # ---------------- headline: mm S^3, Linear forward (NT) ----------------
+    g = torch.Generator().manual_seed(0)
+    x_h = torch.randn(S, S, generator=g)
+    bound = 1.0 / (S ** 0.5)  # torch.nn.Linear default init: U(-1/sqrt(in), 1/sqrt(in))
+    w_h = (torch.rand(S, S, generator=g) * 2 - 1) * bound
+    x_d, w_d = x_h.to(dev), w_h.to(dev)
+    out_holder = {}
+
+    def step():
+        out_holder["y"] = ops.mm(x_d, w_d, transB=True)
+
+    wall_ms, ev_ms, ev_min = time_gpu(step, args.steps, args.warmup)
+    flop = 2.0 * S * S * S
+    gflops = flop / (wall_ms * 1e-3) / 1e9
+    kern_tflops = flop / (ev_ms * 1e-3) / 1e12
+
+    # parity of the headline output against the CPU checker on the same bytes
+    parity = {}
+    y_gpu = out_holder["y"]
+    if not args.quick:
+        t0 = time.perf_counter()
+        y_cpu = oracle.mm(x_h, w_h, False, True)
+        parity["mm"] = {"sha256_gpu": sha(y_gpu), "sha256_cpu": sha(y_cpu), "checker": "oracle (C restatement)",
+                        "checker_s": round(time.perf_counter() - t0, 2)}
+        parity["mm"]["equal"] = parity["mm"]["sha256_gpu"] == parity["mm"]["sha256_cpu"]
+        del y_cpu
+
+    # CPU baseline: the reference's own CPU backend on a row slab of the same product
+    refmods = oracle_ref.load()
+    rows = 256 if not args.quick else 64
+    rows = min(rows, S)
+    if refmods is not None:
+        cpu_fn, kind = (lambda: refmods[0].mm(x_h[:rows], w_h, False, True)), "reference"
+    else:
+        cpu_fn, kind = (lambda: oracle.mm(x_h[:rows], w_h, False, True)), "port"
+    dt, y_slab = cpu_time(cpu_fn)
+    slab_equal = torch.equal(y_slab, y_gpu[:rows].cpu())
+    cpu_baseline = {
+        "value": round(2.0 * rows * S * S / dt / 1e9, 3), "unit": "GFLOP/s", "cores": oracle.threads(),
+        "kind": kind,
+        "sample": "first %d of %d output rows of the same %dx%dx%d NT product (%.1f s); GPU rows bit-equal: %s"
+                  % (rows, S, S, S, S, dt, slab_equal),
+    }
+    del x_d, w_d, y_gpu, out_holder
+
+    result = {
+        "metric": "bit-exact fp32 mm GFLOP/s at 8192^3",
+        "value": round(gflops, 1),
+        "unit": "GFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic (seeded host randn / uniform, same bytes for GPU and CPU checker)",
+        "config": {"workload": "repdl.ops.mm fp32 %dx%dx%d, transB (nn.Linear forward), configs[3]" % (S, S, S),
+                   "device": props.name, "cus": props.multi_processor_count},
+        "roofline": {"bound": "mfma", "achieved": round(kern_tflops, 3), "peak": FP32_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(kern_tflops / FP32_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "mm_kernel<NT>", "kernel_ms": round(ev_ms, 4), "kernel_ms_min": round(ev_min, 4),
+                     "note": "fp32 compute peak; the kernel issues scalar v_fma_f32 only (no MFMA, packed "
+                             "fp32 disabled), whose issue-rate ceiling is half of this peak"},
+        "cpu_baseline": cpu_baseline,
+        "parity": parity,
+        "also": [],
+    }
+
+    if not args.quick:
+        n = 1 << 28
+        want = lambda k: (not only) or (k in only)
+        sample = 1 << 24
+
+        if want("sum2d"):
+            R = 16384
+            g = torch.Generator().manual_seed(1)
+            m_h = torch.randn(R, R, generator=g) * torch.exp2(torch.rand(R, R, generator=g) * 40 - 20)
+            m_d = m_h.to(dev)
+            hold = {}
+            def f(): hold["y"] = ops.sum2d_dim1(m_d)
+            f()
+            y_cpu = oracle.sum2d_dim1(m_h)
+            par = {"equal": sha(hold["y"]) == sha(y_cpu), "sha256_gpu": sha(hold["y"])}
+            dt, _ = cpu_time(lambda: (refmods[0].sum2d_dim1(m_h[:2048], False, False) if refmods else oracle.sum2d_dim1(m_h[:2048])))
+            cpu = {"value": round(2048 * R * 4 / dt / 1e9, 3), "unit": "GB/s", "cores": oracle.threads(),
+                   "kind": kind, "sample": "first 2048 rows"}
+            result["also"].append(hbm_entry("sum2d_dim1", "row sums of 16384x16384 N(0,1)*2^U(-20,20)", 4.0 * R * R + 4 * R,
+                                            f, args.steps, args.warmup, par, cpu))
+            del m_d, m_h, hold
+
+        if want("sum1d"):
+            g = torch.Generator().manual_seed(2)
+            v_h = torch.rand(n, generator=g) * 2 - 1
+            v_d = v_h.to(dev)
+            hold = {}
+            def f(): hold["y"] = ops.sum1d(v_d)
+            f()
+            dt, y_cpu = cpu_time(lambda: (refmods[0].sum1d(v_h, False) if refmods else oracle.sum1d(v_h)))
+            par = {"equal": sha(hold["y"]) == sha(y_cpu), "gpu": float(hold["y"]), "cpu": float(y_cpu)}
+            cpu = {"value": round(n * 4 / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": kind,
+                   "sample": "the full 2^28 vector (the reference's sum1d is single-threaded)"}
+            result["also"].append(hbm_entry("sum1d", "sequential sum of 2^28 uniform[-1,1]", 4.0 * n, f,
+                                            max(2, args.steps // 5), 1, par, cpu))
+            del v_d, v_h, hold
+
+        ew = [k for k in ("exp", "log", "sqrt", "div") if want(k)]
+        if ew:
+            sys.path.insert(0, os.path.join(ROOT, "tests"))
+            import gen  # deterministic config-3 mix (90 % log-uniform, 10 % specials)
+
+            e_h = gen.elementwise_mix(3, n)
+            e_d = e_h.to(dev)
+            for k in ew:
+                hold = {}
+                if k == "div":
+                    fns = [("div_scalar", "x/10.0 on 2^28 mixed values", 8.0 * n, lambda: ops.div(e_d, 10.0),
+                            lambda t: oracle.div(t, 10.0), lambda t: t.div(10.0))]
+                    e2_h = gen.elementwise_mix(4, n)
+                    e2_d = e2_h.to(dev)
+                    fns.append(("div", "x/y on 2^28 mixed values", 12.0 * n, lambda: ops.div(e_d, e2_d), None,
+                                lambda t: t.div(e2_h[: t.numel()])))
+                else:
+                    fns = [(k, "%s on 2^28 mixed values" % k, 8.0 * n, (lambda kk: (lambda: getattr(ops, kk)(e_d)))(k),
+                            (lambda kk: (lambda t: getattr(oracle, kk)(t)))(k), None)]
+                for name, wl, nbytes, gfn, ofn, tfn in fns:
+                    def f(): hold["y"] = gfn()
+                    f()
+                    y_gpu_s = hold["y"][:sample].cpu()
+                    if ofn is None:
+                        y_cpu_s = oracle.div(e_h[:sample], e2_h[:sample])
+                        dt, _ = cpu_time(lambda: oracle.div(e_h[:sample], e2_h[:sample]))
+                    else:
+                        y_cpu_s = ofn(e_h[:sample])
+                        dt, _ = cpu_time(lambda: ofn(e_h[:sample]))
+                    par = {"equal_on_first_2^24": sha(y_gpu_s) == sha(y_cpu_s)}
+                    cpu = {"value": round(nbytes / n * sample / dt / 1e9, 3), "unit": "GB/s",
+                           "cores": oracle.threads(), "kind": "port", "sample": "first 2^24 elements"}
+                    result["also"].append(hbm_entry(name, wl, nbytes, f, args.steps, args.warmup, par, cpu))
+                    hold.clear()
+
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

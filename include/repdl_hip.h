@@ -1,0 +1,121 @@
+/*
+ * repdl_hip.h -- C ABI of the MI355X (gfx950) backend for RepDL's reproducible
+ * operators.
+ *
+ * This is the drop-in boundary: one entry point per function that RepDL's
+ * device backend module exports to repdl/ops.py (backend/cuda/bind.cpp:6-18 and
+ * the m.def lists cited below), plus the elementwise operators that RepDL
+ * composes from PyTorch calls (repdl/ops.py:98-103, 122-123) or keeps internal
+ * (backend/cpu/math.h:14-15).  Plain pointers and sizes only; no PyTorch types.
+ *
+ * Conventions
+ *   - All pointers are DEVICE pointers to contiguous row-major float32 data
+ *     (int64 for class labels) on the device that is current when the call is
+ *     made.  Outputs are caller-allocated.  Inputs are never written.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *     Calls enqueue work and return without synchronising.
+ *   - Return value: 0 on success; a positive value is a hipError_t from the
+ *     runtime; a negative value is one of the REPDL_E_* codes below.
+ *     repdl_hip_error_string() describes either kind.
+ *   - Arithmetic contract: binary32, round to nearest even, subnormals kept;
+ *     one accumulator per output element starting at +0.0f, updated by single
+ *     fused multiply-adds in the loop order of RepDL's CPU backend; results are
+ *     bit-identical to that backend for finite data.  (When a NaN is produced
+ *     inside a multiply-accumulate chain its sign and payload are unspecified;
+ *     the elementwise operators below define NaN bits exactly.)
+ */
+#ifndef REPDL_HIP_H
+#define REPDL_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define REPDL_OK 0
+#define REPDL_E_ARG (-1)         /* null pointer, negative size, size out of range */
+#define REPDL_E_UNSUPPORTED (-2) /* a combination the reference itself does not define */
+#define REPDL_E_WORKSPACE (-3)   /* workspace missing or too small */
+
+const char *repdl_hip_error_string(int code);
+int repdl_hip_abi_version(void);
+
+/* mm -- backend/cuda/matrix_multiplication.cu:234-260 (bound at :267);
+ * semantics backend/cpu/matrix_multiplication.cpp:12-36.
+ * C[M,N] = op(A) op(B); A is [M,K] (or [K,M] when transA), B is [K,N] (or [N,K]
+ * when transB); C(i,j) = fma(a_{K-1}, b_{K-1}, ... fma(a_0, b_0, +0)). */
+int repdl_hip_mm(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K,
+                 int transA, int transB, void *stream);
+
+/* conv2d -- backend/cuda/convolution.cu:153-183 (bound at :385); semantics
+ * backend/cpu/convolution.cpp:12-52.  NCHW; kernel is [OC, IC/groups, KH, KW];
+ * output is [N, OC, OH, OW] with OH = (H + 2 pH - KH) / sH + 1. */
+int repdl_hip_conv2d(const float *input, const float *kernel, float *output, int64_t N, int64_t IC,
+                     int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t sH,
+                     int64_t sW, int64_t pH, int64_t pW, int64_t groups, void *stream);
+
+/* conv2d_grad_input -- backend/cuda/convolution.cu:259-287 (bound at :386);
+ * semantics backend/cpu/convolution.cpp:54-90.  groups == 1.
+ * grad_output is [N, OC, OH, OW], kernel [OC, IC, KH, KW], grad_input [N, IC, H, W]. */
+int repdl_hip_conv2d_grad_input(const float *grad_output, const float *kernel, float *grad_input,
+                                int64_t N, int64_t OC, int64_t OH, int64_t OW, int64_t IC,
+                                int64_t KH, int64_t KW, int64_t H, int64_t W, int64_t sH,
+                                int64_t sW, int64_t pH, int64_t pW, void *stream);
+
+/* conv2d_grad_kernel -- backend/cuda/convolution.cu:359-383 (bound at :387);
+ * semantics backend/cpu/convolution.cpp:92-128.  groups == 1.
+ * grad_kernel is [OC, IC, KH, KW]. */
+int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float *input, float *grad_kernel,
+                                 int64_t N, int64_t IC, int64_t H, int64_t W, int64_t OC,
+                                 int64_t OH, int64_t OW, int64_t KH, int64_t KW, int64_t sH,
+                                 int64_t sW, int64_t pH, int64_t pW, void *stream);
+
+/* sums -- backend/cuda/summation.cu:33-147 (bound at :149-155); semantics
+ * backend/cpu/summation.cpp:12-78: strict left-to-right binary32 chains from
+ * +0.0f, then one multiply by (float)(average ? 1.0/count : 1.0).
+ *   sum1d:        out[0]    = sum_i in[i]                       (count n)
+ *   sum2d_dim0:   out[j]    = sum_i in[i][j],  in [M,N]         (count M)
+ *   sum2d_dim1:   out[i]    = sum_j in[i][j],  in [M,N]         (count N)
+ *   sum4d_dim023: out[c]    = sum_{n,h,w} in[n][c][h][w]        (count N*H*W) */
+int repdl_hip_sum1d(const float *in, float *out, int64_t n, int average, void *stream);
+int repdl_hip_sum2d_dim0(const float *in, float *out, int64_t M, int64_t N, int average,
+                         void *stream);
+int repdl_hip_sum2d_dim1(const float *in, float *out, int64_t M, int64_t N, int average,
+                         void *stream);
+int repdl_hip_sum4d_dim023(const float *in, float *out, int64_t N, int64_t C, int64_t H, int64_t W,
+                           int average, void *stream);
+
+/* exp, log -- backend/cuda/math.cu:15-18, 42-45 (drivers :30-39, :56-65; declared
+ * backend/cuda/math.h, not bound to Python by the reference); semantics
+ * backend/cpu/math.cpp:14-17, 32-35: (float)exp((double)x), (float)log((double)x)
+ * with glibc's binary64 routines.  Any number of elements. */
+int repdl_hip_exp(const float *in, float *out, int64_t n, void *stream);
+int repdl_hip_log(const float *in, float *out, int64_t n, void *stream);
+
+/* sqrt -- repdl/ops.py:122-123: float32(sqrt(float64(x))) == IEEE binary32 sqrt.
+ * Negative arguments give the quiet NaN 0x7FC00000 (PyTorch's CPU convention);
+ * NaN arguments keep sign and payload, quieted; sqrt(-0) = -0. */
+int repdl_hip_sqrt(const float *in, float *out, int64_t n, void *stream);
+
+/* div -- repdl/ops.py:98-103: IEEE binary32 quotient, elementwise, either by a
+ * second tensor of the same length or by one binary32 scalar (a true division,
+ * never a multiplication by the reciprocal).  NaN dividend wins over NaN
+ * divisor; 0/0 and inf/inf give 0xFFC00000. */
+int repdl_hip_div(const float *a, const float *b, float *out, int64_t n, void *stream);
+int repdl_hip_div_scalar(const float *a, float b, float *out, int64_t n, void *stream);
+
+/* softmax -- backend/cuda/softmax.cpp:15-21 (bound at :28); semantics
+ * backend/cpu/softmax.cpp:15-21.  in/out are [M,N]. */
+int repdl_hip_softmax(const float *in, float *out, int64_t M, int64_t N, void *stream);
+
+/* cross_entropy -- backend/cuda/cross_entropy.cpp:15-24 (bound at :31); semantics
+ * backend/cpu/cross_entropy.cpp:15-24.  in is [M,N], target is [M] int64 class
+ * indices in [0,N), out is one float.  workspace: M floats of device memory. */
+int repdl_hip_cross_entropy(const float *in, const int64_t *target, float *out, int64_t M,
+                            int64_t N, float *workspace, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* REPDL_HIP_H */

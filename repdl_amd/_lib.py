@@ -1,0 +1,74 @@
+"""ctypes binding of the C-ABI library ``librepdl_hip.so`` (include/repdl_hip.h).
+
+There is no fallback: if the library has not been built, or a call fails, an
+exception is raised.  PyTorch is used only for device memory and the current
+stream.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "librepdl_hip.so")
+
+_P = ctypes.c_void_p
+_I64 = ctypes.c_int64
+_INT = ctypes.c_int
+_F32 = ctypes.c_float
+
+# name -> argument types (all return int), exactly the declarations of repdl_hip.h
+SIGNATURES = {
+    "repdl_hip_mm": [_P, _P, _P, _I64, _I64, _I64, _INT, _INT, _P],
+    "repdl_hip_conv2d": [_P, _P, _P] + [_I64] * 12 + [_P],
+    "repdl_hip_conv2d_grad_input": [_P, _P, _P] + [_I64] * 13 + [_P],
+    "repdl_hip_conv2d_grad_kernel": [_P, _P, _P] + [_I64] * 13 + [_P],
+    "repdl_hip_sum1d": [_P, _P, _I64, _INT, _P],
+    "repdl_hip_sum2d_dim0": [_P, _P, _I64, _I64, _INT, _P],
+    "repdl_hip_sum2d_dim1": [_P, _P, _I64, _I64, _INT, _P],
+    "repdl_hip_sum4d_dim023": [_P, _P, _I64, _I64, _I64, _I64, _INT, _P],
+    "repdl_hip_exp": [_P, _P, _I64, _P],
+    "repdl_hip_log": [_P, _P, _I64, _P],
+    "repdl_hip_sqrt": [_P, _P, _I64, _P],
+    "repdl_hip_div": [_P, _P, _P, _I64, _P],
+    "repdl_hip_div_scalar": [_P, _F32, _P, _I64, _P],
+    "repdl_hip_softmax": [_P, _P, _I64, _I64, _P],
+    "repdl_hip_cross_entropy": [_P, _P, _P, _I64, _I64, _P, _P],
+}
+
+_lib = None
+
+
+class RepdlHipError(RuntimeError):
+    pass
+
+
+def lib() -> ctypes.CDLL:
+    """Load the library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RepdlHipError(
+                "%s is missing: build it with `python -m repdl_amd.build` (there is no CPU fallback)" % LIB_PATH
+            )
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, argtypes in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.argtypes = argtypes
+            fn.restype = _INT
+        handle.repdl_hip_error_string.argtypes = [_INT]
+        handle.repdl_hip_error_string.restype = ctypes.c_char_p
+        handle.repdl_hip_abi_version.argtypes = []
+        handle.repdl_hip_abi_version.restype = _INT
+        _lib = handle
+    return _lib
+
+
+def check(code: int, what: str) -> None:
+    if code != 0:
+        msg = lib().repdl_hip_error_string(code)
+        raise RepdlHipError("%s failed with code %d: %s" % (what, code, msg.decode() if msg else "?"))
+
+
+def call(name: str, *args) -> None:
+    check(getattr(lib(), name)(*args), name)

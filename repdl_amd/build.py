@@ -1,0 +1,59 @@
+"""Builds ``repdl_amd/librepdl_hip.so`` (the C-ABI library of include/repdl_hip.h)
+from ``repdl_amd/csrc/*.hip`` with hipcc for gfx950.
+
+Flags that matter for reproducibility:
+  -ffp-contract=off -fno-fast-math   nothing is fused or reassociated except the
+                                     explicit fma calls in the sources;
+  (default) denormals preserved      hipcc does not flush fp32 denormals on gfx9;
+  -packed-fp32-ops disabled          no v_pk_{fma,mul,add}_f32 is generated.
+Run as ``python -m repdl_amd.build``.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from glob import glob
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "librepdl_hip.so")
+OBJ = os.path.join(HERE, "csrc", "_obj")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fno-fast-math",
+    "-fvisibility=hidden", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _run(cmd: list[str]) -> None:
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), proc.stdout))
+
+
+def sources() -> list[str]:
+    return sorted(glob(os.path.join(CSRC, "*.hip")))
+
+
+def build(verbose: bool = False) -> str:
+    os.makedirs(OBJ, exist_ok=True)
+    jobs, objs = [], []
+    for src in sources():
+        obj = os.path.join(OBJ, os.path.basename(src)[:-4] + ".o")
+        objs.append(obj)
+        jobs.append([HIPCC] + FLAGS + ["-c", src, "-o", obj])
+    with ThreadPoolExecutor(max_workers=6) as ex:
+        list(ex.map(_run, jobs))
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
+    if verbose:
+        print(LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    build(verbose=True)
+    sys.exit(0)

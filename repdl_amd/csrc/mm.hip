@@ -1,0 +1,246 @@
+// Reproducible fp32 matrix multiplication for gfx950.
+//
+// Contract (RepDL backend/cpu/matrix_multiplication.cpp:22-34): every output
+// element owns one accumulator that starts at +0.0f and receives exactly one
+// fused multiply-add per k, k ascending.  Tiling over M and N and the way the
+// operands are staged are free; the order along K is not, so K is never split
+// across threads, there is no K padding (the last partial K tile runs a shorter
+// loop) and MFMA is not used (its internal accumulation is not a sequence of
+// single-rounding FMAs).
+//
+// Layout: a workgroup of 256 threads computes a 128x128 tile of C; each thread
+// an 8x8 micro-tile held in registers (rows ty*4+{0..3} and 64+ty*4+{0..3},
+// columns tx*4+{0..3} and 64+tx*4+{0..3}).  Both operands are staged through LDS
+// k-major (As[k][m], Bs[k][n]) so the inner loop reads its 8+8 operands with
+// four ds_read_b128 and issues 64 v_fma_f32.  Global loads for tile t+1 are
+// issued before the FMAs of tile t (register prefetch, two LDS buffers).
+#include "common.h"
+
+namespace
+{
+constexpr int BM = 128, BN = 128, BK = 16, NT = 256;
+constexpr int LDA = BM + 4; // padded row of the transposing store path
+constexpr int LDB = BN + 4;
+
+struct Frag
+{
+    float4 v[2];
+};
+
+// One operand tile = 128 "r" positions (rows of C for A, columns of C for B) by
+// BK steps of k.  KC: element (r,k) at X[r*ld + k] (k contiguous in memory);
+// otherwise element (r,k) at X[k*ld + r] (r contiguous).
+template <bool KC>
+__device__ __forceinline__ void load_tile(const float *__restrict__ X, int64_t ld, int64_t R,
+                                          int64_t K, int64_t r0, int64_t k0, bool vec_ok, int tid,
+                                          Frag &f)
+{
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+    {
+        int idx = tid + NT * i;
+        int64_t r, k;
+        if (KC)
+        {
+            r = r0 + (idx >> 2);
+            k = k0 + ((idx & 3) << 2);
+        }
+        else
+        {
+            k = k0 + (idx >> 5);
+            r = r0 + ((idx & 31) << 2);
+        }
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (KC)
+        {
+            if (r < R)
+            {
+                const float *p = X + r * ld + k;
+                if (vec_ok && k + 3 < K)
+                    v = *reinterpret_cast<const float4 *>(p);
+                else
+                {
+                    if (k + 0 < K) v.x = p[0];
+                    if (k + 1 < K) v.y = p[1];
+                    if (k + 2 < K) v.z = p[2];
+                    if (k + 3 < K) v.w = p[3];
+                }
+            }
+        }
+        else
+        {
+            if (k < K)
+            {
+                const float *p = X + k * ld + r;
+                if (vec_ok && r + 3 < R)
+                    v = *reinterpret_cast<const float4 *>(p);
+                else
+                {
+                    if (r + 0 < R) v.x = p[0];
+                    if (r + 1 < R) v.y = p[1];
+                    if (r + 2 < R) v.z = p[2];
+                    if (r + 3 < R) v.w = p[3];
+                }
+            }
+        }
+        f.v[i] = v;
+    }
+}
+
+template <bool KC, int LD>
+__device__ __forceinline__ void store_tile(float *__restrict__ S, int tid, const Frag &f)
+{
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+    {
+        int idx = tid + NT * i;
+        if (KC)
+        {
+            int r = idx >> 2, k = (idx & 3) << 2;
+            S[(k + 0) * LD + r] = f.v[i].x;
+            S[(k + 1) * LD + r] = f.v[i].y;
+            S[(k + 2) * LD + r] = f.v[i].z;
+            S[(k + 3) * LD + r] = f.v[i].w;
+        }
+        else
+        {
+            int k = idx >> 5, r = (idx & 31) << 2;
+            *reinterpret_cast<float4 *>(&S[k * LD + r]) = f.v[i];
+        }
+    }
+}
+
+__device__ __forceinline__ void fma_step(const float *__restrict__ As, const float *__restrict__ Bs,
+                                         int kk, int ty, int tx, float (&acc)[8][8])
+{
+    float4 a0 = *reinterpret_cast<const float4 *>(&As[kk * LDA + ty * 4]);
+    float4 a1 = *reinterpret_cast<const float4 *>(&As[kk * LDA + 64 + ty * 4]);
+    float4 b0 = *reinterpret_cast<const float4 *>(&Bs[kk * LDB + tx * 4]);
+    float4 b1 = *reinterpret_cast<const float4 *>(&Bs[kk * LDB + 64 + tx * 4]);
+    float a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+    float b[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            acc[i][j] = __fmaf_rn(a[i], b[j], acc[i][j]);
+}
+
+// TA: A is stored [K,M]; TB: B is stored [N,K].
+template <bool TA, bool TB>
+__global__ __launch_bounds__(NT) void mm_kernel(const float *__restrict__ A,
+                                                const float *__restrict__ B, float *__restrict__ C,
+                                                int64_t M, int64_t N, int64_t K, int avec, int bvec,
+                                                int cvec)
+{
+    constexpr bool A_KC = !TA; // A[m*K + k]
+    constexpr bool B_KC = TB;  // B[n*K + k]
+    __shared__ __attribute__((aligned(16))) float As[2][BK * LDA];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB];
+
+    const int tid = threadIdx.x;
+    const int tx = tid & 15, ty = tid >> 4;
+    const int64_t m0 = (int64_t)blockIdx.y * BM, n0 = (int64_t)blockIdx.x * BN;
+    const int64_t lda = TA ? M : K, ldb = TB ? K : N;
+
+    float acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            acc[i][j] = 0.0f;
+
+    const int64_t nkt = (K + BK - 1) / BK;
+    Frag fa, fb;
+    if (nkt > 0)
+    {
+        load_tile<A_KC>(A, lda, M, K, m0, 0, avec, tid, fa);
+        load_tile<B_KC>(B, ldb, N, K, n0, 0, bvec, tid, fb);
+        store_tile<A_KC, LDA>(As[0], tid, fa);
+        store_tile<B_KC, LDB>(Bs[0], tid, fb);
+    }
+    __syncthreads();
+
+    for (int64_t kt = 0; kt < nkt; kt++)
+    {
+        const int cur = (int)(kt & 1);
+        const bool more = kt + 1 < nkt;
+        if (more)
+        {
+            load_tile<A_KC>(A, lda, M, K, m0, (kt + 1) * BK, avec, tid, fa);
+            load_tile<B_KC>(B, ldb, N, K, n0, (kt + 1) * BK, bvec, tid, fb);
+        }
+        const int64_t krem = K - kt * BK;
+        if (krem >= BK)
+        {
+#pragma unroll
+            for (int kk = 0; kk < BK; kk++)
+                fma_step(As[cur], Bs[cur], kk, ty, tx, acc);
+        }
+        else
+        {
+            for (int kk = 0; kk < (int)krem; kk++)
+                fma_step(As[cur], Bs[cur], kk, ty, tx, acc);
+        }
+        if (more)
+        {
+            store_tile<A_KC, LDA>(As[cur ^ 1], tid, fa);
+            store_tile<B_KC, LDB>(Bs[cur ^ 1], tid, fb);
+        }
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+    {
+        int64_t m = m0 + ty * 4 + (i & 3) + (i >> 2) * 64;
+        if (m >= M)
+            continue;
+#pragma unroll
+        for (int jh = 0; jh < 2; jh++)
+        {
+            int64_t n = n0 + tx * 4 + jh * 64;
+            float *p = C + m * N + n;
+            if (cvec && n + 3 < N)
+                *reinterpret_cast<float4 *>(p) =
+                    make_float4(acc[i][jh * 4 + 0], acc[i][jh * 4 + 1], acc[i][jh * 4 + 2], acc[i][jh * 4 + 3]);
+            else
+            {
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (n + j < N)
+                        p[j] = acc[i][jh * 4 + j];
+            }
+        }
+    }
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+} // namespace
+
+REPDL_API int repdl_hip_mm(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K,
+                           int transA, int transB, void *stream)
+{
+    REPDL_REQUIRE(M >= 0 && N >= 0 && K >= 0);
+    if (M == 0 || N == 0)
+        return REPDL_OK;
+    REPDL_REQUIRE(C != nullptr);
+    REPDL_REQUIRE(K == 0 || (A != nullptr && B != nullptr));
+    const int64_t gx = repdl_cdiv(N, BN), gy = repdl_cdiv(M, BM);
+    REPDL_REQUIRE(gx <= REPDL_I32_MAX && gy <= 65535);
+    const int64_t lda = transA ? M : K, ldb = transB ? K : N;
+    const int avec = aligned16(A) && (lda % 4 == 0);
+    const int bvec = aligned16(B) && (ldb % 4 == 0);
+    const int cvec = aligned16(C) && (N % 4 == 0);
+    dim3 grid((unsigned)gx, (unsigned)gy), block(NT);
+    hipStream_t s = repdl_stream(stream);
+    if (!transA && !transB)
+        hipLaunchKernelGGL((mm_kernel<false, false>), grid, block, 0, s, A, B, C, M, N, K, avec, bvec, cvec);
+    else if (transA && !transB)
+        hipLaunchKernelGGL((mm_kernel<true, false>), grid, block, 0, s, A, B, C, M, N, K, avec, bvec, cvec);
+    else if (!transA && transB)
+        hipLaunchKernelGGL((mm_kernel<false, true>), grid, block, 0, s, A, B, C, M, N, K, avec, bvec, cvec);
+    else
+        hipLaunchKernelGGL((mm_kernel<true, true>), grid, block, 0, s, A, B, C, M, N, K, avec, bvec, cvec);
+    return repdl_launch_status();
+}

@@ -1,0 +1,82 @@
+"""Autograd helpers built on the reproducible sums -- the counterpart of RepDL's
+``repdl/func.py:11-121`` (``expand_as``, ``mean1d``, ``mean2d_dim0``,
+``mean4d_dim023``).  Forward values come from ``ops.sum*`` with ``average=True``
+(one multiply by float(1/count), never a division); backward passes scale the
+incoming gradient by the Python float ``1 / count`` and broadcast it, as the
+reference does.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import ops
+
+
+class _Broadcast(torch.autograd.Function):
+    """(n) -> (?, n) or (n, 1, 1) -> (?, n, ?, ?); the gradient is the reproducible
+    sum over the broadcast dimensions (reference func.py:11-33)."""
+
+    @staticmethod
+    def forward(ctx, input, shape):
+        return input.expand(shape)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        if not ctx.needs_input_grad[0]:
+            return None, None
+        if grad_output.dim() == 4:
+            return ops.sum4d_dim023(grad_output, keepdim=True).squeeze(0), None
+        return ops.sum2d_dim0(grad_output), None
+
+
+def expand_as(input: torch.Tensor, other: torch.Tensor) -> torch.Tensor:
+    vec_to_rows = input.dim() == 1 and other.dim() == 2 and input.shape[-1] == other.shape[-1]
+    chan_to_maps = (
+        input.dim() == 3 and other.dim() == 4 and input.shape[0] == other.shape[1]
+        and input.shape[1] == 1 and input.shape[2] == 1
+    )
+    if not (vec_to_rows or chan_to_maps):
+        raise NotImplementedError("expand_as supports (n)->(?,n) and (n,1,1)->(?,n,?,?) only")
+    return _Broadcast.apply(input, other.shape)
+
+
+def _mean_function(name: str, reducer, spread):
+    """Build an autograd Function whose forward is ``reducer(input, average=True)``
+    and whose backward spreads grad * (1/count) back over the input shape."""
+
+    def forward(ctx, input):
+        ctx.in_shape = input.shape
+        return reducer(input, average=True)
+
+    def backward(ctx, grad_output):
+        if not ctx.needs_input_grad[0]:
+            return None
+        shape = ctx.in_shape
+        count = shape.numel() // max(grad_output.numel(), 1)
+        return spread(grad_output * (1 / count), shape)
+
+    return type(name, (torch.autograd.Function,), {"forward": staticmethod(forward), "backward": staticmethod(backward)})
+
+
+# reference func.py:47-67, 72-93, 98-119
+_Mean1d = _mean_function("Mean1dFunction", ops.sum1d, lambda g, s: g.expand(s).contiguous())
+# (the reference spreads the 2-D gradient with unsqueeze(-1), func.py:88, which only
+# type-checks for square inputs; the gradient of a column mean is a row broadcast)
+_Mean2dDim0 = _mean_function("Mean2dDim0Function", ops.sum2d_dim0, lambda g, s: g.unsqueeze(0).expand(s))
+_Mean4dDim023 = _mean_function(
+    "Mean4dDim023Function", ops.sum4d_dim023, lambda g, s: g.unsqueeze(-1).unsqueeze(-1).expand(s))
+
+
+def mean1d(input: torch.Tensor) -> torch.Tensor:
+    assert input.dim() == 1
+    return _Mean1d.apply(input)
+
+
+def mean2d_dim0(input: torch.Tensor) -> torch.Tensor:
+    assert input.dim() == 2
+    return _Mean2dDim0.apply(input)
+
+
+def mean4d_dim023(input: torch.Tensor) -> torch.Tensor:
+    assert input.dim() == 4
+    return _Mean4dDim023.apply(input)

@@ -1,0 +1,171 @@
+"""Functional layer API with reproducible forward and backward passes -- the
+counterpart of RepDL's ``repdl/nn/functional.py`` (``linear``, ``conv2d``,
+``cross_entropy``, ``batch_norm``) and of the autograd Functions behind it
+(``repdl/nn/linear.py:11-38``, ``conv.py:11-50``, ``loss.py:11-34``,
+``batchnorm.py:12-66``).  Every tensor contraction, reduction, division and
+square root goes through ``repdl_amd.ops``; which operator is called, in which
+order, and which updates are in place follows the reference.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple, Union
+
+import torch
+
+from .. import func, ops
+
+_Pair = Union[int, Tuple[int, int]]
+
+
+class _Linear(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        ctx.save_for_backward(x, weight)
+        y = ops.mm(x, weight, transB=True)  # x [B,in] . W[out,in]^T
+        if bias is not None:
+            y += bias
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        x, weight = ctx.saved_tensors
+        need_x, need_w, need_b = ctx.needs_input_grad
+        gx = ops.mm(gy, weight) if need_x else None
+        gw = ops.mm(gy, x, transA=True) if need_w else None  # gy^T . x, the batch is K
+        gb = ops.sum2d_dim0(gy) if need_b else None
+        return gx, gw, gb
+
+
+def linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    if input.dim() != 2:
+        raise NotImplementedError("linear: only 2-D input is supported")
+    assert weight.dim() == 2
+    assert bias is None or bias.dim() == 1
+    return _Linear.apply(input, weight, bias)
+
+
+class _Conv2d(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias, stride, padding, groups):
+        ctx.save_for_backward(x, weight)
+        ctx.conf = (stride, padding, groups)
+        y = ops.conv2d(x, weight, stride=stride, padding=padding, groups=groups)
+        if bias is not None:
+            y += bias.unsqueeze(-1).unsqueeze(-1)
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        stride, padding, groups = ctx.conf
+        if groups != 1:
+            raise NotImplementedError("conv2d backward: groups != 1")
+        x, weight = ctx.saved_tensors
+        need_x, need_w, need_b = ctx.needs_input_grad[:3]
+        gx = ops.conv2d_grad_input(x.shape, weight, gy, stride, padding) if need_x else None
+        gw = ops.conv2d_grad_kernel(x, weight.shape, gy, stride, padding) if need_w else None
+        gb = ops.sum4d_dim023(gy) if need_b else None
+        return gx, gw, gb, None, None, None
+
+
+def conv2d(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, stride: _Pair = 1,
+           padding: Union[str, _Pair] = 0, dilation: _Pair = 1, groups: int = 1) -> torch.Tensor:
+    if isinstance(padding, str) or dilation not in (1, (1, 1)) or input.dim() != 4:
+        raise NotImplementedError("conv2d: string padding, dilation != 1 and non-4-D input are not supported")
+    assert weight.dim() == 4
+    assert bias is None or bias.dim() == 1
+    stride = (stride, stride) if isinstance(stride, int) else tuple(stride)
+    padding = (padding, padding) if isinstance(padding, int) else tuple(padding)
+    return _Conv2d.apply(input, weight, bias, stride, padding, groups)
+
+
+class _CrossEntropy(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits, target):
+        ctx.save_for_backward(logits, target)
+        return ops.cross_entropy(logits, target)
+
+    @staticmethod
+    def backward(ctx, g):
+        logits, target = ctx.saved_tensors
+        if not ctx.needs_input_grad[0]:
+            return None, None
+        rows, classes = logits.shape
+        gl = ops.softmax(logits) - torch.nn.functional.one_hot(target, classes)
+        gl *= 1.0 / rows  # first the mean factor, then the incoming gradient (loss.py:32-33)
+        gl *= g
+        return gl, None
+
+
+def cross_entropy(input: torch.Tensor, target: torch.Tensor, weight: Optional[torch.Tensor] = None,
+                  size_average: Optional[bool] = None, ignore_index: int = -100, reduce: Optional[bool] = None,
+                  reduction: str = "mean", label_smoothing: float = 0.0) -> torch.Tensor:
+    plain = (weight is None and size_average is None and ignore_index == -100 and reduce is None
+             and reduction == "mean" and label_smoothing == 0.0)
+    if not plain or input.dim() != 2 or target.dim() != 1:
+        raise NotImplementedError("cross_entropy: only mean reduction of [B,C] logits and [B] class indices")
+    return _CrossEntropy.apply(input, target)
+
+
+def _per_channel(t: torch.Tensor, like: torch.Tensor) -> torch.Tensor:
+    return t.unsqueeze(-1).unsqueeze(-1) if like.dim() == 4 else t
+
+
+class _BatchNorm(torch.autograd.Function):
+    """y = (x - mean) / std * weight + bias with std = sqrt(var + eps); mean and var are
+    inputs with their own gradients (reference batchnorm.py:12-66).  Divisions and
+    the square root go through ops so they are the IEEE results on the GPU as well."""
+
+    @staticmethod
+    def forward(ctx, x, mean, var, weight, bias, eps):
+        std = ops.sqrt(var + eps)
+        ctx.save_for_backward(x, mean, std, weight)
+        y = ops.div(x - _per_channel(mean, x), _per_channel(std, x).expand_as(x))
+        if x.dim() == 4:
+            y *= _per_channel(weight, x)
+            y += _per_channel(bias, x)
+        else:
+            y = weight * y + bias
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        x, mean, std, weight = ctx.saved_tensors
+        mean_b, std_b, weight_b = (_per_channel(t, gy) for t in (mean, std, weight))
+        reduce = ops.sum4d_dim023 if gy.dim() == 4 else ops.sum2d_dim0
+        need = ctx.needs_input_grad
+        w_over_std = ops.div(weight, std)
+        gx = _per_channel(w_over_std, gy) * gy if need[0] else None
+        gmean = (-w_over_std) * reduce(gy) if need[1] else None
+        gvar = None
+        if need[2]:
+            coef = ops.div(weight, 2 * std * std * std)
+            gvar = reduce(gy * (mean_b - x) * _per_channel(coef, gy))
+        gweight = reduce(ops.div(x - mean_b, std_b.expand_as(x)) * gy) if need[3] else None
+        gbias = reduce(gy) if need[4] else None
+        return gx, gmean, gvar, gweight, gbias, None
+
+
+def batch_norm(input: torch.Tensor, running_mean: Optional[torch.Tensor], running_var: Optional[torch.Tensor],
+               weight: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
+               batch_statistics: bool = False, momentum: float = 0.1, eps: float = 1e-5) -> torch.Tensor:
+    if weight is None or bias is None or input.dim() not in (2, 4):
+        raise NotImplementedError("batch_norm: affine parameters and 2-D or 4-D input are required")
+    assert weight.dim() == 1 and bias.dim() == 1
+    if batch_statistics:
+        if input.dim() == 4:
+            mean = func.mean4d_dim023(input)
+            centred = input - func.expand_as(mean.unsqueeze(-1).unsqueeze(-1), input)
+            var = func.mean4d_dim023(centred * centred)
+        else:
+            mean = func.mean2d_dim0(input)
+            centred = input - func.expand_as(mean, input)
+            var = func.mean2d_dim0(centred * centred)
+        if running_mean is not None and running_var is not None:
+            # The reference evaluates these two expressions (batchnorm.py:92-93) but
+            # drops the results; here they are stored, which is what the buffers are for.
+            with torch.no_grad():
+                running_mean.copy_(momentum * mean.detach() + (1.0 - momentum) * running_mean)
+                running_var.copy_(momentum * var.detach() + (1.0 - momentum) * running_var)
+    else:
+        mean, var = running_mean, running_var
+    return _BatchNorm.apply(input, mean, var, weight, bias, eps)
