@@ -55,11 +55,14 @@ CRM_FN float crm_d2f(double d) { return (float)d; }
 // fewer) bits gives the correctly rounded result (53 >= 24 + 2).
 CRM_FN double crm_round_to_odd(double q, double residual)
 {
-    uint64_t u = crm_d2u(q);
-    uint64_t below = (u - 1) | 1; // t in (q - ulp, q)
-    uint64_t above = u | 1;       // t in (q, q + ulp)
-    uint64_t r = residual < 0.0 ? below : above;
-    return residual == 0.0 ? q : crm_u2d(r);
+    const uint64_t ur = crm_d2u(residual);
+    const uint32_t rhi = (uint32_t)(ur >> 32);
+    // the residual is an exact binary64 value that is never subnormal here, so it
+    // is non-zero iff its exponent field is; its sign bit says q lies above t
+    const uint64_t inexact = (rhi & 0x7FF00000u) != 0u;
+    const uint64_t above_t = (uint64_t)(rhi >> 31) & inexact;
+    // t in (q, q+ulp): q|1;  t in (q-ulp, q): (q-1)|1;  t == q: q
+    return crm_u2d((crm_d2u(q) - above_t) | inexact);
 }
 
 // 1 / b for finite positive binary64 b in [2^-149, 2^128), relative error
@@ -110,13 +113,11 @@ CRM_FN float crm_div(float a, float b)
 {
     const uint32_t ua = crm_f2u(a), ub = crm_f2u(b);
     // |a|, |b| as doubles (exact, subnormals included).  Zero, infinity and NaN
-    // run through the arithmetic harmlessly and are overridden afterwards.
-    double da = (double)crm_u2f(ua & 0x7FFFFFFFu);
-    double db = (double)crm_u2f(ub & 0x7FFFFFFFu);
-    const uint32_t ab = ub & 0x7FFFFFFFu;
-    if (ab == 0u || ab >= 0x7F800000u)
-        db = 1.0;
-    float g = crm_div_core(da, db, crm_recip_approx(db));
+    // run through the arithmetic harmlessly (nothing traps, nothing is indexed
+    // by the values) and are overridden afterwards.
+    const double da = (double)crm_u2f(ua & 0x7FFFFFFFu);
+    const double db = (double)crm_u2f(ub & 0x7FFFFFFFu);
+    const float g = crm_div_core(da, db, crm_recip_approx(db));
     return crm_div_special(ua, ub, g);
 }
 
@@ -131,10 +132,7 @@ CRM_FN crm_divisor crm_divisor_make(float b)
 {
     crm_divisor d;
     d.ub = crm_f2u(b);
-    const uint32_t ab = d.ub & 0x7FFFFFFFu;
-    d.db = (double)crm_u2f(ab);
-    if (ab == 0u || ab >= 0x7F800000u)
-        d.db = 1.0;
+    d.db = (double)crm_u2f(d.ub & 0x7FFFFFFFu);
     d.y = crm_recip_approx(d.db);
     return d;
 }
@@ -146,18 +144,20 @@ CRM_FN float crm_div_by(float a, crm_divisor d)
     return crm_div_special(ua, d.ub, crm_div_core(da, d.db, d.y));
 }
 
-// sqrt: reciprocal-square-root seed by integer arithmetic (error < 3.5 %), three
-// Newton steps y <- y + y*(1/2 - (x/2)*y*y), then s = x*y with one residual
-// correction and the round-to-odd fix-up.
+// sqrt: reciprocal-square-root seed by integer arithmetic on the high word
+// (error < 3.5 %), three Newton steps y <- y + y*(1/2 - (x/2)*y*y), then s = x*y
+// with one residual correction: s is within 1 ulp64 of sqrt(x).  That is enough
+// for a correctly rounded binary32 result: sqrt(x) of a 24-bit x is either
+// exactly a 24-bit number (then s, within 1 ulp64 of a binary64 value, rounds to
+// it) or farther than 2^-50.5 relative (2.8 ulp64) from every binary32 value and
+// midpoint, so s lies on the same side of every rounding boundary.
 CRM_FN float crm_sqrt(float x)
 {
     const uint32_t ux = crm_f2u(x);
-    const uint32_t ax = ux & 0x7FFFFFFFu;
-    double dx = (double)x;
-    if (ax == 0u || ux >= 0x7F800000u)
-        dx = 1.0; // zeros, negatives, infinities, NaNs: overridden below
+    const double dx = (double)x; // exact; subnormals become normal
     const double hx = 0.5 * dx;
-    double y = crm_u2d(0x5FE6EB50C7B537A9ULL - (crm_d2u(dx) >> 1));
+    const uint32_t hi = (uint32_t)(crm_d2u(dx) >> 32);
+    double y = crm_u2d((uint64_t)(0x5FE6EB50u - (hi >> 1)) << 32);
     double e = crm_fma(-hx, y * y, 0.5);
     y = crm_fma(y, e, y);
     e = crm_fma(-hx, y * y, 0.5);
@@ -165,16 +165,19 @@ CRM_FN float crm_sqrt(float x)
     e = crm_fma(-hx, y * y, 0.5);
     y = crm_fma(y, e, y);
     double s = dx * y;
-    double r = crm_fma(-s, s, dx);
+    const double r = crm_fma(-s, s, dx);
     s = crm_fma(r, 0.5 * y, s);
-    r = crm_fma(-s, s, dx);
-    uint32_t res = crm_f2u(crm_d2f(crm_round_to_odd(s, r)));
-    if (ax == 0u || ux == 0x7F800000u)
-        res = ux; // +-0, +inf
-    if (ux > 0x80000000u)
+    uint32_t res = crm_f2u(crm_d2f(s));
+    // +-0, +inf, negatives, -inf and NaNs: (ux - 1) wraps 0 to the top
+    if (ux - 1u >= 0x7F7FFFFFu)
+    {
+        const uint32_t ax = ux & 0x7FFFFFFFu;
         res = CRM_QNAN_POS; // negative, -inf (PyTorch CPU convention)
-    if (ax > 0x7F800000u)
-        res = ux | 0x00400000u; // NaN: sign and payload kept, quieted
+        if (ax == 0u || ux == 0x7F800000u)
+            res = ux; // +-0, +inf
+        if (ax > 0x7F800000u)
+            res = ux | 0x00400000u; // NaN: sign and payload kept, quieted
+    }
     return crm_u2f(res);
 }
 
@@ -216,17 +219,16 @@ CRM_FN float crm_exp(float x, const uint64_t *tab)
 {
     const uint32_t ux = crm_f2u(x);
     const uint32_t ax = ux & 0x7FFFFFFFu;
-    // Outside [-104, 89] the binary32 result is 0 or +inf whatever the binary64
-    // value is (exp(-104) < 2^-150, exp(89) > 2^128); clamping keeps 2^(k/N)
-    // inside the normal binary64 range.
-    float xc = x;
-    if (ax > 0x42D00000u) // |x| > 104 (also inf, NaN)
-        xc = 0.0f;
-    uint32_t res = crm_f2u(crm_d2f(crm_exp64_core((double)xc, tab)));
+    // |x| > 104 (also inf, NaN): the binary32 result is 0 or +inf whatever the
+    // binary64 value is (exp(-104) < 2^-150, exp(89) > 2^128).  Such arguments
+    // still run through the core harmlessly: the table index is masked.
+    uint32_t res = crm_f2u(crm_d2f(crm_exp64_core((double)x, tab)));
     if (ax > 0x42D00000u)
+    {
         res = (ux >> 31) ? 0u : 0x7F800000u;
-    if (ax > 0x7F800000u)
-        res = ux | 0x00400000u; // NaN + 1.0: sign and payload kept, quieted
+        if (ax > 0x7F800000u)
+            res = ux | 0x00400000u; // NaN + 1.0: sign and payload kept, quieted
+    }
     return crm_u2f(res);
 }
 
@@ -238,16 +240,19 @@ CRM_FN float crm_exp(float x, const uint64_t *tab)
 CRM_FN double crm_log64_core(double x, const double *tab)
 {
     const uint64_t ix = crm_d2u(x);
-    const uint64_t tmp = ix - 0x3FE6000000000000ULL;
-    const uint32_t i = (uint32_t)(tmp >> 45) & 127u;
-    const int32_t k = (int32_t)((int64_t)tmp >> 52);
-    const double z = crm_u2d(ix - (tmp & 0xFFF0000000000000ULL));
+    // only the high word takes part in the reduction (the offset has a zero low word)
+    const uint32_t hi = (uint32_t)(ix >> 32);
+    const uint32_t tmp = hi - 0x3FE60000u;
+    const uint32_t i = (tmp >> 13) & 127u;
+    const int32_t k = (int32_t)tmp >> 20;
+    const uint32_t zhi = hi - (tmp & 0xFFF00000u);
+    const double z = crm_u2d(((uint64_t)zhi << 32) | (ix & 0xFFFFFFFFu));
     const double invc = tab[4 * i], logc_hi = tab[4 * i + 1], logc_lo = tab[4 * i + 2];
     const double kd = (double)k;
     const double r = crm_fma(z, invc, -1.0);
     const double w = crm_fma(kd, CRM_LN2_HI, logc_hi); // exact
-    const double hi = w + r;
-    double lo = (w - hi) + r;
+    const double hi_sum = w + r;
+    double lo = (w - hi_sum) + r;
     lo += crm_fma(kd, CRM_LN2_LO, logc_lo);
     const double r2 = r * r;
     double p = crm_fma(r, 0x1.c71c71c71c71cp-4, -0.125); // r^9/9 - r^8/8
@@ -257,24 +262,25 @@ CRM_FN double crm_log64_core(double x, const double *tab)
     p = crm_fma(r, p, -0.25);
     p = crm_fma(r, p, 0x1.5555555555555p-2);
     p = crm_fma(r, p, -0.5);
-    return hi + crm_fma(r2, p, lo);
+    return hi_sum + crm_fma(r2, p, lo);
 }
 
 CRM_FN float crm_log(float x, const double *tab)
 {
     const uint32_t ux = crm_f2u(x);
-    const uint32_t ax = ux & 0x7FFFFFFFu;
-    float xc = x;
-    if (ax == 0u || ux >= 0x7F800000u)
-        xc = 1.0f;
-    uint32_t res = crm_f2u(crm_d2f(crm_log64_core((double)xc, tab)));
-    if (ux == 0x7F800000u)
-        res = 0x7F800000u; // log(+inf)
-    if (ux > 0x80000000u)
+    // zeros, negatives, infinities and NaNs run through the core harmlessly (the
+    // table index is masked) and are overridden
+    uint32_t res = crm_f2u(crm_d2f(crm_log64_core((double)x, tab)));
+    if (ux - 1u >= 0x7F7FFFFFu)
+    {
+        const uint32_t ax = ux & 0x7FFFFFFFu;
         res = CRM_QNAN_NEG; // log(negative), log(-inf): (x-x)/(x-x) on x86
-    if (ax == 0u)
-        res = 0xFF800000u; // log(+-0) = -inf
-    if (ax > 0x7F800000u)
-        res = ux | 0x00400000u; // NaN: sign and payload kept, quieted
+        if (ux == 0x7F800000u)
+            res = 0x7F800000u; // log(+inf)
+        if (ax == 0u)
+            res = 0xFF800000u; // log(+-0) = -inf
+        if (ax > 0x7F800000u)
+            res = ux | 0x00400000u; // NaN: sign and payload kept, quieted
+    }
     return crm_u2f(res);
 }

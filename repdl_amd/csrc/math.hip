@@ -4,8 +4,8 @@
 // routine followed by one rounding to binary32) and repdl/ops.py:98-103, 122-123
 // (div, sqrt: the IEEE binary32 results).  The arithmetic lives in crmath.h and
 // uses no approximate-function instruction and no '/' operator; this file only
-// streams the data: 16-byte loads and stores, grid-stride, several loads in
-// flight per lane; the exp/log tables (2 KiB / 4 KiB) are copied to LDS once per
+// streams the data: 16-byte non-temporal loads and stores, one contiguous
+// chunk per workgroup, several loads in flight per lane; the exp/log tables (2 KiB / 4 KiB) are copied to LDS once per
 // workgroup.  All four are HBM-bound: 8 bytes per element (12 for tensor/tensor
 // division).
 #include "common.h"
@@ -17,7 +17,16 @@ __device__ const uint64_t g_exp_tab[256] = CRM_EXP_TAB_INIT;
 __device__ const double g_log_tab[512] = CRM_LOG_TAB_INIT;
 
 constexpr int EW_THREADS = 256;
-constexpr int EW_UNROLL = 4; // float4 per lane per iteration
+constexpr int EW_UNROLL = 4;                                // 16-byte accesses in flight per lane
+constexpr int EW_ITERS = 4;                                 // iterations per workgroup
+constexpr int EW_CHUNK = EW_THREADS * EW_UNROLL * EW_ITERS; // float4 per workgroup (64 KiB in, 64 KiB out)
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// Streaming accesses: every byte is touched once, so loads and stores carry the
+// non-temporal hint and each workgroup owns one contiguous chunk.
+__device__ __forceinline__ v4f ld_stream(const v4f *p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void st_stream(v4f v, v4f *p) { __builtin_nontemporal_store(v, p); }
 
 enum Op
 {
@@ -43,6 +52,15 @@ struct Ctx
             return crm_sqrt(x);
         return crm_div_by(x, divisor);
     }
+    __device__ __forceinline__ v4f apply4(v4f v) const
+    {
+        v4f r;
+        r.x = apply(v.x);
+        r.y = apply(v.y);
+        r.z = apply(v.z);
+        r.w = apply(v.w);
+        return r;
+    }
 };
 
 template <int OP>
@@ -50,7 +68,7 @@ __global__ __launch_bounds__(EW_THREADS) void unary_kernel(const float *__restri
                                                            float *__restrict__ out, int64_t n,
                                                            float scalar, int vec_ok)
 {
-    __shared__ __attribute__((aligned(16))) uint64_t tab[512];
+    __shared__ __attribute__((aligned(16))) uint64_t tab[OP == OP_LOG ? 512 : 256];
     Ctx<OP> ctx;
     ctx.exp_tab = tab;
     ctx.log_tab = reinterpret_cast<const double *>(tab);
@@ -69,102 +87,99 @@ __global__ __launch_bounds__(EW_THREADS) void unary_kernel(const float *__restri
     if (OP == OP_DIV_SCALAR)
         ctx.divisor = crm_divisor_make(scalar);
 
-    const int64_t tid = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x;
-    const int64_t nthreads = (int64_t)gridDim.x * EW_THREADS;
-    int64_t done = 0;
     if (vec_ok)
     {
         const int64_t n4 = n >> 2;
-        const float4 *in4 = reinterpret_cast<const float4 *>(in);
-        float4 *out4 = reinterpret_cast<float4 *>(out);
-        int64_t i = tid;
-        for (; i + (EW_UNROLL - 1) * nthreads < n4; i += EW_UNROLL * nthreads)
+        const v4f *in4 = reinterpret_cast<const v4f *>(in);
+        v4f *out4 = reinterpret_cast<v4f *>(out);
+        const int64_t b0 = (int64_t)blockIdx.x * EW_CHUNK;
+        const int64_t b1 = b0 + EW_CHUNK < n4 ? b0 + EW_CHUNK : n4;
+        int64_t i = b0 + threadIdx.x;
+        for (; i + (EW_UNROLL - 1) * EW_THREADS < b1; i += EW_UNROLL * EW_THREADS)
         {
-            float4 v[EW_UNROLL];
+            v4f v[EW_UNROLL];
 #pragma unroll
             for (int u = 0; u < EW_UNROLL; u++)
-                v[u] = in4[i + u * nthreads];
+                v[u] = ld_stream(&in4[i + u * EW_THREADS]);
 #pragma unroll
             for (int u = 0; u < EW_UNROLL; u++)
-            {
-                float4 r;
-                r.x = ctx.apply(v[u].x);
-                r.y = ctx.apply(v[u].y);
-                r.z = ctx.apply(v[u].z);
-                r.w = ctx.apply(v[u].w);
-                out4[i + u * nthreads] = r;
-            }
+                st_stream(ctx.apply4(v[u]), &out4[i + u * EW_THREADS]);
         }
-        for (; i < n4; i += nthreads)
-        {
-            float4 v = in4[i], r;
-            r.x = ctx.apply(v.x);
-            r.y = ctx.apply(v.y);
-            r.z = ctx.apply(v.z);
-            r.w = ctx.apply(v.w);
-            out4[i] = r;
-        }
-        done = n4 << 2;
+        for (; i < b1; i += EW_THREADS)
+            st_stream(ctx.apply4(ld_stream(&in4[i])), &out4[i]);
+        // the last (n mod 4) elements
+        if (blockIdx.x == 0 && threadIdx.x < (n & 3))
+            out[(n4 << 2) + threadIdx.x] = ctx.apply(in[(n4 << 2) + threadIdx.x]);
     }
-    for (int64_t i = done + tid; i < n; i += nthreads)
-        out[i] = ctx.apply(in[i]);
+    else
+    {
+        const int64_t b0 = (int64_t)blockIdx.x * EW_CHUNK * 4;
+        const int64_t b1 = b0 + EW_CHUNK * 4 < n ? b0 + EW_CHUNK * 4 : n;
+        for (int64_t i = b0 + threadIdx.x; i < b1; i += EW_THREADS)
+            out[i] = ctx.apply(in[i]);
+    }
 }
+
+__device__ __forceinline__ v4f div4(v4f a, v4f b)
+{
+    v4f r;
+    r.x = crm_div(a.x, b.x);
+    r.y = crm_div(a.y, b.y);
+    r.z = crm_div(a.z, b.z);
+    r.w = crm_div(a.w, b.w);
+    return r;
+}
+
+constexpr int DIV_UNROLL = 2;
 
 __global__ __launch_bounds__(EW_THREADS) void div_kernel(const float *__restrict__ a,
                                                          const float *__restrict__ b,
                                                          float *__restrict__ out, int64_t n,
                                                          int vec_ok)
 {
-    const int64_t tid = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x;
-    const int64_t nthreads = (int64_t)gridDim.x * EW_THREADS;
-    int64_t done = 0;
     if (vec_ok)
     {
         const int64_t n4 = n >> 2;
-        const float4 *a4 = reinterpret_cast<const float4 *>(a);
-        const float4 *b4 = reinterpret_cast<const float4 *>(b);
-        float4 *out4 = reinterpret_cast<float4 *>(out);
-        int64_t i = tid;
-        for (; i + nthreads < n4; i += 2 * nthreads)
+        const v4f *a4 = reinterpret_cast<const v4f *>(a);
+        const v4f *b4 = reinterpret_cast<const v4f *>(b);
+        v4f *out4 = reinterpret_cast<v4f *>(out);
+        const int64_t b0 = (int64_t)blockIdx.x * EW_CHUNK;
+        const int64_t b1 = b0 + EW_CHUNK < n4 ? b0 + EW_CHUNK : n4;
+        int64_t i = b0 + threadIdx.x;
+        for (; i + (DIV_UNROLL - 1) * EW_THREADS < b1; i += DIV_UNROLL * EW_THREADS)
         {
-            float4 x0 = a4[i], y0 = b4[i], x1 = a4[i + nthreads], y1 = b4[i + nthreads], r;
-            r.x = crm_div(x0.x, y0.x);
-            r.y = crm_div(x0.y, y0.y);
-            r.z = crm_div(x0.z, y0.z);
-            r.w = crm_div(x0.w, y0.w);
-            out4[i] = r;
-            r.x = crm_div(x1.x, y1.x);
-            r.y = crm_div(x1.y, y1.y);
-            r.z = crm_div(x1.z, y1.z);
-            r.w = crm_div(x1.w, y1.w);
-            out4[i + nthreads] = r;
+            v4f x[DIV_UNROLL], y[DIV_UNROLL];
+#pragma unroll
+            for (int u = 0; u < DIV_UNROLL; u++)
+            {
+                x[u] = ld_stream(&a4[i + u * EW_THREADS]);
+                y[u] = ld_stream(&b4[i + u * EW_THREADS]);
+            }
+#pragma unroll
+            for (int u = 0; u < DIV_UNROLL; u++)
+                st_stream(div4(x[u], y[u]), &out4[i + u * EW_THREADS]);
         }
-        for (; i < n4; i += nthreads)
-        {
-            float4 x = a4[i], y = b4[i], r;
-            r.x = crm_div(x.x, y.x);
-            r.y = crm_div(x.y, y.y);
-            r.z = crm_div(x.z, y.z);
-            r.w = crm_div(x.w, y.w);
-            out4[i] = r;
-        }
-        done = n4 << 2;
+        for (; i < b1; i += EW_THREADS)
+            st_stream(div4(ld_stream(&a4[i]), ld_stream(&b4[i])), &out4[i]);
+        if (blockIdx.x == 0 && threadIdx.x < (n & 3))
+            out[(n4 << 2) + threadIdx.x] = crm_div(a[(n4 << 2) + threadIdx.x], b[(n4 << 2) + threadIdx.x]);
     }
-    for (int64_t i = done + tid; i < n; i += nthreads)
-        out[i] = crm_div(a[i], b[i]);
+    else
+    {
+        const int64_t b0 = (int64_t)blockIdx.x * EW_CHUNK * 4;
+        const int64_t b1 = b0 + EW_CHUNK * 4 < n ? b0 + EW_CHUNK * 4 : n;
+        for (int64_t i = b0 + threadIdx.x; i < b1; i += EW_THREADS)
+            out[i] = crm_div(a[i], b[i]);
+    }
 }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-inline unsigned ew_grid(int64_t n)
+// one workgroup per EW_CHUNK float4 (at least one, so the n < 4 tail is served)
+inline int64_t ew_grid(int64_t n)
 {
-    // 8 workgroups per CU on 256 CUs, fewer for small inputs
-    int64_t want = repdl_cdiv(repdl_cdiv(n, 4), EW_THREADS);
-    if (want > 2048)
-        want = 2048;
-    if (want < 1)
-        want = 1;
-    return (unsigned)want;
+    int64_t g = repdl_cdiv(repdl_cdiv(n, 4), EW_CHUNK);
+    return g < 1 ? 1 : g;
 }
 
 template <int OP>
@@ -175,7 +190,9 @@ int launch_unary(const float *in, float *out, int64_t n, float scalar, void *str
         return REPDL_OK;
     REPDL_REQUIRE(in != nullptr && out != nullptr);
     const int vec_ok = aligned16(in) && aligned16(out);
-    hipLaunchKernelGGL((unary_kernel<OP>), dim3(ew_grid(n)), dim3(EW_THREADS), 0, repdl_stream(stream), in,
+    const int64_t grid = ew_grid(n);
+    REPDL_REQUIRE(grid <= REPDL_I32_MAX);
+    hipLaunchKernelGGL((unary_kernel<OP>), dim3((unsigned)grid), dim3(EW_THREADS), 0, repdl_stream(stream), in,
                        out, n, scalar, vec_ok);
     return repdl_launch_status();
 }
@@ -208,7 +225,9 @@ REPDL_API int repdl_hip_div(const float *a, const float *b, float *out, int64_t 
         return REPDL_OK;
     REPDL_REQUIRE(a != nullptr && b != nullptr && out != nullptr);
     const int vec_ok = aligned16(a) && aligned16(b) && aligned16(out);
-    hipLaunchKernelGGL(div_kernel, dim3(ew_grid(n)), dim3(EW_THREADS), 0, repdl_stream(stream), a, b, out, n,
+    const int64_t grid = ew_grid(n);
+    REPDL_REQUIRE(grid <= REPDL_I32_MAX);
+    hipLaunchKernelGGL(div_kernel, dim3((unsigned)grid), dim3(EW_THREADS), 0, repdl_stream(stream), a, b, out, n,
                        vec_ok);
     return repdl_launch_status();
 }
