@@ -17,73 +17,106 @@ namespace
 //   sum2d_dim1  [M,N]:      rows=M, nseg=1, seglen=N,   row_stride=N
 //   sum4d_dim023 [N,C,H,W]: rows=C, nseg=N, seglen=H*W, row_stride=H*W, seg_stride=C*H*W
 //   sum1d:                  rows=1, nseg=1, seglen=n
-// A workgroup of RW waves owns 64 chains.  All waves load TILE_R x TILE_C tiles
-// (coalesced along the segment) into LDS; wave 0 then walks the 64 chains, lane
-// l adding row l's TILE_C values in order.  Rows are padded by one float so the
-// 64 lanes of the walking wave hit 64 different... banks (stride 65 mod 32 = 1).
+// A workgroup of RT threads owns RR chains (4 to 64, chosen from the number of
+// rows) and moves through them in tiles of RR x RC floats = 32 KiB.  All its
+// waves stream the NEXT tile from global memory into registers with 16-byte
+// non-temporal loads (each wave reads contiguous pieces of one row at a time)
+// while one wave walks the CURRENT tile in LDS: lane l adds row l's RC values in
+// order, reading them back with ds_read_b128.  One LDS buffer (33 KiB) lets four
+// workgroups share a CU, which keeps up to 128 KiB of loads in flight per CU --
+// what it takes to cover loaded HBM latency.  The walking wave rotates with the
+// workgroup index to spread the walks over the SIMDs; a walk costs one dependent
+// v_add_f32 per element and chain, well below the memory time of the tile as
+// long as enough lanes walk (hence more chains per workgroup when rows abound).
 // ---------------------------------------------------------------------------
-constexpr int ROWS = 64;   // chains per workgroup
-constexpr int TC = 64;     // tile columns
-constexpr int LDT = TC + 1;
-constexpr int RT = 256;    // threads per workgroup
+constexpr int RTILE = 8192;    // floats per tile
 
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+template <int RR, int RT, bool VEC>
 __global__ __launch_bounds__(RT) void rowchain_kernel(const float *__restrict__ in,
                                                       float *__restrict__ out, int64_t rows,
                                                       int64_t nseg, int64_t seglen,
                                                       int64_t row_stride, int64_t seg_stride,
                                                       float factor)
 {
-    __shared__ float tile[2][ROWS * LDT];
+    constexpr int RC = RTILE / RR; // tile columns
+    constexpr int RLD = RC + 4;    // padded LDS row: keeps 16-byte alignment, shifts banks by 4
+    constexpr int C4 = RC / 4;     // float4 per tile row
+    constexpr int RV = RTILE / 4 / RT; // float4 per thread and tile
+    __shared__ __attribute__((aligned(16))) float tile[RR * RLD];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int64_t r0 = (int64_t)blockIdx.x * ROWS;
-    const int64_t tiles_per_seg = (seglen + TC - 1) / TC;
+    const int walker = blockIdx.x % (RT / 64);
+    const int64_t r0 = (int64_t)blockIdx.x * RR;
+    const int64_t tiles_per_seg = (seglen + RC - 1) / RC;
     const int64_t ntiles = nseg * tiles_per_seg;
 
     float acc = 0.0f;
-    float stage[ROWS / 4];
+    v4f stage[RV];
 
     auto load = [&](int64_t t) {
-        const int64_t s = t / tiles_per_seg, c0 = (t - s * tiles_per_seg) * TC;
-        const float *base = in + s * seg_stride + c0;
+        const int64_t sgm = t / tiles_per_seg, c0 = (t - sgm * tiles_per_seg) * RC;
+        const float *base = in + sgm * seg_stride + c0;
 #pragma unroll
-        for (int i = 0; i < ROWS / 4; i++)
+        for (int i = 0; i < RV; i++)
         {
-            const int64_t r = r0 + wave + 4 * i;
-            float v = 0.0f;
-            if (r < rows && c0 + lane < seglen)
-                v = base[r * row_stride + lane];
+            const int idx = tid + RT * i;
+            const int64_t r = r0 + idx / C4;
+            const int c = (idx % C4) << 2;
+            v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (r < rows)
+            {
+                const float *p = base + r * row_stride + c;
+                if (VEC && c0 + c + 3 < seglen)
+                    v = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(p));
+                else
+                {
+                    if (c0 + c + 0 < seglen) v.x = p[0];
+                    if (c0 + c + 1 < seglen) v.y = p[1];
+                    if (c0 + c + 2 < seglen) v.z = p[2];
+                    if (c0 + c + 3 < seglen) v.w = p[3];
+                }
+            }
             stage[i] = v;
         }
     };
-    auto store = [&](int buf) {
+    auto store = [&]() {
 #pragma unroll
-        for (int i = 0; i < ROWS / 4; i++)
-            tile[buf][(wave + 4 * i) * LDT + lane] = stage[i];
+        for (int i = 0; i < RV; i++)
+        {
+            const int idx = tid + RT * i;
+            *reinterpret_cast<v4f *>(&tile[(idx / C4) * RLD + ((idx % C4) << 2)]) = stage[i];
+        }
     };
 
     if (ntiles > 0)
     {
         load(0);
-        store(0);
+        store();
     }
     __syncthreads();
     for (int64_t t = 0; t < ntiles; t++)
     {
-        const int cur = (int)(t & 1);
         const bool more = t + 1 < ntiles;
         if (more)
             load(t + 1);
-        if (wave == 0)
+        if (wave == walker && lane < RR)
         {
-            const int64_t s = t / tiles_per_seg, c0 = (t - s * tiles_per_seg) * TC;
+            const int64_t sgm = t / tiles_per_seg, c0 = (t - sgm * tiles_per_seg) * RC;
             const int64_t rem = seglen - c0;
-            const float *row = &tile[cur][lane * LDT];
-            if (rem >= TC)
+            const float *row = &tile[lane * RLD];
+            if (rem >= RC)
             {
-#pragma unroll
-                for (int c = 0; c < TC; c++)
-                    acc = acc + row[c];
+#pragma unroll 8
+                for (int c = 0; c < RC; c += 4)
+                {
+                    const v4f v = *reinterpret_cast<const v4f *>(&row[c]);
+                    acc = acc + v.x;
+                    acc = acc + v.y;
+                    acc = acc + v.z;
+                    acc = acc + v.w;
+                }
             }
             else
             {
@@ -91,11 +124,12 @@ __global__ __launch_bounds__(RT) void rowchain_kernel(const float *__restrict__ 
                     acc = acc + row[c];
             }
         }
+        __syncthreads(); // the walk of tile t is over: the buffer may be overwritten
         if (more)
-            store(cur ^ 1);
+            store();
         __syncthreads();
     }
-    if (wave == 0 && r0 + lane < rows)
+    if (wave == walker && lane < RR && r0 + lane < rows)
         out[r0 + lane] = factor * acc;
 }
 
@@ -136,10 +170,33 @@ static int launch_rowchain(const float *in, float *out, int64_t rows, int64_t ns
 {
     if (rows == 0)
         return REPDL_OK;
-    const int64_t grid = repdl_cdiv(rows, ROWS);
+    // Chains per workgroup: enough workgroups to fill 256 CUs two to four times
+    // over, all resident at once, and as many walking lanes as that allows.
+    const bool vec = (reinterpret_cast<uintptr_t>(in) & 15) == 0 && row_stride % 4 == 0 && seg_stride % 4 == 0;
+    const int rr = rows >= 49152 ? 64 : rows >= 12288 ? 32 : rows >= 6144 ? 16 : 4;
+    const int64_t grid = repdl_cdiv(rows, rr);
     REPDL_REQUIRE(grid <= REPDL_I32_MAX);
-    hipLaunchKernelGGL(rowchain_kernel, dim3((unsigned)grid), dim3(RT), 0, repdl_stream(stream), in, out,
-                       rows, nseg, seglen, row_stride, seg_stride, factor);
+    const dim3 g((unsigned)grid);
+    hipStream_t st = repdl_stream(stream);
+#define REPDL_ROWCHAIN(RRv, RTv)                                                                                \
+    do                                                                                                         \
+    {                                                                                                          \
+        if (vec)                                                                                               \
+            hipLaunchKernelGGL((rowchain_kernel<RRv, RTv, true>), g, dim3(RTv), 0, st, in, out, rows, nseg,    \
+                               seglen, row_stride, seg_stride, factor);                                        \
+        else                                                                                                   \
+            hipLaunchKernelGGL((rowchain_kernel<RRv, RTv, false>), g, dim3(RTv), 0, st, in, out, rows, nseg,   \
+                               seglen, row_stride, seg_stride, factor);                                        \
+    } while (0)
+    if (rr == 64)
+        REPDL_ROWCHAIN(64, 256);
+    else if (rr == 32)
+        REPDL_ROWCHAIN(32, 128);
+    else if (rr == 16)
+        REPDL_ROWCHAIN(16, 256);
+    else
+        REPDL_ROWCHAIN(4, 256);
+#undef REPDL_ROWCHAIN
     return repdl_launch_status();
 }
 
