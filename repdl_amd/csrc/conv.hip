@@ -4,12 +4,23 @@
 // output element, starting at +0.0f, one fused multiply-add per contributing
 // tap in the reference's lexicographic loop order; taps that fall outside the
 // image (or, for grad-input, between strides) are SKIPPED, not multiplied by a
-// padded zero -- fma(0, w, acc) differs from a skip when acc is -0.0f or w is
-// not finite.
+// padded zero.
 //
-// These kernels walk each output's chain directly, one lane per output element
-// (grad-kernel: one lane per kernel element), with the spatially fastest index
-// on the lane so that neighbouring lanes read neighbouring addresses.
+// Forward and grad-input run as implicit GEMMs on the tiling of the mm kernel
+// (k-major LDS tiles, 8x8 register micro-tiles of v_fma_f32, K never split):
+//     forward     C[oc, pixel]  = sum_k W[oc, k] * im2col(X)[k, pixel],     k = (ic, kh, kw)
+//     grad-input  C[ic, pixel]  = sum_k W^T[ic, k] * col(GO)[k, pixel],     k = (oc, kh, kw)
+// with k running in exactly the reference's order.  The gathered operand holds a
+// zero where the reference skips a tap.  For finite data fma(0, w, acc) = acc
+// unless acc is -0.0f, and a zero sign can only survive to the end if the final
+// result is itself a zero; with non-finite data the padded product is a NaN that
+// sticks.  So a result that is neither zero nor NaN is already exactly the
+// reference's, and the epilogue recomputes the rare +-0 / NaN results with the
+// literal skip-the-tap chain (the *_exact functions below, which are also the
+// whole of the direct kernels).
+//
+// grad-kernel has only OC*IC*KH*KW outputs, each a chain as long as the batch
+// (N*OH*OW): it is limited by chain length and parallelism, not by FMA rate.
 #include "common.h"
 
 namespace
@@ -19,21 +30,14 @@ struct ConvDims
     int N, IC, H, W, OC, KH, KW, OH, OW, sH, sW, pH, pW, groups;
 };
 
-// backend/cpu/convolution.cpp:26-50
-__global__ __launch_bounds__(256) void conv2d_direct(const float *__restrict__ I,
-                                                     const float *__restrict__ Kr,
-                                                     float *__restrict__ O, ConvDims d,
-                                                     int64_t total)
+// ---------------------------------------------------------------------------
+// The literal chains (exact by construction).
+// ---------------------------------------------------------------------------
+
+// backend/cpu/convolution.cpp:30-48
+__device__ __forceinline__ float conv2d_exact(const float *__restrict__ I, const float *__restrict__ Kr,
+                                              const ConvDims &d, int n, int oc, int oh, int ow)
 {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= total)
-        return;
-    const int ow = (int)(idx % d.OW);
-    int64_t t = idx / d.OW;
-    const int oh = (int)(t % d.OH);
-    t /= d.OH;
-    const int oc = (int)(t % d.OC);
-    const int n = (int)(t / d.OC);
     const int ICg = d.IC / d.groups, OCg = d.OC / d.groups;
     const int g = oc / OCg;
     float sum = 0.0f;
@@ -56,24 +60,15 @@ __global__ __launch_bounds__(256) void conv2d_direct(const float *__restrict__ I
             }
         }
     }
-    O[idx] = sum;
+    return sum;
 }
 
-// backend/cpu/convolution.cpp:65-88
-__global__ __launch_bounds__(256) void conv2d_grad_input_direct(const float *__restrict__ GO,
-                                                                const float *__restrict__ Kr,
-                                                                float *__restrict__ GI, ConvDims d,
-                                                                int64_t total)
+// backend/cpu/convolution.cpp:71-86.  '/' truncates toward zero and '%' takes the
+// sign of the dividend, as in the reference (:75-77).
+__device__ __forceinline__ float conv2d_grad_input_exact(const float *__restrict__ GO,
+                                                         const float *__restrict__ Kr, const ConvDims &d,
+                                                         int n, int ic, int h, int w)
 {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= total)
-        return;
-    const int w = (int)(idx % d.W);
-    int64_t t = idx / d.W;
-    const int h = (int)(t % d.H);
-    t /= d.H;
-    const int ic = (int)(t % d.IC);
-    const int n = (int)(t / d.IC);
     float sum = 0.0f;
     for (int oc = 0; oc < d.OC; oc++)
     {
@@ -81,8 +76,6 @@ __global__ __launch_bounds__(256) void conv2d_grad_input_direct(const float *__r
         const float *kp = Kr + ((int64_t)oc * d.IC + ic) * d.KH * d.KW;
         for (int kh = 0; kh < d.KH; kh++)
         {
-            // C semantics: '/' truncates toward zero and '%' takes the sign of
-            // the dividend, as in the reference (:75-77).
             const int th = h - kh + d.pH;
             const int oh = th / d.sH;
             if (oh < 0 || oh >= d.OH || (th % d.sH) != 0)
@@ -97,24 +90,14 @@ __global__ __launch_bounds__(256) void conv2d_grad_input_direct(const float *__r
             }
         }
     }
-    GI[idx] = sum;
+    return sum;
 }
 
-// backend/cpu/convolution.cpp:103-126
-__global__ __launch_bounds__(64) void conv2d_grad_kernel_direct(const float *__restrict__ GO,
-                                                                const float *__restrict__ I,
-                                                                float *__restrict__ GK, ConvDims d,
-                                                                int64_t total)
+// backend/cpu/convolution.cpp:108-124
+__device__ __forceinline__ float conv2d_grad_kernel_exact(const float *__restrict__ GO,
+                                                          const float *__restrict__ I, const ConvDims &d,
+                                                          int oc, int ic, int kh, int kw)
 {
-    const int64_t idx = (int64_t)blockIdx.x * 64 + threadIdx.x;
-    if (idx >= total)
-        return;
-    const int kw = (int)(idx % d.KW);
-    int64_t t = idx / d.KW;
-    const int kh = (int)(t % d.KH);
-    t /= d.KH;
-    const int ic = (int)(t % d.IC);
-    const int oc = (int)(t / d.IC);
     float sum = 0.0f;
     for (int n = 0; n < d.N; n++)
     {
@@ -134,10 +117,670 @@ __global__ __launch_bounds__(64) void conv2d_grad_kernel_direct(const float *__r
             }
         }
     }
-    GK[idx] = sum;
+    return sum;
+}
+
+__global__ __launch_bounds__(64) void conv2d_grad_kernel_direct(const float *__restrict__ GO,
+                                                                const float *__restrict__ I,
+                                                                float *__restrict__ GK, ConvDims d,
+                                                                int64_t total)
+{
+    const int64_t idx = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (idx >= total)
+        return;
+    const int kw = (int)(idx % d.KW);
+    int64_t t = idx / d.KW;
+    const int kh = (int)(t % d.KH);
+    t /= d.KH;
+    const int ic = (int)(t % d.IC);
+    const int oc = (int)(t / d.IC);
+    GK[idx] = conv2d_grad_kernel_exact(GO, I, d, oc, ic, kh, kw);
+}
+
+// ---------------------------------------------------------------------------
+// Implicit GEMM for forward (MODE_FWD) and grad-input (MODE_DGRAD).
+// Tile BM x 128 outputs (BM = 64 or 128 rows = output / input channels, 128
+// columns = pixels of one image), BK = 16, 2*BM threads, 8x8 micro-tile per lane.
+// ---------------------------------------------------------------------------
+constexpr int BN = 128, BK = 16, LDB = BN + 4;
+enum
+{
+    MODE_FWD = 0,
+    MODE_DGRAD = 1
+};
+
+// position of a k index in the (channel, kh, kw) mixed radix, advanced by BK per
+// k-tile without divisions
+struct KPos
+{
+    int c, kh, kw;
+};
+
+struct KStep
+{
+    int dc, dkh, dkw; // BK = dc*KH*KW + dkh*KW + dkw
+};
+
+__device__ __forceinline__ void kpos_advance(KPos &p, const KStep &s, int KH, int KW)
+{
+    p.kw += s.dkw;
+    if (p.kw >= KW)
+    {
+        p.kw -= KW;
+        p.kh++;
+    }
+    p.kh += s.dkh;
+    if (p.kh >= KH)
+    {
+        p.kh -= KH;
+        p.c++;
+    }
+    p.c += s.dc;
+}
+
+template <int BM, int MODE>
+__global__ __launch_bounds__(2 * BM) void conv_gemm_kernel(const float *__restrict__ Xg, // gathered operand: input (FWD) / grad_output (DGRAD)
+                                                           const float *__restrict__ Wt, // kernel
+                                                           float *__restrict__ Out, ConvDims d, int wvec,
+                                                           int ovec)
+{
+    constexpr int NT = 2 * BM;
+    constexpr int LDA = BM + 4;
+    constexpr int NA = BM * BK / 4 / NT;  // float4 slots of A per thread (2)
+    constexpr int NB = BN * BK / 4 / NT;  // float4 slots of B per thread (4 or 2)
+    constexpr int KSTRIDE_B = NT / 32;    // k rows between two B slots of a thread
+    __shared__ __attribute__((aligned(16))) float As[2][BK * LDA];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB];
+
+    const int tid = threadIdx.x;
+    const int tx = tid & 15, ty = tid >> 4;
+    const int KHW = d.KH * d.KW;
+    const int ICg = d.IC / d.groups, OCg = d.OC / d.groups;
+    // GEMM extents
+    const int M = MODE == MODE_FWD ? OCg : d.IC;
+    const int K = (MODE == MODE_FWD ? ICg : d.OC) * KHW;
+    const int P = MODE == MODE_FWD ? d.OH * d.OW : d.H * d.W; // pixels (columns) per image
+    const int PW = MODE == MODE_FWD ? d.OW : d.W;
+    const int n = MODE == MODE_FWD ? blockIdx.z / d.groups : blockIdx.z;
+    const int g = MODE == MODE_FWD ? blockIdx.z % d.groups : 0;
+    const int m0 = blockIdx.y * BM, p0 = blockIdx.x * BN;
+
+    KStep kstep;
+    kstep.dc = BK / KHW;
+    kstep.dkh = (BK % KHW) / d.KW;
+    kstep.dkw = (BK % KHW) % d.KW;
+
+    // ---- B (gathered) operand: this thread's four pixels ----
+    const int p4 = (tid & 31) << 2;
+    int pb_h[4], pb_w[4]; // FWD: oh*sH-pH, ow*sW-pW;  DGRAD: h+pH, w+pW
+    bool pvalid[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+    {
+        const int pix = p0 + p4 + j;
+        pvalid[j] = pix < P;
+        const int ph = pix / PW, pw = pix - ph * PW;
+        if (MODE == MODE_FWD)
+        {
+            pb_h[j] = ph * d.sH - d.pH;
+            pb_w[j] = pw * d.sW - d.pW;
+        }
+        else
+        {
+            pb_h[j] = ph + d.pH;
+            pb_w[j] = pw + d.pW;
+        }
+    }
+    KPos bpos[NB];
+    int bk[NB];
+#pragma unroll
+    for (int i = 0; i < NB; i++)
+    {
+        const int k = (tid >> 5) + KSTRIDE_B * i;
+        bk[i] = k;
+        bpos[i].c = k / KHW;
+        const int rem = k - bpos[i].c * KHW;
+        bpos[i].kh = rem / d.KW;
+        bpos[i].kw = rem - bpos[i].kh * d.KW;
+    }
+    // ---- A (kernel) operand ----
+    // FWD: element (m, k) = Wg[m*K + k] (k contiguous): slot = (row idx>>2, 4 k's).
+    // DGRAD: element (m=ic, k=(oc,kh,kw)) = W[(oc*IC + ic)*KHW + kh*KW + kw]: slot =
+    // (k row, 4 consecutive ic), gathered with stride KHW.
+    const float *Wg = MODE == MODE_FWD ? Wt + (int64_t)g * OCg * K : Wt;
+    constexpr int A_R4 = BM / 4;             // DGRAD: float4 groups per k row
+    constexpr int KSTRIDE_A = NT / A_R4;     // DGRAD: k rows between two A slots (8)
+    KPos apos[NA];
+    int ak[NA];
+    if (MODE == MODE_DGRAD)
+    {
+#pragma unroll
+        for (int i = 0; i < NA; i++)
+        {
+            const int k = tid / A_R4 + KSTRIDE_A * i;
+            ak[i] = k;
+            apos[i].c = k / KHW;
+            const int rem = k - apos[i].c * KHW;
+            apos[i].kh = rem / d.KW;
+            apos[i].kw = rem - apos[i].kh * d.KW;
+        }
+    }
+
+    float4 fa[NA], fb[NB];
+
+    auto load_a = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < NA; i++)
+        {
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (MODE == MODE_FWD)
+            {
+                const int idx = tid + NT * i;
+                const int r = m0 + (idx >> 2), k = k0 + ((idx & 3) << 2);
+                if (r < M)
+                {
+                    const float *p = Wg + (int64_t)r * K + k;
+                    if (wvec && k + 3 < K)
+                        v = *reinterpret_cast<const float4 *>(p);
+                    else
+                    {
+                        if (k + 0 < K) v.x = p[0];
+                        if (k + 1 < K) v.y = p[1];
+                        if (k + 2 < K) v.z = p[2];
+                        if (k + 3 < K) v.w = p[3];
+                    }
+                }
+            }
+            else
+            {
+                const int r = m0 + ((tid % A_R4) << 2);
+                if (ak[i] < K)
+                {
+                    const float *p = Wg + ((int64_t)apos[i].c * d.IC + r) * KHW + apos[i].kh * d.KW + apos[i].kw;
+                    if (r + 0 < M) v.x = p[0];
+                    if (r + 1 < M) v.y = p[KHW];
+                    if (r + 2 < M) v.z = p[2 * KHW];
+                    if (r + 3 < M) v.w = p[3 * KHW];
+                }
+                ak[i] += BK;
+                kpos_advance(apos[i], kstep, d.KH, d.KW);
+            }
+            fa[i] = v;
+        }
+    };
+    auto store_a = [&](float *S) {
+#pragma unroll
+        for (int i = 0; i < NA; i++)
+        {
+            if (MODE == MODE_FWD)
+            {
+                const int idx = tid + NT * i;
+                const int r = idx >> 2, k = (idx & 3) << 2;
+                S[(k + 0) * LDA + r] = fa[i].x;
+                S[(k + 1) * LDA + r] = fa[i].y;
+                S[(k + 2) * LDA + r] = fa[i].z;
+                S[(k + 3) * LDA + r] = fa[i].w;
+            }
+            else
+            {
+                const int k = tid / A_R4 + KSTRIDE_A * i, r = (tid % A_R4) << 2;
+                *reinterpret_cast<float4 *>(&S[k * LDA + r]) = fa[i];
+            }
+        }
+    };
+    auto load_b = [&]() {
+#pragma unroll
+        for (int i = 0; i < NB; i++)
+        {
+            float v[4] = {0.f, 0.f, 0.f, 0.f};
+            if (bk[i] < K)
+            {
+                if (MODE == MODE_FWD)
+                {
+                    const float *base = Xg + ((int64_t)n * d.IC + g * ICg + bpos[i].c) * d.H * d.W;
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                    {
+                        const int h = pb_h[j] + bpos[i].kh, w = pb_w[j] + bpos[i].kw;
+                        if (pvalid[j] && (unsigned)h < (unsigned)d.H && (unsigned)w < (unsigned)d.W)
+                            v[j] = base[h * d.W + w];
+                    }
+                }
+                else
+                {
+                    const float *base = Xg + ((int64_t)n * d.OC + bpos[i].c) * d.OH * d.OW;
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                    {
+                        const int th = pb_h[j] - bpos[i].kh, tw = pb_w[j] - bpos[i].kw;
+                        int oh = th, ow = tw;
+                        bool ok = pvalid[j] && th >= 0 && tw >= 0;
+                        if (d.sH != 1)
+                        {
+                            oh = th / d.sH;
+                            ok = ok && (th - oh * d.sH) == 0;
+                        }
+                        if (d.sW != 1)
+                        {
+                            ow = tw / d.sW;
+                            ok = ok && (tw - ow * d.sW) == 0;
+                        }
+                        if (ok && oh < d.OH && ow < d.OW)
+                            v[j] = base[oh * d.OW + ow];
+                    }
+                }
+            }
+            bk[i] += BK;
+            kpos_advance(bpos[i], kstep, d.KH, d.KW);
+            fb[i] = make_float4(v[0], v[1], v[2], v[3]);
+        }
+    };
+    auto store_b = [&](float *S) {
+#pragma unroll
+        for (int i = 0; i < NB; i++)
+        {
+            const int k = (tid >> 5) + KSTRIDE_B * i;
+            *reinterpret_cast<float4 *>(&S[k * LDB + p4]) = fb[i];
+        }
+    };
+
+    float acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            acc[i][j] = 0.0f;
+
+    auto fma_step = [&](const float *A, const float *B, int kk) {
+        const float4 a0 = *reinterpret_cast<const float4 *>(&A[kk * LDA + ty * 4]);
+        const float4 a1 = *reinterpret_cast<const float4 *>(&A[kk * LDA + BM / 2 + ty * 4]);
+        const float4 b0 = *reinterpret_cast<const float4 *>(&B[kk * LDB + tx * 4]);
+        const float4 b1 = *reinterpret_cast<const float4 *>(&B[kk * LDB + 64 + tx * 4]);
+        const float a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+        const float b[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                acc[i][j] = __fmaf_rn(a[i], b[j], acc[i][j]);
+    };
+
+    const int nkt = (K + BK - 1) / BK;
+    if (nkt > 0)
+    {
+        load_a(0);
+        load_b();
+        store_a(As[0]);
+        store_b(Bs[0]);
+    }
+    __syncthreads();
+    for (int kt = 0; kt < nkt; kt++)
+    {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < nkt;
+        if (more)
+        {
+            load_a((kt + 1) * BK);
+            load_b();
+        }
+        const int krem = K - kt * BK;
+        if (krem >= BK)
+        {
+#pragma unroll
+            for (int kk = 0; kk < BK; kk++)
+                fma_step(As[cur], Bs[cur], kk);
+        }
+        else
+        {
+            for (int kk = 0; kk < krem; kk++)
+                fma_step(As[cur], Bs[cur], kk);
+        }
+        if (more)
+        {
+            store_a(As[cur ^ 1]);
+            store_b(Bs[cur ^ 1]);
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue: exact recompute of +-0 / NaN results, then store ----
+    float *Oimg = Out + (int64_t)n * (MODE == MODE_FWD ? d.OC : d.IC) * P;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+    {
+        const int m = m0 + ty * 4 + (i & 3) + (i >> 2) * (BM / 2);
+        if (m >= M)
+            continue;
+        const int ch = MODE == MODE_FWD ? g * OCg + m : m; // output channel (FWD) / input channel (DGRAD)
+#pragma unroll
+        for (int jh = 0; jh < 2; jh++)
+        {
+            const int pix = p0 + tx * 4 + jh * 64;
+            float v[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+            {
+                v[j] = acc[i][jh * 4 + j];
+                const bool suspect = ((__float_as_uint(v[j]) << 1) == 0u) || (v[j] != v[j]);
+                if (suspect && pix + j < P)
+                {
+                    const int ph = (pix + j) / PW, pw = (pix + j) - ph * PW;
+                    v[j] = MODE == MODE_FWD ? conv2d_exact(Xg, Wt, d, n, ch, ph, pw)
+                                            : conv2d_grad_input_exact(Xg, Wt, d, n, ch, ph, pw);
+                }
+            }
+            float *p = Oimg + (int64_t)ch * P + pix;
+            if (ovec && pix + 3 < P)
+                *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+            else
+            {
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (pix + j < P)
+                        p[j] = v[j];
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// grad-kernel.  GK[oc][ic][kh][kw] is a chain over k = (n, oh, ow): there are
+// only OC*IC*KH*KW chains and K = N*OH*OW cannot be split, so one LANE owns one
+// chain (one dependent v_fma_f32 per k) and the kernel is shaped to make a k
+// step cost little more than that FMA:
+//   * a wave = one oc x 64 consecutive (ic,kh,kw) columns.  Its grad_output
+//     value is wave-uniform: lane l loads element l of a 64-wide piece of an
+//     output row (one coalesced load, issued a whole chunk ahead), and step k
+//     broadcasts lane k with v_readlane_b32 into an SGPR that feeds the FMA;
+//   * a workgroup = 4 waves (4 oc) sharing the same columns; the input rows
+//     those columns touch are staged once per workgroup in LDS, zero-padded
+//     left and right, so a lane's tap for consecutive ow is a ds_read_b32 at a
+//     fixed offset (+ow*sW) and out-of-image taps read a zero;
+//   * a chunk = R output rows of one image; the next chunk's input rows and
+//     grad_output pieces are loaded into registers before the FMAs of the
+//     current one (two LDS buffers).
+// Every piece runs PIECE (16/32/64) steps: steps beyond the end of the row read
+// the zero pad and a zero grad_output.  These padded zeros make the same +-0 /
+// NaN results suspect as in the implicit GEMMs; those are recomputed with the
+// literal chain.
+// ---------------------------------------------------------------------------
+// value of v in lane k (a compile-time lane index), broadcast as a wave-uniform scalar
+__device__ __forceinline__ float lane_value(float v, int k)
+{
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), k));
+}
+
+// One step of a chain, written as an instruction pair so that the broadcast for step
+// k+16 is issued next to the FMA of step k: v_readlane_b32 has a long latency before
+// its SGPR result can feed a VALU operand (about 12 clocks measured), short enough to
+// hide behind sixteen dependent FMAs but not behind one.
+#define REPDL_WG_STEP(u)                                                                                     \
+    asm volatile("v_readlane_b32 %0, %2, %3\n\tv_fmac_f32_e32 %1, %4, %5"                                    \
+                 : "=&s"(gn[u]), "+v"(acc)                                                                   \
+                 : "v"(g), "n"(K0 + 16 + (u)), "s"(gc[u]), "v"(xv[u]))
+#define REPDL_WG_LAST(u) asm volatile("v_fmac_f32_e32 %0, %1, %2" : "+v"(acc) : "s"(gc[u]), "v"(xv[u]))
+
+// sixteen steps K0..K0+15 of a piece; gc = broadcast values of these steps, gn receives
+// those of the next sixteen (when there are any)
+template <int K0, bool MORE>
+__device__ __forceinline__ float wgrad_steps16(int g, const int (&gc)[16], int (&gn)[16], const float (&xv)[16],
+                                               float acc)
+{
+    if (MORE)
+    {
+        REPDL_WG_STEP(0); REPDL_WG_STEP(1); REPDL_WG_STEP(2); REPDL_WG_STEP(3);
+        REPDL_WG_STEP(4); REPDL_WG_STEP(5); REPDL_WG_STEP(6); REPDL_WG_STEP(7);
+        REPDL_WG_STEP(8); REPDL_WG_STEP(9); REPDL_WG_STEP(10); REPDL_WG_STEP(11);
+        REPDL_WG_STEP(12); REPDL_WG_STEP(13); REPDL_WG_STEP(14); REPDL_WG_STEP(15);
+    }
+    else
+    {
+        REPDL_WG_LAST(0); REPDL_WG_LAST(1); REPDL_WG_LAST(2); REPDL_WG_LAST(3);
+        REPDL_WG_LAST(4); REPDL_WG_LAST(5); REPDL_WG_LAST(6); REPDL_WG_LAST(7);
+        REPDL_WG_LAST(8); REPDL_WG_LAST(9); REPDL_WG_LAST(10); REPDL_WG_LAST(11);
+        REPDL_WG_LAST(12); REPDL_WG_LAST(13); REPDL_WG_LAST(14); REPDL_WG_LAST(15);
+    }
+    return acc;
+}
+#undef REPDL_WG_STEP
+#undef REPDL_WG_LAST
+
+template <bool UNIT>
+__device__ __forceinline__ void wgrad_read16(const float *__restrict__ xr, int k0, int sW, float (&xv)[16])
+{
+#pragma unroll
+    for (int u = 0; u < 16; u++)
+        xv[u] = UNIT ? xr[k0 + u] : xr[(k0 + u) * sW];
+}
+
+// PIECE steps of one chain: the taps come from LDS sixteen at a time (the next sixteen
+// are read before the FMAs of the current ones), the grad_output values from lane k of g.
+template <int PIECE, bool UNIT>
+__device__ __forceinline__ float wgrad_piece(float gf, const float *__restrict__ xr, int sW, float acc)
+{
+    const int g = __float_as_int(gf);
+    int ga[16], gb[16];
+    float xa[16], xb[16];
+#pragma unroll
+    for (int u = 0; u < 16; u++)
+        ga[u] = __builtin_amdgcn_readlane(g, u);
+    wgrad_read16<UNIT>(xr, 0, sW, xa);
+    if (PIECE == 16)
+        return wgrad_steps16<0, false>(g, ga, gb, xa, acc);
+    wgrad_read16<UNIT>(xr, 16, sW, xb);
+    acc = wgrad_steps16<0, true>(g, ga, gb, xa, acc);
+    if (PIECE == 32)
+        return wgrad_steps16<16, false>(g, gb, ga, xb, acc);
+    wgrad_read16<UNIT>(xr, 32, sW, xa);
+    acc = wgrad_steps16<16, true>(g, gb, ga, xb, acc);
+    wgrad_read16<UNIT>(xr, 48, sW, xb);
+    acc = wgrad_steps16<32, true>(g, ga, gb, xa, acc);
+    return wgrad_steps16<48, false>(g, gb, ga, xb, acc);
+}
+
+constexpr int WG_SLOTS = 16; // float4 staging slots per thread (16 rows x 64 floats per pass)
+constexpr int WG_Q = 16;    // row pieces per chunk (one register of grad_output each)
+
+template <int PIECE>
+__global__ __launch_bounds__(256) void conv_wgrad_kernel(const float *__restrict__ GO,
+                                                         const float *__restrict__ X,
+                                                         float *__restrict__ GK, ConvDims d, int R, int NP,
+                                                         int Wp, int CP, int hrows, int bufsz, int xvec)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int KHW = d.KH * d.KW, NC = d.IC * KHW;
+    const int c0 = blockIdx.x * 64;
+    const int col = c0 + lane;
+    const bool cvalid = col < NC;
+    const int colc = cvalid ? col : NC - 1;
+    const int ic = colc / KHW;
+    const int rem = colc - ic * KHW;
+    const int kh = rem / d.KW, kw = rem - kh * d.KW;
+    const int ic_first = c0 / KHW;
+    const int last_col = (c0 + 63 < NC) ? c0 + 63 : NC - 1;
+    const int nic = last_col / KHW - ic_first + 1;
+    const int nrows = nic * hrows; // staged rows per chunk
+    const int oc = blockIdx.y * 4 + wave;
+    const bool ovalid = oc < d.OC;
+    const int occ = ovalid ? oc : d.OC - 1;
+    const int lane_off = (ic - ic_first) * CP + kh * Wp + kw;
+
+    // both buffers start as zeros; staging only ever writes [pW, pW + roundup4(W)) of a
+    // row, with zeros beyond W, so the left and right pads stay zero
+    for (int i = tid; i < 2 * bufsz; i += 256)
+        lds[i] = 0.0f;
+
+    // staging slots of this thread: slot q covers row (tid>>4) + 16*(q / nseg), floats
+    // [64*(q % nseg) + 4*(tid&15), +4) of that row
+    const int nseg = (d.W + 63) >> 6;
+    const int npass = (nrows + 15) >> 4;
+    int s_goff[WG_SLOTS], s_hr[WG_SLOTS], s_w[WG_SLOTS], s_loff[WG_SLOTS];
+#pragma unroll
+    for (int q = 0; q < WG_SLOTS; q++)
+    {
+        const int pass = q / nseg, seg = q - pass * nseg;
+        const int row = (tid >> 4) + 16 * pass;
+        const int w = 64 * seg + 4 * (tid & 15);
+        const bool on = pass < npass && row < nrows && w < d.W;
+        const int icl = row / hrows, hr = row - icl * hrows;
+        s_goff[q] = (ic_first + icl) * d.H * d.W + w;
+        s_hr[q] = hr;
+        s_w[q] = w;
+        s_loff[q] = on ? icl * CP + hr * Wp + d.pW + w : -1;
+    }
+    __syncthreads();
+
+    float4 stage[WG_SLOTS];
+    float gnext[WG_Q], gcur[WG_Q];
+    // input rows and grad_output pieces of chunk (n, oh0) -> registers
+    auto chunk_load = [&](int n, int oh0) {
+        const float *Xn = X + (int64_t)n * d.IC * d.H * d.W;
+        const int hbase = oh0 * d.sH - d.pH;
+#pragma unroll
+        for (int q = 0; q < WG_SLOTS; q++)
+        {
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            const int h = hbase + s_hr[q];
+            if (s_loff[q] >= 0 && h >= 0 && h < d.H)
+            {
+                const float *p = Xn + s_goff[q] + h * d.W;
+                if (xvec && s_w[q] + 3 < d.W)
+                    v = *reinterpret_cast<const float4 *>(p);
+                else
+                {
+                    if (s_w[q] + 0 < d.W) v.x = p[0];
+                    if (s_w[q] + 1 < d.W) v.y = p[1];
+                    if (s_w[q] + 2 < d.W) v.z = p[2];
+                    if (s_w[q] + 3 < d.W) v.w = p[3];
+                }
+            }
+            stage[q] = v;
+        }
+        const float *gp = GO + (((int64_t)n * d.OC + occ) * d.OH + oh0) * d.OW;
+        const int Rc = (d.OH - oh0 < R) ? d.OH - oh0 : R;
+        int r = 0, pc = 0;
+#pragma unroll
+        for (int q = 0; q < WG_Q; q++)
+        {
+            float g = 0.0f;
+            const int ow = pc * PIECE + lane;
+            if (r < Rc && lane < PIECE && ow < d.OW)
+                g = gp[r * d.OW + ow];
+            gnext[q] = g;
+            if (++pc == NP)
+            {
+                pc = 0;
+                r++;
+            }
+        }
+    };
+    auto stage_store = [&](int buf) {
+#pragma unroll
+        for (int q = 0; q < WG_SLOTS; q++)
+            if (s_loff[q] >= 0)
+            {
+                float *p = &lds[buf * bufsz + s_loff[q]];
+                p[0] = stage[q].x;
+                p[1] = stage[q].y;
+                p[2] = stage[q].z;
+                p[3] = stage[q].w;
+            }
+    };
+
+    float acc = 0.0f;
+    int n = 0, oh0 = 0;
+    const bool any = d.N > 0 && d.OH > 0 && d.OW > 0;
+    if (any)
+    {
+        chunk_load(0, 0);
+        stage_store(0);
+    }
+    __syncthreads();
+    int buf = 0;
+    while (any)
+    {
+#pragma unroll
+        for (int q = 0; q < WG_Q; q++)
+            gcur[q] = gnext[q];
+        int n1 = n, oh1 = oh0 + R;
+        if (oh1 >= d.OH)
+        {
+            oh1 = 0;
+            n1 = n + 1;
+        }
+        const bool more = n1 < d.N;
+        if (more)
+            chunk_load(n1, oh1);
+        {
+            const int nq = ((d.OH - oh0 < R) ? d.OH - oh0 : R) * NP;
+            const float *xs = lds + buf * bufsz + lane_off;
+            int r = 0, pc = 0;
+#pragma unroll
+            for (int q = 0; q < WG_Q; q++)
+            {
+                if (q < nq)
+                {
+                    const float *xr = xs + r * d.sH * Wp + pc * PIECE * d.sW;
+                    if (d.sW == 1)
+                        acc = wgrad_piece<PIECE, true>(gcur[q], xr, 1, acc);
+                    else
+                        acc = wgrad_piece<PIECE, false>(gcur[q], xr, d.sW, acc);
+                }
+                if (++pc == NP)
+                {
+                    pc = 0;
+                    r++;
+                }
+            }
+        }
+        if (more)
+            stage_store(buf ^ 1);
+        __syncthreads();
+        if (!more)
+            break;
+        buf ^= 1;
+        n = n1;
+        oh0 = oh1;
+    }
+    if (ovalid && cvalid)
+    {
+        if (((__float_as_uint(acc) << 1) == 0u) || (acc != acc))
+            acc = conv2d_grad_kernel_exact(GO, X, d, oc, ic, kh, kw);
+        GK[(int64_t)oc * NC + col] = acc;
+    }
 }
 
 inline bool fits_i32(int64_t v) { return v >= 0 && v <= REPDL_I32_MAX; }
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+template <int MODE>
+int launch_conv_gemm(const float *gathered, const float *kernel, float *out, const ConvDims &d, void *stream)
+{
+    const int KHW = d.KH * d.KW;
+    const int M = MODE == MODE_FWD ? d.OC / d.groups : d.IC;
+    const int64_t K = (int64_t)(MODE == MODE_FWD ? d.IC / d.groups : d.OC) * KHW;
+    const int64_t P = MODE == MODE_FWD ? (int64_t)d.OH * d.OW : (int64_t)d.H * d.W;
+    const int64_t gz = MODE == MODE_FWD ? (int64_t)d.N * d.groups : d.N;
+    const int64_t gx = repdl_cdiv(P, BN);
+    REPDL_REQUIRE(gz <= 65535 && fits_i32(gx) && fits_i32(K));
+    const int wvec = MODE == MODE_FWD && aligned16(kernel) && (K % 4 == 0);
+    const int ovec = aligned16(out) && (P % 4 == 0);
+    hipStream_t s = repdl_stream(stream);
+    if (M <= 64)
+    {
+        dim3 grid((unsigned)gx, (unsigned)repdl_cdiv(M, 64), (unsigned)gz);
+        hipLaunchKernelGGL((conv_gemm_kernel<64, MODE>), grid, dim3(128), 0, s, gathered, kernel, out, d, wvec, ovec);
+    }
+    else
+    {
+        dim3 grid((unsigned)gx, (unsigned)repdl_cdiv(M, 128), (unsigned)gz);
+        REPDL_REQUIRE(grid.y <= 65535);
+        hipLaunchKernelGGL((conv_gemm_kernel<128, MODE>), grid, dim3(256), 0, s, gathered, kernel, out, d, wvec, ovec);
+    }
+    return repdl_launch_status();
+}
 } // namespace
 
 REPDL_API int repdl_hip_conv2d(const float *input, const float *kernel, float *output, int64_t N,
@@ -155,13 +798,10 @@ REPDL_API int repdl_hip_conv2d(const float *input, const float *kernel, float *o
         return REPDL_OK;
     REPDL_REQUIRE(input != nullptr && kernel != nullptr && output != nullptr);
     REPDL_REQUIRE(fits_i32(H * W) && fits_i32(OH * OW) && fits_i32(IC * KH * KW) && fits_i32(N) && fits_i32(OC));
-    const int64_t grid = repdl_cdiv(total, 256);
-    REPDL_REQUIRE(fits_i32(grid));
+    REPDL_REQUIRE(fits_i32(OH * sH + KH + pH) && fits_i32(OW * sW + KW + pW));
     ConvDims d{(int)N, (int)IC, (int)H, (int)W, (int)OC, (int)KH, (int)KW, (int)OH,
                (int)OW, (int)sH, (int)sW, (int)pH, (int)pW, (int)groups};
-    hipLaunchKernelGGL(conv2d_direct, dim3((unsigned)grid), dim3(256), 0, repdl_stream(stream), input, kernel,
-                       output, d, total);
-    return repdl_launch_status();
+    return launch_conv_gemm<MODE_FWD>(input, kernel, output, d, stream);
 }
 
 REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float *kernel,
@@ -178,14 +818,10 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
     REPDL_REQUIRE(grad_input != nullptr);
     REPDL_REQUIRE(OC * OH * OW == 0 || (grad_output != nullptr && kernel != nullptr));
     REPDL_REQUIRE(fits_i32(H * W) && fits_i32(OH * OW) && fits_i32(OC * KH * KW) && fits_i32(N) && fits_i32(IC));
-    REPDL_REQUIRE(fits_i32(H + pH) && fits_i32(W + pW));
-    const int64_t grid = repdl_cdiv(total, 256);
-    REPDL_REQUIRE(fits_i32(grid));
+    REPDL_REQUIRE(fits_i32(H + pH + KH) && fits_i32(W + pW + KW) && fits_i32(IC * KH * KW * 4));
     ConvDims d{(int)N, (int)IC, (int)H, (int)W, (int)OC, (int)KH, (int)KW, (int)OH,
                (int)OW, (int)sH, (int)sW, (int)pH, (int)pW, 1};
-    hipLaunchKernelGGL(conv2d_grad_input_direct, dim3((unsigned)grid), dim3(256), 0, repdl_stream(stream),
-                       grad_output, kernel, grad_input, d, total);
-    return repdl_launch_status();
+    return launch_conv_gemm<MODE_DGRAD>(grad_output, kernel, grad_input, d, stream);
 }
 
 REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float *input,
@@ -203,11 +839,71 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
     REPDL_REQUIRE(N * OH * OW == 0 || (grad_output != nullptr && input != nullptr));
     REPDL_REQUIRE(fits_i32(H * W) && fits_i32(OH * OW) && fits_i32(N) && fits_i32(IC) && fits_i32(OC));
     REPDL_REQUIRE(fits_i32(OH * sH + KH) && fits_i32(OW * sW + KW));
-    const int64_t grid = repdl_cdiv(total, 64);
-    REPDL_REQUIRE(fits_i32(grid));
     ConvDims d{(int)N, (int)IC, (int)H, (int)W, (int)OC, (int)KH, (int)KW, (int)OH,
                (int)OW, (int)sH, (int)sW, (int)pH, (int)pW, 1};
-    hipLaunchKernelGGL(conv2d_grad_kernel_direct, dim3((unsigned)grid), dim3(64), 0, repdl_stream(stream),
-                       grad_output, input, grad_kernel, d, total);
+    hipStream_t s = repdl_stream(stream);
+
+    // Geometry.  A row of OW outputs is cut into NP pieces of PIECE (16/32/64) steps;
+    // steps past the end of the row must read zeros, so the staged row pitch Wp covers
+    // what is written (pW + roundup4(W)) and what the taps of NP*PIECE steps reach.
+    // Lane l of a wave reads LDS word (ic-ic0)*CP + kh*Wp + kw (+ a wave-uniform offset);
+    // with Wp = KW and CP = KH*KW modulo 32 that is l + const modulo 32: two lanes per
+    // bank, the minimum for 64 lanes.
+    const int64_t KHW = KH * KW, NC = IC * KHW;
+    const int piece = OW <= 16 ? 16 : OW <= 32 ? 32 : 64;
+    const int64_t NP = repdl_cdiv(OW, piece);
+    int64_t Wp = pW + (W + 3) / 4 * 4;
+    const int64_t reach = (NP * piece - 1) * sW + KW;
+    if (reach > Wp)
+        Wp = reach;
+    while (Wp % 32 != KW % 32)
+        Wp++;
+    const int64_t span = (63 + KHW - 1) / KHW + 1; // channels a 64-column block can span
+    const int64_t nic_max = span < IC ? span : IC;
+    const int64_t nseg = (W + 63) / 64;
+    // largest R (output rows per chunk) that fits WG_Q pieces, WG_SLOTS staging slots per
+    // thread and 150 KiB of LDS
+    int64_t R = 0, hrows = 0;
+    for (int64_t r = (OH < WG_Q ? OH : WG_Q); r >= 1; r--)
+    {
+        const int64_t hr = (r - 1) * sH + KH;
+        const int64_t slots = repdl_cdiv(nic_max * hr, 16) * nseg;
+        if (r * NP <= WG_Q && slots <= WG_SLOTS && 2 * nic_max * (hr * Wp + 31) * 4 <= 150 * 1024)
+        {
+            R = r;
+            hrows = hr;
+            break;
+        }
+    }
+    int64_t CP = hrows * Wp; // channel pitch
+    while (CP % 32 != KHW % 32)
+        CP++;
+    const int64_t bufsz = nic_max * CP;
+    const int xvec = aligned16(input) && (W % 4 == 0);
+    const int64_t gx = repdl_cdiv(NC, 64), gy = repdl_cdiv(OC, 4);
+    REPDL_REQUIRE(fits_i32(gx) && gy <= 65535);
+    const dim3 grid((unsigned)gx, (unsigned)gy);
+    // More than half of a CU's 160 KiB of LDS: one workgroup per CU, so that each of its
+    // four waves has a SIMD to itself (the chains are latency-bound, not throughput-bound).
+    size_t shmem = (size_t)(2 * bufsz * 4);
+    if (shmem < 84 * 1024)
+        shmem = 84 * 1024;
+#define REPDL_WGRAD(P)                                                                                          \
+    do                                                                                                         \
+    {                                                                                                          \
+        hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_wgrad_kernel<P>),             \
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);           \
+        if (e_ != hipSuccess)                                                                                  \
+            return (int)e_;                                                                                    \
+        hipLaunchKernelGGL((conv_wgrad_kernel<P>), grid, dim3(256), shmem, s, grad_output, input, grad_kernel, \
+                           d, (int)R, (int)NP, (int)Wp, (int)CP, (int)hrows, (int)bufsz, xvec);                \
+    } while (0)
+    if (piece == 16)
+        REPDL_WGRAD(16);
+    else if (piece == 32)
+        REPDL_WGRAD(32);
+    else
+        REPDL_WGRAD(64);
+#undef REPDL_WGRAD
     return repdl_launch_status();
 }
