@@ -1,0 +1,163 @@
+"""The Python glue (autograd Functions, modules, from_torch_module, optimizers) run
+on CPU tensors with the oracle behind repdl_amd.ops (a test-only monkeypatch):
+gradients must equal PyTorch autograd exactly on integer-valued data and within
+float tolerance on random data; which operator is called in which order follows
+the reference (repdl/nn/linear.py:11-38, conv.py:11-50, loss.py:11-34)."""
+import numpy as np
+import pytest
+import torch
+
+import gen
+import models
+import repdl_amd
+from oracle_ops import oracle_for_cpu_tensors
+
+
+def test_linear_matches_autograd():
+    with oracle_for_cpu_tensors():
+        lin_t = torch.nn.Linear(7, 5)
+        with torch.no_grad():
+            lin_t.weight.copy_(gen.small_ints(1, 5, 7))
+            lin_t.bias.copy_(gen.small_ints(2, 5))
+        lin_r = repdl_amd.from_torch_module(lin_t)
+        x1 = gen.small_ints(3, 9, 7).requires_grad_(True)
+        x2 = x1.detach().clone().requires_grad_(True)
+        go = gen.small_ints(4, 9, 5)
+        lin_t(x1).backward(go)
+        y = lin_r(x2)
+        y.backward(go)
+        assert torch.equal(y, lin_t(x1))
+        assert torch.equal(x2.grad, x1.grad)
+        assert torch.equal(lin_r.weight.grad, lin_t.weight.grad)
+        assert torch.equal(lin_r.bias.grad, lin_t.bias.grad)
+        with pytest.raises(NotImplementedError):
+            lin_r(torch.zeros(2, 3, 7))
+
+
+@pytest.mark.parametrize("stride,padding", [(1, 1), (2, 0), ((2, 1), (0, 2))])
+def test_conv2d_matches_autograd(stride, padding):
+    with oracle_for_cpu_tensors():
+        c_t = torch.nn.Conv2d(3, 4, 3, stride=stride, padding=padding)
+        with torch.no_grad():
+            c_t.weight.copy_(gen.small_ints(11, 4, 3, 3, 3, lo=-3, hi=3))
+            c_t.bias.copy_(gen.small_ints(12, 4))
+        c_r = repdl_amd.from_torch_module(c_t)
+        x1 = gen.small_ints(13, 2, 3, 9, 8, lo=-3, hi=3).requires_grad_(True)
+        x2 = x1.detach().clone().requires_grad_(True)
+        y_t = c_t(x1)
+        go = gen.small_ints(14, *y_t.shape, lo=-3, hi=3)
+        y_t.backward(go)
+        y_r = c_r(x2)
+        y_r.backward(go)
+        assert torch.equal(y_r, y_t)
+        assert torch.equal(x2.grad, x1.grad)
+        assert torch.equal(c_r.weight.grad, c_t.weight.grad)
+        assert torch.equal(c_r.bias.grad, c_t.bias.grad)
+
+
+def test_conv2d_rejections():
+    with oracle_for_cpu_tensors():
+        F = repdl_amd.nn.functional
+        x, w = torch.zeros(1, 2, 5, 5), torch.zeros(2, 2, 3, 3)
+        with pytest.raises(NotImplementedError):
+            F.conv2d(x, w, padding="same")
+        with pytest.raises(NotImplementedError):
+            F.conv2d(x, w, dilation=2)
+        y = F.conv2d(x.requires_grad_(True), torch.zeros(2, 1, 3, 3).requires_grad_(True), groups=2)
+        with pytest.raises(NotImplementedError):
+            y.sum().backward()
+
+
+def test_cross_entropy_matches_torch():
+    with oracle_for_cpu_tensors():
+        x1 = (gen.normal_like(21, 12, 10) * 3).requires_grad_(True)
+        x2 = x1.detach().clone().requires_grad_(True)
+        t = gen.labels(22, 12, 10)
+        l_t = torch.nn.functional.cross_entropy(x1, t)
+        l_r = repdl_amd.nn.functional.cross_entropy(x2, t)
+        assert l_r.shape == l_t.shape and abs(float(l_r) - float(l_t)) < 1e-6
+        (l_t * 3).backward()
+        (l_r * 3).backward()
+        assert torch.allclose(x2.grad, x1.grad, atol=1e-6)
+        loss = repdl_amd.from_torch_module(torch.nn.CrossEntropyLoss())
+        assert float(loss(x2.detach(), t)) == float(l_r)
+        with pytest.raises(NotImplementedError):
+            repdl_amd.nn.functional.cross_entropy(x2, t, reduction="sum")
+
+
+def test_batchnorm_close_to_torch():
+    with oracle_for_cpu_tensors():
+        for bn_t, x in ((torch.nn.BatchNorm2d(5), gen.normal_like(31, 4, 5, 6, 7)),
+                        (torch.nn.BatchNorm1d(6), gen.normal_like(32, 9, 6))):
+            with torch.no_grad():
+                bn_t.weight.copy_(gen.normal_like(33, bn_t.num_features))
+                bn_t.bias.copy_(gen.normal_like(34, bn_t.num_features))
+            bn_r = repdl_amd.from_torch_module(bn_t)
+            x1, x2 = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+            y_t, y_r = bn_t(x1), bn_r(x2)
+            assert torch.allclose(y_r, y_t, atol=2e-5)
+            go = gen.normal_like(35, *x.shape)
+            y_t.backward(go)
+            y_r.backward(go)
+            assert torch.allclose(x2.grad, x1.grad, atol=2e-4)
+            assert torch.allclose(bn_r.weight.grad, bn_t.weight.grad, atol=2e-4)
+            assert torch.allclose(bn_r.bias.grad, bn_t.bias.grad, atol=2e-4)
+            # running mean follows PyTorch; the running variance uses the biased batch
+            # variance, as the reference's expression does (batchnorm.py:93)
+            assert torch.allclose(bn_r.running_mean, bn_t.running_mean, atol=1e-6)
+            bn_r.eval()
+            assert torch.isfinite(bn_r(x)).all()
+
+
+def test_func_means():
+    with oracle_for_cpu_tensors():
+        f = repdl_amd.func
+        v = gen.normal_like(41, 37).requires_grad_(True)
+        m = f.mean1d(v)
+        assert float(m) == float(repdl_amd.ops.sum1d(v.detach(), True))
+        m.backward()
+        assert torch.equal(v.grad, torch.full((37,), 1 / 37))
+        a = gen.normal_like(42, 6, 4).requires_grad_(True)
+        f.mean2d_dim0(a).sum().backward()
+        assert torch.equal(a.grad, torch.full((6, 4), 1 / 6))
+        b = gen.normal_like(43, 2, 3, 4, 5).requires_grad_(True)
+        f.mean4d_dim023(b).sum().backward()
+        assert torch.equal(b.grad, torch.full((2, 3, 4, 5), 1 / 40))
+        with pytest.raises(NotImplementedError):
+            f.expand_as(torch.zeros(3), torch.zeros(2, 4))
+
+
+def test_cnn_training_step_tracks_torch():
+    """End to end through from_torch_module: losses stay close to PyTorch's own
+    (not bit-equal: PyTorch sums in another order), and the run is deterministic."""
+    x, y = models.images(51, 16), gen.labels(52, 16, 10)
+    with oracle_for_cpu_tensors():
+        outs = []
+        for _ in range(2):
+            m = repdl_amd.from_torch_module(models.cnn(0))
+            logits, losses = models.train_steps(m, repdl_amd.nn.CrossEntropyLoss(), repdl_amd.optim.SGD(m.parameters(), 0.01), x, y, 3)
+            outs.append((repdl_amd.utils.get_hash(m), repdl_amd.utils.get_hash(logits), losses))
+        assert outs[0][:2] == outs[1][:2]
+    mt = models.cnn(0)
+    _, losses_t = models.train_steps(mt, torch.nn.CrossEntropyLoss(), torch.optim.SGD(mt.parameters(), 0.01), x, y, 3)
+    for a, b in zip(outs[0][2], losses_t):
+        assert abs(float(a) - float(b)) < 1e-4
+
+
+def test_adam_matches_formula():
+    with oracle_for_cpu_tensors():
+        p = torch.nn.Parameter(gen.normal_like(61, 50))
+        g = gen.normal_like(62, 50)
+        opt = repdl_amd.optim.Adam([p], lr=0.01)
+        p0 = p.detach().clone()
+        p.grad = g.clone()
+        opt.step()
+        m = g * np.float32(1 - 0.9)
+        v = (g * g) * np.float32(1 - 0.999)
+        denom = repdl_amd.ops.div(repdl_amd.ops.sqrt(v), (1 - 0.999) ** 0.5) + 1e-8
+        want = p0 + repdl_amd.ops.div(m, denom) * (-(0.01 / (1 - 0.9)))
+        assert torch.equal(p.detach(), want)
+        pt = torch.nn.Parameter(p0.clone())
+        pt.grad = g.clone()
+        torch.optim.Adam([pt], lr=0.01).step()
+        assert torch.allclose(p.detach(), pt.detach(), atol=1e-6)

@@ -1,0 +1,105 @@
+"""GPU parity through the Python glue: the same repdl_amd modules run once on CPU
+tensors (oracle behind repdl_amd.ops, a test-only monkeypatch) and once on GPU
+tensors (HIP backend); outputs, gradients and trained weights must hash equal."""
+import pytest
+import torch
+
+import gen
+import models
+import repdl_amd
+from oracle_ops import oracle_for_cpu_tensors
+
+pytestmark = pytest.mark.gpu
+
+
+def _both(build, run):
+    """run(module, device) on cpu (oracle) and cuda (hip); returns the two results."""
+    with oracle_for_cpu_tensors():
+        res = []
+        for dev in ("cpu", "cuda"):
+            m = build().to(dev)
+            res.append(run(m, dev))
+    return res
+
+
+def test_linear_forward_backward_bits():
+    def build():
+        torch.manual_seed(3)
+        return repdl_amd.from_torch_module(torch.nn.Linear(300, 130))
+
+    def run(m, dev):
+        x = gen.normal_like(1, 77, 300).to(dev).requires_grad_(True)
+        y = m(x)
+        y.backward(gen.normal_like(2, 77, 130).to(dev))
+        return [gen.sha256(t) for t in (y, x.grad, m.weight.grad, m.bias.grad)]
+
+    a, b = _both(build, run)
+    assert a == b
+
+
+@pytest.mark.parametrize("cfg", [(3, 8, 3, 1, 1), (8, 16, 3, 2, 1), (16, 8, 1, 1, 0), (4, 6, 5, 1, 2)])
+def test_conv2d_forward_backward_bits(cfg):
+    ic, oc, k, s, p = cfg
+
+    def build():
+        torch.manual_seed(4)
+        return repdl_amd.from_torch_module(torch.nn.Conv2d(ic, oc, k, stride=s, padding=p))
+
+    def run(m, dev):
+        x = gen.relu_like(5, 6, ic, 20, 17).to(dev).requires_grad_(True)
+        y = m(x)
+        y.backward(gen.normal_like(6, *y.shape).to(dev))
+        return [gen.sha256(t) for t in (y, x.grad, m.weight.grad, m.bias.grad)]
+
+    a, b = _both(build, run)
+    assert a == b
+
+
+def test_cross_entropy_and_softmax_bits():
+    def build():
+        return repdl_amd.nn.CrossEntropyLoss()
+
+    def run(m, dev):
+        x = (gen.normal_like(7, 64, 10) * 4).to(dev).requires_grad_(True)
+        t = gen.labels(8, 64, 10).to(dev)
+        loss = m(x, t)
+        loss.backward()
+        return [gen.sha256(loss), gen.sha256(x.grad)]
+
+    a, b = _both(build, run)
+    assert a == b
+
+
+def test_batchnorm_bits():
+    def build():
+        torch.manual_seed(9)
+        return repdl_amd.from_torch_module(torch.nn.Sequential(torch.nn.Conv2d(3, 8, 3, padding=1), torch.nn.BatchNorm2d(8)))
+
+    def run(m, dev):
+        x = gen.normal_like(10, 4, 3, 12, 12).to(dev).requires_grad_(True)
+        y = m(x)
+        y.backward(gen.normal_like(11, *y.shape).to(dev))
+        return [gen.sha256(t) for t in (y, x.grad, m[1].weight.grad, m[1].bias.grad, m[0].weight.grad)]
+
+    a, b = _both(build, run)
+    assert a == b
+
+
+@pytest.mark.parametrize("optim", ["sgd", "adam"])
+def test_cnn_training_bits(optim):
+    """BASELINE config 5, end to end: 2-conv + 2-FC CNN from from_torch_module, batch
+    64 of synthetic 1x28x28 images, 10 random classes, SGD lr 0.01 (explicit
+    two-rounding update) -- hashes of the final weights and logits, CPU vs GPU."""
+    x, y = models.images(21, 64), gen.labels(22, 64, 10)
+
+    def build():
+        return repdl_amd.from_torch_module(models.cnn(0))
+
+    def run(m, dev):
+        opt = repdl_amd.optim.SGD(m.parameters(), 0.01) if optim == "sgd" else repdl_amd.optim.Adam(m.parameters(), 0.01)
+        logits, losses = models.train_steps(m, repdl_amd.nn.CrossEntropyLoss(), opt, x.to(dev), y.to(dev), 3)
+        return [repdl_amd.utils.get_hash(m), repdl_amd.utils.get_hash(logits)] + [gen.sha256(l) for l in losses]
+
+    a, b = _both(build, run)
+    print(optim, "weights", b[0], "logits", b[1], flush=True)
+    assert a == b
