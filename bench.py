@@ -93,8 +93,11 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--quick", action="store_true", help="headline only, no secondary operators, no full parity")
-    ap.add_argument("--only", default="", help="comma list of secondary ops to run (sum2d,sum1d,exp,log,sqrt,div)")
+    ap.add_argument("--only", default="", help="comma list of secondary ops to run (sum2d,sum1d,exp,log,sqrt,div,conv)")
     ap.add_argument("--size", type=int, default=8192, help="mm size (M=N=K); the metric is quoted at 8192")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 1 GiB elementwise copy kernel (torch.add(x, 0)), the known-size kernel "
+                         "against which FETCH_SIZE / WRITE_SIZE counters are calibrated")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (every operator shards by outputs with no "
@@ -259,6 +262,46 @@ def main() -> int:
                            "cores": oracle.threads(), "kind": "port", "sample": "first 2^24 elements"}
                     result["also"].append(hbm_entry(name, wl, nbytes, f, args.steps, args.warmup, par, cpu))
                     hold.clear()
+
+        if want("conv"):
+            for (N, IC, H, W, OC, Kk, st, pd) in [(64, 64, 56, 56, 64, 3, 1, 1), (64, 256, 56, 56, 64, 1, 1, 0)]:
+                g = torch.Generator().manual_seed(5 + Kk)
+                x_h = torch.randn(N, IC, H, W, generator=g).clamp_(min=0)
+                w_h = torch.randn(OC, IC, Kk, Kk, generator=g) * (2.0 / (IC * Kk * Kk)) ** 0.5  # Kaiming normal
+                OH, OW = (H + 2 * pd - Kk) // st + 1, (W + 2 * pd - Kk) // st + 1
+                go_h = torch.randn(N, OC, OH, OW, generator=g)
+                x_d, w_d, go_d = x_h.to(dev), w_h.to(dev), go_h.to(dev)
+                flop = 2.0 * N * OC * OH * OW * IC * Kk * Kk
+                legs = [
+                    ("conv2d", lambda: ops.conv2d(x_d, w_d, (st, st), (pd, pd), 1),
+                     lambda: oracle.conv2d(x_h, w_h, st, st, pd, pd, 1)),
+                    ("conv2d_grad_input", lambda: ops.conv2d_grad_input(x_h.shape, w_d, go_d, (st, st), (pd, pd)),
+                     lambda: oracle.conv2d_grad_input(go_h, w_h, H, W, st, st, pd, pd)),
+                    ("conv2d_grad_kernel", lambda: ops.conv2d_grad_kernel(x_d, w_h.shape, go_d, (st, st), (pd, pd)),
+                     lambda: oracle.conv2d_grad_kernel(go_h, x_h, Kk, Kk, st, st, pd, pd)),
+                ]
+                for name, gfn, ofn in legs:
+                    hold = {}
+                    def f(): hold["y"] = gfn()
+                    wall, ev_mean, ev_min = time_gpu(f, args.steps, args.warmup)
+                    dt, y_cpu = cpu_time(ofn)
+                    tf = flop / (ev_mean * 1e-3) / 1e12
+                    result["also"].append({
+                        "op": name, "workload": "batch %d, %dx%d conv %d->%d at %dx%d" % (N, Kk, Kk, IC, OC, H, W),
+                        "value": round(tf * 1e3, 1), "unit": "GFLOP/s", "ms_per_step": round(ev_mean, 4),
+                        "roofline": {"bound": "mfma", "achieved": round(tf, 3), "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                     "frac": round(tf / FP32_PEAK_TFLOPS, 4), "traffic": None},
+                        "parity": {"equal": sha(hold["y"]) == sha(y_cpu), "sha256_gpu": sha(hold["y"])},
+                        "cpu_baseline": {"value": round(flop / dt / 1e9, 2), "unit": "GFLOP/s", "cores": oracle.threads(),
+                                         "kind": "port", "sample": "the full layer"}})
+                del x_d, w_d, go_d
+
+    if args.copy_probe:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 0.0, out=dst)  # an elementwise kernel: reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
 
     print(json.dumps(result))
     return 0

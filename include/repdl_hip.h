@@ -27,6 +27,7 @@
 #ifndef REPDL_HIP_H
 #define REPDL_HIP_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -79,6 +80,14 @@ int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float *input, f
  *   sum2d_dim1:   out[i]    = sum_j in[i][j],  in [M,N]         (count N)
  *   sum4d_dim023: out[c]    = sum_{n,h,w} in[n][c][h][w]        (count N*H*W) */
 int repdl_hip_sum1d(const float *in, float *out, int64_t n, int average, void *stream);
+/* sum1d with caller-provided scratch memory (same result).  Long inputs are evaluated in
+ * parallel -- exactly: the result is the sequential chain's, bit for bit -- which needs
+ * repdl_hip_sum1d_workspace_bytes(n) bytes of 16-byte aligned device memory (about n/2
+ * bytes; 0 for short inputs).  repdl_hip_sum1d itself takes that memory from the
+ * stream-ordered allocator (hipMallocAsync / hipFreeAsync on `stream`). */
+size_t repdl_hip_sum1d_workspace_bytes(int64_t n);
+int repdl_hip_sum1d_ws(const float *in, float *out, int64_t n, int average, void *workspace,
+                       size_t workspace_bytes, void *stream);
 int repdl_hip_sum2d_dim0(const float *in, float *out, int64_t M, int64_t N, int average,
                          void *stream);
 int repdl_hip_sum2d_dim1(const float *in, float *out, int64_t M, int64_t N, int average,

@@ -24,6 +24,7 @@ SIGNATURES = {
     "repdl_hip_conv2d_grad_input": [_P, _P, _P] + [_I64] * 13 + [_P],
     "repdl_hip_conv2d_grad_kernel": [_P, _P, _P] + [_I64] * 13 + [_P],
     "repdl_hip_sum1d": [_P, _P, _I64, _INT, _P],
+    "repdl_hip_sum1d_ws": [_P, _P, _I64, _INT, _P, ctypes.c_size_t, _P],
     "repdl_hip_sum2d_dim0": [_P, _P, _I64, _I64, _INT, _P],
     "repdl_hip_sum2d_dim1": [_P, _P, _I64, _I64, _INT, _P],
     "repdl_hip_sum4d_dim023": [_P, _P, _I64, _I64, _I64, _I64, _INT, _P],
@@ -58,6 +59,8 @@ def lib() -> ctypes.CDLL:
             fn.restype = _INT
         handle.repdl_hip_error_string.argtypes = [_INT]
         handle.repdl_hip_error_string.restype = ctypes.c_char_p
+        handle.repdl_hip_sum1d_workspace_bytes.argtypes = [_I64]
+        handle.repdl_hip_sum1d_workspace_bytes.restype = ctypes.c_size_t
         handle.repdl_hip_abi_version.argtypes = []
         handle.repdl_hip_abi_version.restype = _INT
         _lib = handle

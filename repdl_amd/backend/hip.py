@@ -108,8 +108,16 @@ def conv2d_grad_kernel(grad_output, input, KH, KW, strideH, strideW, paddingH, p
 def sum1d(input, average: bool = False) -> torch.Tensor:
     x = _check(input, "input", 1)
     out = torch.empty((), dtype=torch.float32, device=x.device)
+    n = x.shape[0]
+    nbytes = int(_lib.lib().repdl_hip_sum1d_workspace_bytes(n))
     with torch.cuda.device(x.device):
-        _lib.call("repdl_hip_sum1d", _ptr(x), _ptr(out), x.shape[0], int(bool(average)), _stream(x))
+        if nbytes:
+            # scratch for the parallel evaluation of the sequential chain, from PyTorch's allocator
+            work = torch.empty((nbytes,), dtype=torch.uint8, device=x.device)
+            _lib.call("repdl_hip_sum1d_ws", _ptr(x), _ptr(out), n, int(bool(average)), _ptr(work),
+                      ctypes.c_size_t(nbytes), _stream(x))
+        else:
+            _lib.call("repdl_hip_sum1d", _ptr(x), _ptr(out), n, int(bool(average)), _stream(x))
     return out
 
 

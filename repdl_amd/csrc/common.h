@@ -16,6 +16,9 @@
             return REPDL_E_ARG; \
     } while (0)
 
+// Inputs at least this long take the parallel evaluation of the sequential sum.
+#define REPDL_SUM1D_MIN_PARALLEL 32768
+
 // Largest extent a kernel indexes with 32-bit arithmetic.
 #define REPDL_I32_MAX 2147483647LL
 

@@ -21,6 +21,7 @@ namespace
 constexpr int BM = 128, BN = 128, BK = 16, NT = 256;
 constexpr int LDA = BM + 4; // padded row of the transposing store path
 constexpr int LDB = BN + 4;
+constexpr int GROUP_M = 8; // tile-rows walked together (see the tile order in the kernel)
 
 struct Frag
 {
@@ -131,7 +132,7 @@ template <bool TA, bool TB>
 __global__ __launch_bounds__(NT) void mm_kernel(const float *__restrict__ A,
                                                 const float *__restrict__ B, float *__restrict__ C,
                                                 int64_t M, int64_t N, int64_t K, int avec, int bvec,
-                                                int cvec)
+                                                int cvec, int64_t gx, int64_t gy, int64_t ntiles8)
 {
     constexpr bool A_KC = !TA; // A[m*K + k]
     constexpr bool B_KC = TB;  // B[n*K + k]
@@ -140,7 +141,20 @@ __global__ __launch_bounds__(NT) void mm_kernel(const float *__restrict__ A,
 
     const int tid = threadIdx.x;
     const int tx = tid & 15, ty = tid >> 4;
-    const int64_t m0 = (int64_t)blockIdx.y * BM, n0 = (int64_t)blockIdx.x * BN;
+    // Tile order.  Workgroups are handed to the 8 XCDs round-robin by linear id, and
+    // each XCD has its own L2: give every XCD one contiguous band of tile ids, and walk
+    // the tiles of a band in groups of GROUP_M tile-rows, column by column, so that the
+    // tiles resident on one XCD at a time share A row panels and B column panels.
+    int64_t tile = blockIdx.x;
+    if (tile < ntiles8)
+        tile = (tile & 7) * (ntiles8 >> 3) + (tile >> 3);
+    const int64_t group_sz = (int64_t)GROUP_M * gx;
+    const int64_t group = tile / group_sz;
+    const int64_t first_row = group * GROUP_M;
+    const int64_t rows_here = (gy - first_row < GROUP_M) ? gy - first_row : GROUP_M;
+    const int64_t in_group = tile - group * group_sz;
+    const int64_t trow = first_row + in_group % rows_here, tcol = in_group / rows_here;
+    const int64_t m0 = trow * BM, n0 = tcol * BN;
     const int64_t lda = TA ? M : K, ldb = TB ? K : N;
 
     float acc[8][8];
@@ -227,20 +241,21 @@ REPDL_API int repdl_hip_mm(const float *A, const float *B, float *C, int64_t M, 
     REPDL_REQUIRE(C != nullptr);
     REPDL_REQUIRE(K == 0 || (A != nullptr && B != nullptr));
     const int64_t gx = repdl_cdiv(N, BN), gy = repdl_cdiv(M, BM);
-    REPDL_REQUIRE(gx <= REPDL_I32_MAX && gy <= 65535);
+    REPDL_REQUIRE(gx * gy <= REPDL_I32_MAX);
+    const int64_t ntiles8 = (gx * gy) & ~(int64_t)7; // tiles covered by whole rounds over the 8 XCDs
     const int64_t lda = transA ? M : K, ldb = transB ? K : N;
     const int avec = aligned16(A) && (lda % 4 == 0);
     const int bvec = aligned16(B) && (ldb % 4 == 0);
     const int cvec = aligned16(C) && (N % 4 == 0);
-    dim3 grid((unsigned)gx, (unsigned)gy), block(NT);
+    dim3 grid((unsigned)(gx * gy)), block(NT);
     hipStream_t s = repdl_stream(stream);
     if (!transA && !transB)
-        hipLaunchKernelGGL((mm_kernel<false, false>), grid, block, 0, s, A, B, C, M, N, K, avec, bvec, cvec);
+        hipLaunchKernelGGL((mm_kernel<false, false>), grid, block, 0, s, A, B, C, M, N, K, avec, bvec, cvec, gx, gy, ntiles8);
     else if (transA && !transB)
-        hipLaunchKernelGGL((mm_kernel<true, false>), grid, block, 0, s, A, B, C, M, N, K, avec, bvec, cvec);
+        hipLaunchKernelGGL((mm_kernel<true, false>), grid, block, 0, s, A, B, C, M, N, K, avec, bvec, cvec, gx, gy, ntiles8);
     else if (!transA && transB)
-        hipLaunchKernelGGL((mm_kernel<false, true>), grid, block, 0, s, A, B, C, M, N, K, avec, bvec, cvec);
+        hipLaunchKernelGGL((mm_kernel<false, true>), grid, block, 0, s, A, B, C, M, N, K, avec, bvec, cvec, gx, gy, ntiles8);
     else
-        hipLaunchKernelGGL((mm_kernel<true, true>), grid, block, 0, s, A, B, C, M, N, K, avec, bvec, cvec);
+        hipLaunchKernelGGL((mm_kernel<true, true>), grid, block, 0, s, A, B, C, M, N, K, avec, bvec, cvec, gx, gy, ntiles8);
     return repdl_launch_status();
 }

@@ -200,7 +200,9 @@ static int launch_rowchain(const float *in, float *out, int64_t rows, int64_t ns
     return repdl_launch_status();
 }
 
-REPDL_API int repdl_hip_sum1d(const float *in, float *out, int64_t n, int average, void *stream)
+// The single serial chain (one lane walks): used for short inputs; long ones take the
+// parallel evaluation of sum1d.hip.
+int repdl_sum1d_serial(const float *in, float *out, int64_t n, int average, void *stream)
 {
     REPDL_REQUIRE(n >= 0 && out != nullptr && (n == 0 || in != nullptr));
     return launch_rowchain(in, out, 1, 1, n, n, 0, repdl_sum_factor(average, n), stream);

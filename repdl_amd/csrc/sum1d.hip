@@ -1,0 +1,520 @@
+// sum1d: the strictly sequential binary32 sum  s = +0; for i: s = RN(s + x[i])
+// (RepDL backend/cpu/summation.cpp:12-20), evaluated exactly but mostly in
+// parallel.
+//
+// Idea.  While the running sum stays inside one binade [2^E, 2^(E+1)) with one sign,
+// it is an integer S in [2^23, 2^24) times the quantum q = 2^(E-23), and adding x is
+//     S  ->  S + a[S & 1],   a[p] = X + [r > 1/2] + [r == 1/2] * ((p + X) & 1)
+// where sign*x/q = X + r, X integer, 0 <= r < 1 (round to nearest, ties to even: only
+// a tie looks at S, and only at its parity).  Such maps compose associatively:
+//     (a then b)[p] = a[p] + b[(p + a[p]) & 1]
+// so the map of a whole chunk is again one pair of integers, computable in any
+// grouping.  Carrying, per starting parity, the minimum of the exact sums before
+// rounding and the maximum of the rounded sums over all prefixes tells, once the real
+// incoming S is known, whether the sum really stayed inside the binade (the map is
+// valid) -- in O(1).
+//
+// Pipeline (n >= SUM1D_MIN_PARALLEL; shorter inputs take the serial kernel of sum.hip):
+//   1. block sums in binary64 over blocks of 4096 elements        (parallel, reads x once)
+//   2. exclusive prefix of the block sums                          (one workgroup)
+//   3. per chunk of 64 elements: the binade/sign HYPOTHESIS is read off the binary64
+//      prefix at the chunk start; tuple (a0,a1,lo0,hi0,lo1,hi1) of the chunk under that
+//      hypothesis; tuples of groups of 8 chunks and of the block (64 chunks) wherever
+//      the hypotheses agree                                        (parallel, reads x again)
+//   4. one wave walks the blocks in order with the true state: a block whose hypothesis
+//      matches the state and whose tuple is valid for it is applied in O(1); otherwise
+//      its 8 groups are tried, then the 8 chunks of a failing group, and a chunk that
+//      fails is replayed with 64 real binary32 additions.
+// The hypotheses come from an approximation, but they only decide how much is replayed:
+// every applied map is checked against the true state, so the result is the sequential
+// sum bit for bit for every input (NaN, infinities, zeros and subnormal states simply
+// fall through to the replay).
+#include "common.h"
+
+namespace
+{
+constexpr int CH = 64;            // elements per chunk
+constexpr int BLK = 4096;         // elements per block (64 chunks)
+constexpr int GROUPS = 8;         // groups of 8 chunks per block
+constexpr int HYP_NONE = -1;      // no usable hypothesis: replay
+constexpr int HYP_ANY = 0x200;    // every element is +-0: the identity for any state
+constexpr int BIG = 1 << 26;      // "leaves the binade for sure"
+constexpr int SAT = 1 << 28;      // saturation bound of all tuple fields
+
+struct __attribute__((aligned(16))) Tup
+{
+    int t0, t1;   // S -> S + t[p] for starting parity p
+    int lo0, hi0; // over all prefixes: min of (offset + X) before rounding, max of offset after
+    int lo1, hi1;
+    int hyp;      // (sign << 8) | biased exponent of the state this tuple assumes, or HYP_*
+    int pad;
+};
+
+__device__ __forceinline__ int clampi(int v) { return v < -SAT ? -SAT : (v > SAT ? SAT : v); }
+
+__device__ __forceinline__ Tup tup_identity(int hyp)
+{
+    Tup t;
+    t.t0 = t.t1 = t.lo0 = t.hi0 = t.lo1 = t.hi1 = 0;
+    t.hyp = hyp;
+    t.pad = 0;
+    return t;
+}
+
+// a then b (same hypothesis)
+__device__ __forceinline__ Tup tup_compose(const Tup &a, const Tup &b)
+{
+    Tup c;
+    const bool p0 = (a.t0 & 1) != 0;       // parity after a, starting even
+    const bool p1 = ((1 + a.t1) & 1) != 0; // parity after a, starting odd
+    const int bt0 = p0 ? b.t1 : b.t0, blo0 = p0 ? b.lo1 : b.lo0, bhi0 = p0 ? b.hi1 : b.hi0;
+    const int bt1 = p1 ? b.t1 : b.t0, blo1 = p1 ? b.lo1 : b.lo0, bhi1 = p1 ? b.hi1 : b.hi0;
+    c.t0 = clampi(a.t0 + bt0);
+    c.t1 = clampi(a.t1 + bt1);
+    c.lo0 = clampi(min(a.lo0, a.t0 + blo0));
+    c.hi0 = clampi(max(a.hi0, a.t0 + bhi0));
+    c.lo1 = clampi(min(a.lo1, a.t1 + blo1));
+    c.hi1 = clampi(max(a.hi1, a.t1 + bhi1));
+    c.hyp = a.hyp;
+    c.pad = 0;
+    return c;
+}
+
+// append element x (bit pattern ux, finite) to tuple t under hypothesis (sg, e)
+__device__ __forceinline__ void tup_append(Tup &t, uint32_t ux, int sg, int e)
+{
+    int ex = (int)((ux >> 23) & 0xFFu);
+    int m = (int)(ux & 0x7FFFFFu);
+    if (ex == 0)
+        ex = 1; // subnormal: same scale as the smallest normal, no implicit bit
+    else
+        m |= 0x800000;
+    if (m == 0)
+        return; // +-0 changes nothing
+    const bool neg = (int)(ux >> 31) != sg; // the element pulls the magnitude down
+    const int d = e - ex;
+    int X, a0, a1;
+    if (d < 0)
+    {
+        X = a0 = a1 = neg ? -BIG : BIG; // |x| >= 2^(E+1): out of the binade whatever S is
+    }
+    else if (d > 25)
+    {
+        X = neg ? -1 : 0; // |x| < q/4: rounds away, but a negative one dips below S first
+        a0 = a1 = 0;
+    }
+    else
+    {
+        const int v = neg ? -m : m;
+        X = v >> d; // floor
+        const int rem = v & ((1 << d) - 1);
+        const int half = d == 0 ? 0 : (1 << (d - 1));
+        const int gt = (d != 0 && rem > half) ? 1 : 0;
+        const int tie = (d != 0 && rem == half) ? 1 : 0;
+        a0 = X + gt + (tie & (X & 1));       // S even: S + X has the parity of X
+        a1 = X + gt + (tie & ((X + 1) & 1)); // S odd
+    }
+    // compose (t then this element)
+    const bool p0 = (t.t0 & 1) != 0, p1 = ((1 + t.t1) & 1) != 0;
+    const int ea0 = p0 ? a1 : a0, ea1 = p1 ? a1 : a0;
+    t.lo0 = clampi(min(t.lo0, t.t0 + X));
+    t.lo1 = clampi(min(t.lo1, t.t1 + X));
+    t.t0 = clampi(t.t0 + ea0);
+    t.t1 = clampi(t.t1 + ea1);
+    t.hi0 = max(t.hi0, t.t0);
+    t.hi1 = max(t.hi1, t.t1);
+}
+
+__device__ __forceinline__ Tup tup_shfl_down(const Tup &t, int delta)
+{
+    Tup r;
+    r.t0 = __shfl_down(t.t0, delta, 64);
+    r.t1 = __shfl_down(t.t1, delta, 64);
+    r.lo0 = __shfl_down(t.lo0, delta, 64);
+    r.hi0 = __shfl_down(t.hi0, delta, 64);
+    r.lo1 = __shfl_down(t.lo1, delta, 64);
+    r.hi1 = __shfl_down(t.hi1, delta, 64);
+    r.hyp = __shfl_down(t.hyp, delta, 64);
+    r.pad = 0;
+    return r;
+}
+
+// hypotheses merge: ANY is a wildcard, NONE (or a disagreement) poisons
+__device__ __forceinline__ int hyp_merge(int a, int b)
+{
+    if (a == HYP_ANY)
+        return b;
+    if (b == HYP_ANY)
+        return a;
+    return a == b ? a : HYP_NONE;
+}
+
+__device__ __forceinline__ Tup tup_join(const Tup &a, const Tup &b)
+{
+    const int h = hyp_merge(a.hyp, b.hyp);
+    Tup c = tup_compose(a, b);
+    c.hyp = h;
+    return c;
+}
+
+// ---- step 1: binary64 block sums -------------------------------------------------------
+__device__ __forceinline__ void load16(const float *__restrict__ x, int64_t n, int64_t i0, bool vec, float (&v)[16])
+{
+    if (vec && i0 + 15 < n)
+    {
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+        {
+            const float4 f = reinterpret_cast<const float4 *>(x + i0)[q];
+            v[4 * q + 0] = f.x;
+            v[4 * q + 1] = f.y;
+            v[4 * q + 2] = f.z;
+            v[4 * q + 3] = f.w;
+        }
+    }
+    else
+    {
+#pragma unroll
+        for (int q = 0; q < 16; q++)
+            v[q] = (i0 + q < n) ? x[i0 + q] : 0.0f;
+    }
+}
+
+__device__ __forceinline__ double wave_sum(double v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1)
+        v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+__global__ __launch_bounds__(256) void sum1d_blocksum_kernel(const float *__restrict__ x, int64_t n,
+                                                             double *__restrict__ bsum, int vec)
+{
+    __shared__ double part[4];
+    const int tid = threadIdx.x;
+    float v[16];
+    load16(x, n, (int64_t)blockIdx.x * BLK + tid * 16, vec, v);
+    double d = 0.0;
+#pragma unroll
+    for (int q = 0; q < 16; q++)
+        d += (double)v[q];
+    d = wave_sum(d);
+    if ((tid & 63) == 0)
+        part[tid >> 6] = d;
+    __syncthreads();
+    if (tid == 0)
+        bsum[blockIdx.x] = (part[0] + part[1]) + (part[2] + part[3]);
+}
+
+// ---- step 2: exclusive prefix of the block sums (one workgroup) ---------------------------
+__global__ __launch_bounds__(256) void sum1d_prefix_kernel(const double *__restrict__ bsum,
+                                                           double *__restrict__ prefix, int64_t nblk)
+{
+    __shared__ double seg[256];
+    const int tid = threadIdx.x;
+    const int64_t per = (nblk + 255) / 256;
+    const int64_t b0 = tid * per, b1 = (b0 + per < nblk) ? b0 + per : nblk;
+    double s = 0.0;
+    for (int64_t b = b0; b < b1; b++)
+        s += bsum[b];
+    seg[tid] = s;
+    __syncthreads();
+    if (tid == 0)
+    {
+        double run = 0.0;
+        for (int t = 0; t < 256; t++)
+        {
+            const double v = seg[t];
+            seg[t] = run;
+            run += v;
+        }
+    }
+    __syncthreads();
+    double run = seg[tid];
+    for (int64_t b = b0; b < b1; b++)
+    {
+        prefix[b] = run;
+        run += bsum[b];
+    }
+}
+
+// ---- step 3: chunk and block tuples --------------------------------------------------------
+__global__ __launch_bounds__(256) void sum1d_tuple_kernel(const float *__restrict__ x, int64_t n,
+                                                          const double *__restrict__ prefix,
+                                                          Tup *__restrict__ T1, Tup *__restrict__ TG,
+                                                          Tup *__restrict__ T2, int vec)
+{
+    __shared__ double wtot[4];
+    __shared__ Tup wt[4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t blk = blockIdx.x;
+    float v[16];
+    load16(x, n, blk * BLK + tid * 16, vec, v);
+
+    // binary64 exclusive prefix over the threads of the block
+    double d = 0.0;
+    bool finite = true, allzero = true;
+#pragma unroll
+    for (int q = 0; q < 16; q++)
+    {
+        d += (double)v[q];
+        const uint32_t a = __float_as_uint(v[q]) & 0x7FFFFFFFu;
+        finite = finite && a < 0x7F800000u;
+        allzero = allzero && a == 0u;
+    }
+    double inc = d;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1)
+    {
+        const double o = __shfl_up(inc, off, 64);
+        if (lane >= off)
+            inc += o;
+    }
+    if (lane == 63)
+        wtot[wave] = inc;
+    __syncthreads();
+    double base = prefix[blk];
+    for (int w = 0; w < wave; w++)
+        base += wtot[w];
+    const double excl = base + (inc - d);
+    // the chunk (4 consecutive lanes) takes its hypothesis from the prefix at its first lane
+    const double cstart = __shfl(excl, lane & ~3, 64);
+    const bool cfinite = ((__ballot(finite) >> (lane & ~3)) & 0xFull) == 0xFull;
+    const bool czero = ((__ballot(allzero) >> (lane & ~3)) & 0xFull) == 0xFull;
+    const uint32_t us = __float_as_uint((float)cstart);
+    const int eh = (int)((us >> 23) & 0xFFu);
+    int hyp = (eh >= 1 && eh <= 254) ? (int)(us >> 23) : HYP_NONE;
+    if (!cfinite)
+        hyp = HYP_NONE;
+    if (czero)
+        hyp = HYP_ANY;
+
+    Tup t = tup_identity(hyp);
+    if (hyp >= 0 && hyp != HYP_ANY)
+    {
+        const int sg = hyp >> 8, e = hyp & 0xFF;
+#pragma unroll
+        for (int q = 0; q < 16; q++)
+            tup_append(t, __float_as_uint(v[q]), sg, e);
+    }
+    // ordered reduction: 4 lanes -> chunk
+    t = tup_compose(t, tup_shfl_down(t, 1));
+    t = tup_compose(t, tup_shfl_down(t, 2));
+    if ((lane & 3) == 0)
+        T1[blk * (BLK / CH) + (tid >> 2)] = t;
+    // 8 chunks -> group, 2 groups -> wave, 4 waves -> block (hypotheses merged on the way)
+    t = tup_join(t, tup_shfl_down(t, 4));
+    t = tup_join(t, tup_shfl_down(t, 8));
+    t = tup_join(t, tup_shfl_down(t, 16));
+    if ((lane & 31) == 0)
+        TG[blk * GROUPS + wave * 2 + (lane >> 5)] = t;
+    t = tup_join(t, tup_shfl_down(t, 32));
+    if (lane == 0)
+        wt[wave] = t;
+    __syncthreads();
+    if (tid == 0)
+        T2[blk] = tup_join(tup_join(wt[0], wt[1]), tup_join(wt[2], wt[3]));
+}
+
+// ---- step 4: the walk -----------------------------------------------------------------------
+// The state s (a binary32 bit pattern) lives in scalar registers: it is identical in every
+// lane.  A tuple with hypothesis h applies to s iff (s >> 23) == h and need_lo <= S0 <= need_hi
+// for the parity of S0 = (s & 0x7FFFFF) | 0x800000; both tests together are one interval test
+// on s itself, smin[p] <= s <= smax[p] (unsigned), and applying the tuple is s += t[p] (the sum
+// stays inside the binade, so nothing carries into the exponent).  The tuples of up to 64
+// consecutive nodes sit one per lane in that form; stepping to node i broadcasts lane i's six
+// words with v_readlane_b32 (independent of s, so they run ahead of the dependency chain).
+struct LaneTup
+{
+    uint32_t smin0, smax0, smin1, smax1;
+    int t0, t1;
+};
+
+__device__ __forceinline__ LaneTup lane_tup(const Tup &t)
+{
+    LaneTup l;
+    l.t0 = t.t0;
+    l.t1 = t.t1;
+    if (t.hyp == HYP_ANY)
+    {
+        l.smin0 = l.smin1 = 0u;
+        l.smax0 = l.smax1 = 0xFFFFFFFFu;
+        l.t0 = l.t1 = 0;
+    }
+    else
+    {
+        const uint32_t top = (uint32_t)t.hyp << 23;
+        // S0 + lo >= 2^23  <=>  frac >= -lo ;  S0 + hi <= 2^24 - 1  <=>  frac <= 0x7FFFFF - hi
+        const int a0 = -t.lo0, b0 = 0x7FFFFF - t.hi0, a1 = -t.lo1, b1 = 0x7FFFFF - t.hi1;
+        const bool ok0 = t.hyp >= 0 && a0 <= 0x7FFFFF && b0 >= 0 && a0 <= b0;
+        const bool ok1 = t.hyp >= 0 && a1 <= 0x7FFFFF && b1 >= 0 && a1 <= b1;
+        l.smin0 = ok0 ? top + (uint32_t)a0 : 0xFFFFFFFFu; // empty interval: nothing applies
+        l.smax0 = ok0 ? top + (uint32_t)b0 : 0u;
+        l.smin1 = ok1 ? top + (uint32_t)a1 : 0xFFFFFFFFu;
+        l.smax1 = ok1 ? top + (uint32_t)b1 : 0u;
+    }
+    return l;
+}
+
+// Try node i (wave-uniform) of those held in l; false if it does not apply to state s.
+__device__ __forceinline__ bool lane_tup_apply(uint32_t &s, const LaneTup &l, int i)
+{
+    const uint32_t smin0 = __builtin_amdgcn_readlane(l.smin0, i), smax0 = __builtin_amdgcn_readlane(l.smax0, i);
+    const uint32_t smin1 = __builtin_amdgcn_readlane(l.smin1, i), smax1 = __builtin_amdgcn_readlane(l.smax1, i);
+    const int t0 = __builtin_amdgcn_readlane(l.t0, i), t1 = __builtin_amdgcn_readlane(l.t1, i);
+    const bool odd = (s & 1u) != 0u;
+    const uint32_t smin = odd ? smin1 : smin0, smax = odd ? smax1 : smax0;
+    const int tt = odd ? t1 : t0;
+    const bool ok = s >= smin && s <= smax;
+    s = ok ? s + (uint32_t)tt : s;
+    return ok;
+}
+
+__global__ __launch_bounds__(64) void sum1d_walk_kernel(const float *__restrict__ x, int64_t n,
+                                                        const Tup *__restrict__ T1,
+                                                        const Tup *__restrict__ TG,
+                                                        const Tup *__restrict__ T2, int64_t nblk, float factor,
+                                                        float *__restrict__ out, int vec)
+{
+    __shared__ __attribute__((aligned(16))) float xd[BLK];
+    const int lane = threadIdx.x;
+    uint32_t s = 0u; // +0.0f; wave-uniform throughout
+    Tup next = (lane < nblk) ? T2[lane] : tup_identity(HYP_ANY);
+    for (int64_t g0 = 0; g0 < nblk; g0 += 64)
+    {
+        const LaneTup lb = lane_tup(next);
+        if (g0 + 64 < nblk) // the next 64 block tuples, loaded while these are walked
+            next = (g0 + 64 + lane < nblk) ? T2[g0 + 64 + lane] : tup_identity(HYP_ANY);
+        const int cnt = (nblk - g0 < 64) ? (int)(nblk - g0) : 64;
+        for (int i = 0; i < cnt; i++)
+        {
+            if (lane_tup_apply(s, lb, i))
+                continue;
+            // The block as a whole does not apply: bring in its group and chunk tuples and its
+            // data (all loads issued before any is waited for).
+            const int64_t blk = g0 + i;
+            const Tup tgr = TG[blk * GROUPS + (lane & (GROUPS - 1))];
+            const Tup tch = T1[blk * (BLK / CH) + lane];
+            const int64_t e0 = blk * BLK;
+            float4 f[BLK / 256];
+            if (vec && e0 + BLK <= n)
+            {
+#pragma unroll
+                for (int q = 0; q < BLK / 256; q++)
+                    f[q] = reinterpret_cast<const float4 *>(x + e0)[q * 64 + lane];
+            }
+            else
+            {
+#pragma unroll
+                for (int q = 0; q < BLK / 256; q++)
+                {
+                    const int64_t idx = e0 + (int64_t)(q * 64 + lane) * 4;
+                    f[q].x = (idx + 0 < n) ? x[idx + 0] : 0.0f;
+                    f[q].y = (idx + 1 < n) ? x[idx + 1] : 0.0f;
+                    f[q].z = (idx + 2 < n) ? x[idx + 2] : 0.0f;
+                    f[q].w = (idx + 3 < n) ? x[idx + 3] : 0.0f;
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int q = 0; q < BLK / 256; q++)
+                *reinterpret_cast<float4 *>(&xd[(q * 64 + lane) * 4]) = f[q];
+            __syncthreads();
+            const LaneTup lg = lane_tup(tgr), lc = lane_tup(tch);
+            for (int gr = 0; gr < GROUPS; gr++)
+            {
+                if (lane_tup_apply(s, lg, gr))
+                    continue;
+                for (int j = gr * (BLK / CH / GROUPS); j < (gr + 1) * (BLK / CH / GROUPS); j++)
+                {
+                    if (lane_tup_apply(s, lc, j))
+                        continue;
+                    // replay: 64 real additions (elements past n were loaded as +0.0f: s + 0 = s)
+                    const float4 *p = reinterpret_cast<const float4 *>(&xd[j * CH]);
+                    float4 v[CH / 4];
+#pragma unroll
+                    for (int k = 0; k < CH / 4; k++)
+                        v[k] = p[k];
+                    float acc = __uint_as_float(s);
+#pragma unroll
+                    for (int k = 0; k < CH / 4; k++)
+                    {
+                        acc = acc + v[k].x;
+                        acc = acc + v[k].y;
+                        acc = acc + v[k].z;
+                        acc = acc + v[k].w;
+                    }
+                    s = __builtin_amdgcn_readfirstlane(__float_as_uint(acc));
+                }
+            }
+        }
+    }
+    if (lane == 0)
+        out[0] = factor * __uint_as_float(s);
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+inline size_t round256(size_t v) { return (v + 255) & ~(size_t)255; }
+} // namespace
+
+// serial single-chain kernel of sum.hip
+int repdl_sum1d_serial(const float *in, float *out, int64_t n, int average, void *stream);
+
+REPDL_API size_t repdl_hip_sum1d_workspace_bytes(int64_t n)
+{
+    if (n < REPDL_SUM1D_MIN_PARALLEL)
+        return 0;
+    const size_t nblk = (size_t)repdl_cdiv(n, BLK);
+    return round256(nblk * sizeof(double)) * 2 + round256(nblk * sizeof(Tup)) + round256(nblk * GROUPS * sizeof(Tup)) +
+           round256(nblk * (BLK / CH) * sizeof(Tup));
+}
+
+REPDL_API int repdl_hip_sum1d_ws(const float *in, float *out, int64_t n, int average, void *workspace,
+                                 size_t workspace_bytes, void *stream)
+{
+    REPDL_REQUIRE(n >= 0 && out != nullptr && (n == 0 || in != nullptr));
+    if (n < REPDL_SUM1D_MIN_PARALLEL)
+        return repdl_sum1d_serial(in, out, n, average, stream);
+    if (workspace == nullptr || workspace_bytes < repdl_hip_sum1d_workspace_bytes(n) ||
+        (reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
+        return REPDL_E_WORKSPACE;
+    const int64_t nblk = repdl_cdiv(n, BLK);
+    REPDL_REQUIRE(nblk <= REPDL_I32_MAX);
+    char *w = static_cast<char *>(workspace);
+    double *bsum = reinterpret_cast<double *>(w);
+    w += round256(nblk * sizeof(double));
+    double *prefix = reinterpret_cast<double *>(w);
+    w += round256(nblk * sizeof(double));
+    Tup *T2 = reinterpret_cast<Tup *>(w);
+    w += round256(nblk * sizeof(Tup));
+    Tup *TG = reinterpret_cast<Tup *>(w);
+    w += round256(nblk * GROUPS * sizeof(Tup));
+    Tup *T1 = reinterpret_cast<Tup *>(w);
+    hipStream_t s = repdl_stream(stream);
+    const int vec = aligned16(in);
+    hipLaunchKernelGGL(sum1d_blocksum_kernel, dim3((unsigned)nblk), dim3(256), 0, s, in, n, bsum, vec);
+    hipLaunchKernelGGL(sum1d_prefix_kernel, dim3(1), dim3(256), 0, s, bsum, prefix, nblk);
+    hipLaunchKernelGGL(sum1d_tuple_kernel, dim3((unsigned)nblk), dim3(256), 0, s, in, n, prefix, T1, TG, T2, vec);
+    hipLaunchKernelGGL(sum1d_walk_kernel, dim3(1), dim3(64), 0, s, in, n, T1, TG, T2, nblk,
+                       repdl_sum_factor(average, n), out, vec);
+    return repdl_launch_status();
+}
+
+REPDL_API int repdl_hip_sum1d(const float *in, float *out, int64_t n, int average, void *stream)
+{
+    REPDL_REQUIRE(n >= 0 && out != nullptr && (n == 0 || in != nullptr));
+    if (n < REPDL_SUM1D_MIN_PARALLEL)
+        return repdl_sum1d_serial(in, out, n, average, stream);
+    // no workspace given: take it from the stream-ordered allocator for the duration of the call
+    const size_t bytes = repdl_hip_sum1d_workspace_bytes(n);
+    void *ws = nullptr;
+    hipError_t e = hipMallocAsync(&ws, bytes, repdl_stream(stream));
+    if (e != hipSuccess)
+        return (int)e;
+    const int rc = repdl_hip_sum1d_ws(in, out, n, average, ws, bytes, stream);
+    e = hipFreeAsync(ws, repdl_stream(stream));
+    if (rc != REPDL_OK)
+        return rc;
+    return e == hipSuccess ? REPDL_OK : (int)e;
+}

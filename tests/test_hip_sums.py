@@ -1,0 +1,92 @@
+"""GPU parity of the sums against the oracle beyond the golden cases: the parallel
+evaluation of sum1d on data that crosses binades, changes sign, ties, hovers at binade
+edges, holds infinities / NaNs / zeros, on odd lengths and unaligned pointers; and the
+row / column / channel sums on shapes around the tile sizes."""
+import numpy as np
+import pytest
+import torch
+
+import gen
+from oracle import api as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _rng(seed):
+    return np.random.Generator(np.random.PCG64(seed))
+
+
+def _cases():
+    r = _rng(11)
+    n = 300_000
+    yield "uniform_pm1", gen.uniform_pm1(1, 1_000_003).numpy()
+    yield "scaled_normal", gen.scaled_normal(2, 777_777).numpy()
+    yield "positive_drift", (r.random(n) * 3).astype(np.float32)
+    yield "negative_drift", (-r.random(n) * 3).astype(np.float32)
+    yield "hover_edge", np.concatenate([[1024.0], np.where(r.random(n) < 0.5, 1.0, -1.0) + r.standard_normal(n) * 1e-3]).astype(np.float32)
+    yield "ties", np.concatenate([[2.0**24], np.ones(100_000), [-2.0**23], np.full(100_000, 0.5)]).astype(np.float32)
+    yield "tiny_after_big", np.concatenate([[1e8], r.random(n) * 1e-3, [-1e8], r.random(n)]).astype(np.float32)
+    yield "zeros", np.zeros(200_000, dtype=np.float32)
+    yield "zeros_then_values", np.concatenate([np.zeros(70_000), -np.zeros(5_000), r.standard_normal(100_000)]).astype(np.float32)
+    yield "inf_nan", np.concatenate([r.standard_normal(90_000), [np.inf], r.standard_normal(50_000), [-np.inf], r.standard_normal(50_000)]).astype(np.float32)
+    yield "subnormal_state", (r.integers(-2**20, 2**20, n).astype(np.float64) * 2.0**-149).astype(np.float32)
+    yield "cancel_to_zero", np.tile(np.array([3.25, -3.25, 1e-3, -1e-3], dtype=np.float32), 60_000)
+    yield "just_long_enough", gen.uniform_pm1(3, 32768).numpy()
+    yield "just_too_short", gen.uniform_pm1(4, 32767).numpy()
+
+
+@pytest.mark.parametrize("name,x", list(_cases()), ids=[n for n, _ in _cases()])
+def test_sum1d_parallel_path(name, x):
+    from repdl_amd import ops
+
+    t = torch.from_numpy(np.ascontiguousarray(x))
+    for avg in (False, True):
+        got = ops.sum1d(t.cuda(), avg).cpu()
+        want = oracle.sum1d(t, avg)
+        assert got.shape == want.shape
+        assert got.view(torch.int32).item() == want.view(torch.int32).item() or (torch.isnan(got) and torch.isnan(want)), (name, avg)
+
+
+def test_sum1d_unaligned_and_plain_entry():
+    """Unaligned input pointer, and the C entry point without a workspace (which takes
+    its scratch from the stream-ordered allocator)."""
+    import ctypes
+
+    from repdl_amd import _lib, ops
+
+    buf = gen.uniform_pm1(5, 400_001).cuda()
+    x = buf[1:]
+    assert x.data_ptr() % 16 != 0
+    want = oracle.sum1d(x.cpu())
+    assert torch.equal(ops.sum1d(x).cpu(), want)
+    out = torch.empty((), dtype=torch.float32, device="cuda")
+    _lib.call("repdl_hip_sum1d", ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(out.data_ptr()), x.numel(), 0,
+              ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu(), want)
+    small = ctypes.c_size_t(16)
+    rc = _lib.lib().repdl_hip_sum1d_ws(ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(out.data_ptr()), x.numel(), 0,
+                                       ctypes.c_void_p(buf.data_ptr()), small, None)
+    assert rc == -3  # workspace too small
+
+
+@pytest.mark.parametrize("shape", [(1, 5000), (3, 8193), (17, 511), (100, 100), (6200, 300), (13000, 65), (50000, 33)])
+def test_row_and_column_sums(shape):
+    from repdl_amd import ops
+
+    M, N = shape
+    x = gen.scaled_normal(M + N, M, N)
+    for avg in (False, True):
+        assert torch.equal(ops.sum2d_dim1(x.cuda(), False, avg).cpu(), oracle.sum2d_dim1(x, False, avg))
+        assert torch.equal(ops.sum2d_dim0(x.cuda(), True, avg).cpu(), oracle.sum2d_dim0(x, True, avg))
+    xu = gen.scaled_normal(7, M * N + 1).cuda()[1:].view(M, N)  # unaligned rows
+    assert torch.equal(ops.sum2d_dim1(xu).cpu(), oracle.sum2d_dim1(xu.cpu()))
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 5, 7), (4, 64, 14, 14), (3, 130, 8, 8), (1, 7000, 3, 3)])
+def test_channel_sums(shape):
+    from repdl_amd import ops
+
+    x = gen.scaled_normal(sum(shape), *shape)
+    assert torch.equal(ops.sum4d_dim023(x.cuda()).cpu(), oracle.sum4d_dim023(x))
+    assert torch.equal(ops.sum(x.cuda(), dim=(0, 2, 3), keepdim=True, average=True).cpu(), oracle.sum4d_dim023(x, True, True))
