@@ -4,8 +4,8 @@
 // routine followed by one rounding to binary32) and repdl/ops.py:98-103, 122-123
 // (div, sqrt: the IEEE binary32 results).  The arithmetic lives in crmath.h and
 // uses no approximate-function instruction and no '/' operator; this file only
-// streams the data: 16-byte non-temporal loads and stores, one contiguous
-// chunk per workgroup, several loads in flight per lane; the exp/log tables (2 KiB / 4 KiB) are copied to LDS once per
+// streams the data: 16-byte non-temporal loads and stores, one small contiguous
+// chunk per workgroup, four loads in flight per lane; the exp/log tables (2 KiB / 4 KiB) are copied to LDS once per
 // workgroup.  All four are HBM-bound: 8 bytes per element (12 for tensor/tensor
 // division).
 #include "common.h"
@@ -17,14 +17,14 @@ __device__ const uint64_t g_exp_tab[256] = CRM_EXP_TAB_INIT;
 __device__ const double g_log_tab[512] = CRM_LOG_TAB_INIT;
 
 constexpr int EW_THREADS = 256;
-constexpr int EW_UNROLL = 4;                                // 16-byte accesses in flight per lane
-constexpr int EW_ITERS = 4;                                 // iterations per workgroup
-constexpr int EW_CHUNK = EW_THREADS * EW_UNROLL * EW_ITERS; // float4 per workgroup (64 KiB in, 64 KiB out)
+constexpr int EW_UNROLL = 4;                     // 16-byte accesses in flight per lane
+constexpr int EW_CHUNK = EW_THREADS * EW_UNROLL; // float4 per workgroup (16 KiB in, 16 KiB out)
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 // Streaming accesses: every byte is touched once, so loads and stores carry the
-// non-temporal hint and each workgroup owns one contiguous chunk.
+// non-temporal hint and each workgroup owns one small contiguous chunk (many small
+// workgroups keep more independent loads in flight than few long-running ones).
 __device__ __forceinline__ v4f ld_stream(const v4f *p) { return __builtin_nontemporal_load(p); }
 __device__ __forceinline__ void st_stream(v4f v, v4f *p) { __builtin_nontemporal_store(v, p); }
 
@@ -72,6 +72,24 @@ __global__ __launch_bounds__(EW_THREADS) void unary_kernel(const float *__restri
     Ctx<OP> ctx;
     ctx.exp_tab = tab;
     ctx.log_tab = reinterpret_cast<const double *>(tab);
+    if (OP == OP_DIV_SCALAR)
+        ctx.divisor = crm_divisor_make(scalar);
+
+    const int64_t n4 = n >> 2;
+    const int64_t b0 = (int64_t)blockIdx.x * EW_CHUNK;
+    const bool full = vec_ok && b0 + EW_CHUNK <= n4;
+    const v4f *in4 = reinterpret_cast<const v4f *>(in);
+    v4f *out4 = reinterpret_cast<v4f *>(out);
+
+    // the streaming loads go out first, then the table fill, so that both are in flight
+    // together
+    v4f v[EW_UNROLL];
+    if (full)
+    {
+#pragma unroll
+        for (int u = 0; u < EW_UNROLL; u++)
+            v[u] = ld_stream(&in4[b0 + threadIdx.x + u * EW_THREADS]);
+    }
     if (OP == OP_EXP)
     {
         for (int i = threadIdx.x; i < 256; i += EW_THREADS)
@@ -84,40 +102,18 @@ __global__ __launch_bounds__(EW_THREADS) void unary_kernel(const float *__restri
             tab[i] = crm_d2u(g_log_tab[i]);
         __syncthreads();
     }
-    if (OP == OP_DIV_SCALAR)
-        ctx.divisor = crm_divisor_make(scalar);
-
-    if (vec_ok)
+    if (full)
     {
-        const int64_t n4 = n >> 2;
-        const v4f *in4 = reinterpret_cast<const v4f *>(in);
-        v4f *out4 = reinterpret_cast<v4f *>(out);
-        const int64_t b0 = (int64_t)blockIdx.x * EW_CHUNK;
-        const int64_t b1 = b0 + EW_CHUNK < n4 ? b0 + EW_CHUNK : n4;
-        int64_t i = b0 + threadIdx.x;
-        for (; i + (EW_UNROLL - 1) * EW_THREADS < b1; i += EW_UNROLL * EW_THREADS)
-        {
-            v4f v[EW_UNROLL];
 #pragma unroll
-            for (int u = 0; u < EW_UNROLL; u++)
-                v[u] = ld_stream(&in4[i + u * EW_THREADS]);
-#pragma unroll
-            for (int u = 0; u < EW_UNROLL; u++)
-                st_stream(ctx.apply4(v[u]), &out4[i + u * EW_THREADS]);
-        }
-        for (; i < b1; i += EW_THREADS)
-            st_stream(ctx.apply4(ld_stream(&in4[i])), &out4[i]);
-        // the last (n mod 4) elements
-        if (blockIdx.x == 0 && threadIdx.x < (n & 3))
-            out[(n4 << 2) + threadIdx.x] = ctx.apply(in[(n4 << 2) + threadIdx.x]);
+        for (int u = 0; u < EW_UNROLL; u++)
+            st_stream(ctx.apply4(v[u]), &out4[b0 + threadIdx.x + u * EW_THREADS]);
+        return;
     }
-    else
-    {
-        const int64_t b0 = (int64_t)blockIdx.x * EW_CHUNK * 4;
-        const int64_t b1 = b0 + EW_CHUNK * 4 < n ? b0 + EW_CHUNK * 4 : n;
-        for (int64_t i = b0 + threadIdx.x; i < b1; i += EW_THREADS)
-            out[i] = ctx.apply(in[i]);
-    }
+    // partial last chunk, the (n mod 4) tail, or unaligned pointers: element by element
+    const int64_t e0 = b0 * 4;
+    const int64_t e1 = e0 + EW_CHUNK * 4 < n ? e0 + EW_CHUNK * 4 : n;
+    for (int64_t i = e0 + threadIdx.x; i < e1; i += EW_THREADS)
+        out[i] = ctx.apply(in[i]);
 }
 
 __device__ __forceinline__ v4f div4(v4f a, v4f b)
@@ -130,57 +126,40 @@ __device__ __forceinline__ v4f div4(v4f a, v4f b)
     return r;
 }
 
-constexpr int DIV_UNROLL = 2;
-
 __global__ __launch_bounds__(EW_THREADS) void div_kernel(const float *__restrict__ a,
                                                          const float *__restrict__ b,
                                                          float *__restrict__ out, int64_t n,
                                                          int vec_ok)
 {
-    if (vec_ok)
+    const int64_t n4 = n >> 2;
+    const int64_t b0 = (int64_t)blockIdx.x * EW_CHUNK;
+    if (vec_ok && b0 + EW_CHUNK <= n4)
     {
-        const int64_t n4 = n >> 2;
         const v4f *a4 = reinterpret_cast<const v4f *>(a);
         const v4f *b4 = reinterpret_cast<const v4f *>(b);
         v4f *out4 = reinterpret_cast<v4f *>(out);
-        const int64_t b0 = (int64_t)blockIdx.x * EW_CHUNK;
-        const int64_t b1 = b0 + EW_CHUNK < n4 ? b0 + EW_CHUNK : n4;
-        int64_t i = b0 + threadIdx.x;
-        for (; i + (DIV_UNROLL - 1) * EW_THREADS < b1; i += DIV_UNROLL * EW_THREADS)
+        v4f x[EW_UNROLL], y[EW_UNROLL];
+#pragma unroll
+        for (int u = 0; u < EW_UNROLL; u++)
         {
-            v4f x[DIV_UNROLL], y[DIV_UNROLL];
-#pragma unroll
-            for (int u = 0; u < DIV_UNROLL; u++)
-            {
-                x[u] = ld_stream(&a4[i + u * EW_THREADS]);
-                y[u] = ld_stream(&b4[i + u * EW_THREADS]);
-            }
-#pragma unroll
-            for (int u = 0; u < DIV_UNROLL; u++)
-                st_stream(div4(x[u], y[u]), &out4[i + u * EW_THREADS]);
+            x[u] = ld_stream(&a4[b0 + threadIdx.x + u * EW_THREADS]);
+            y[u] = ld_stream(&b4[b0 + threadIdx.x + u * EW_THREADS]);
         }
-        for (; i < b1; i += EW_THREADS)
-            st_stream(div4(ld_stream(&a4[i]), ld_stream(&b4[i])), &out4[i]);
-        if (blockIdx.x == 0 && threadIdx.x < (n & 3))
-            out[(n4 << 2) + threadIdx.x] = crm_div(a[(n4 << 2) + threadIdx.x], b[(n4 << 2) + threadIdx.x]);
+#pragma unroll
+        for (int u = 0; u < EW_UNROLL; u++)
+            st_stream(div4(x[u], y[u]), &out4[b0 + threadIdx.x + u * EW_THREADS]);
+        return;
     }
-    else
-    {
-        const int64_t b0 = (int64_t)blockIdx.x * EW_CHUNK * 4;
-        const int64_t b1 = b0 + EW_CHUNK * 4 < n ? b0 + EW_CHUNK * 4 : n;
-        for (int64_t i = b0 + threadIdx.x; i < b1; i += EW_THREADS)
-            out[i] = crm_div(a[i], b[i]);
-    }
+    const int64_t e0 = b0 * 4;
+    const int64_t e1 = e0 + EW_CHUNK * 4 < n ? e0 + EW_CHUNK * 4 : n;
+    for (int64_t i = e0 + threadIdx.x; i < e1; i += EW_THREADS)
+        out[i] = crm_div(a[i], b[i]);
 }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-// one workgroup per EW_CHUNK float4 (at least one, so the n < 4 tail is served)
-inline int64_t ew_grid(int64_t n)
-{
-    int64_t g = repdl_cdiv(repdl_cdiv(n, 4), EW_CHUNK);
-    return g < 1 ? 1 : g;
-}
+// one workgroup per EW_CHUNK float4 (4 * EW_CHUNK elements)
+inline int64_t ew_grid(int64_t n) { return repdl_cdiv(n, 4 * (int64_t)EW_CHUNK); }
 
 template <int OP>
 int launch_unary(const float *in, float *out, int64_t n, float scalar, void *stream)
