@@ -124,6 +124,13 @@ CRM_FN float crm_div(float a, float b)
 // Division of many dividends by one divisor: the reciprocal is computed once.
 typedef struct
 {
+    const float *invc;
+    const double *logc_hi;
+    const float *logc_lo;
+} crm_log_tables;
+
+typedef struct
+{
     double db, y;
     uint32_t ub;
 } crm_divisor;
@@ -167,18 +174,14 @@ CRM_FN float crm_sqrt(float x)
     double s = dx * y;
     const double r = crm_fma(-s, s, dx);
     s = crm_fma(r, 0.5 * y, s);
-    uint32_t res = crm_f2u(crm_d2f(s));
-    // +-0, +inf, negatives, -inf and NaNs: (ux - 1) wraps 0 to the top
-    if (ux - 1u >= 0x7F7FFFFFu)
-    {
-        const uint32_t ax = ux & 0x7FFFFFFFu;
-        res = CRM_QNAN_POS; // negative, -inf (PyTorch CPU convention)
-        if (ax == 0u || ux == 0x7F800000u)
-            res = ux; // +-0, +inf
-        if (ax > 0x7F800000u)
-            res = ux | 0x00400000u; // NaN: sign and payload kept, quieted
-    }
-    return crm_u2f(res);
+    const uint32_t gen = crm_f2u(crm_d2f(s));
+    // +-0, +inf, negatives, -inf and NaNs ((ux - 1) wraps 0 to the top); written as
+    // selects, not branches, so that consecutive elements interleave
+    const uint32_t ax = ux & 0x7FFFFFFFu;
+    uint32_t sp = CRM_QNAN_POS;                          // negative, -inf (PyTorch CPU convention)
+    sp = (ax == 0u || ux == 0x7F800000u) ? ux : sp;      // +-0, +inf
+    sp = (ax > 0x7F800000u) ? (ux | 0x00400000u) : sp;   // NaN: sign and payload kept, quieted
+    return crm_u2f((ux - 1u >= 0x7F7FFFFFu) ? sp : gen);
 }
 
 // ---- exp --------------------------------------------------------------------
@@ -222,22 +225,18 @@ CRM_FN float crm_exp(float x, const uint64_t *tab)
     // |x| > 104 (also inf, NaN): the binary32 result is 0 or +inf whatever the
     // binary64 value is (exp(-104) < 2^-150, exp(89) > 2^128).  Such arguments
     // still run through the core harmlessly: the table index is masked.
-    uint32_t res = crm_f2u(crm_d2f(crm_exp64_core((double)x, tab)));
-    if (ax > 0x42D00000u)
-    {
-        res = (ux >> 31) ? 0u : 0x7F800000u;
-        if (ax > 0x7F800000u)
-            res = ux | 0x00400000u; // NaN + 1.0: sign and payload kept, quieted
-    }
-    return crm_u2f(res);
+    const uint32_t gen = crm_f2u(crm_d2f(crm_exp64_core((double)x, tab)));
+    uint32_t sp = (ux >> 31) ? 0u : 0x7F800000u;
+    sp = (ax > 0x7F800000u) ? (ux | 0x00400000u) : sp; // NaN + 1.0: sign and payload kept, quieted
+    return crm_u2f((ax > 0x42D00000u) ? sp : gen);
 }
 
 // ---- log --------------------------------------------------------------------
 // x = 2^k z, z in [0.6875, 1.375); r = z*invc - 1 (exact for 24-bit z);
 // log(x) = k ln2 + logc + log1p(r), summed as an exact head
 // w = k*LN2_HI + logc_hi, a compensated hi + lo, and a degree-9 polynomial.
-// tab: CRM_LOG_TAB_INIT, four doubles per entry (invc, logc_hi, logc_lo, 0).
-CRM_FN double crm_log64_core(double x, const double *tab)
+// Tables (crmath_tables.h): invc[128] binary32, logc_hi[128] binary64, logc_lo[128] binary32.
+CRM_FN double crm_log64_core(double x, crm_log_tables tab)
 {
     const uint64_t ix = crm_d2u(x);
     // only the high word takes part in the reduction (the offset has a zero low word)
@@ -247,7 +246,7 @@ CRM_FN double crm_log64_core(double x, const double *tab)
     const int32_t k = (int32_t)tmp >> 20;
     const uint32_t zhi = hi - (tmp & 0xFFF00000u);
     const double z = crm_u2d(((uint64_t)zhi << 32) | (ix & 0xFFFFFFFFu));
-    const double invc = tab[4 * i], logc_hi = tab[4 * i + 1], logc_lo = tab[4 * i + 2];
+    const double invc = (double)tab.invc[i], logc_hi = tab.logc_hi[i], logc_lo = (double)tab.logc_lo[i];
     const double kd = (double)k;
     const double r = crm_fma(z, invc, -1.0);
     const double w = crm_fma(kd, CRM_LN2_HI, logc_hi); // exact
@@ -265,22 +264,16 @@ CRM_FN double crm_log64_core(double x, const double *tab)
     return hi_sum + crm_fma(r2, p, lo);
 }
 
-CRM_FN float crm_log(float x, const double *tab)
+CRM_FN float crm_log(float x, crm_log_tables tab)
 {
     const uint32_t ux = crm_f2u(x);
     // zeros, negatives, infinities and NaNs run through the core harmlessly (the
     // table index is masked) and are overridden
-    uint32_t res = crm_f2u(crm_d2f(crm_log64_core((double)x, tab)));
-    if (ux - 1u >= 0x7F7FFFFFu)
-    {
-        const uint32_t ax = ux & 0x7FFFFFFFu;
-        res = CRM_QNAN_NEG; // log(negative), log(-inf): (x-x)/(x-x) on x86
-        if (ux == 0x7F800000u)
-            res = 0x7F800000u; // log(+inf)
-        if (ax == 0u)
-            res = 0xFF800000u; // log(+-0) = -inf
-        if (ax > 0x7F800000u)
-            res = ux | 0x00400000u; // NaN: sign and payload kept, quieted
-    }
-    return crm_u2f(res);
+    const uint32_t gen = crm_f2u(crm_d2f(crm_log64_core((double)x, tab)));
+    const uint32_t ax = ux & 0x7FFFFFFFu;
+    uint32_t sp = CRM_QNAN_NEG;                        // log(negative), log(-inf): (x-x)/(x-x) on x86
+    sp = (ux == 0x7F800000u) ? 0x7F800000u : sp;       // log(+inf)
+    sp = (ax == 0u) ? 0xFF800000u : sp;                // log(+-0) = -inf
+    sp = (ax > 0x7F800000u) ? (ux | 0x00400000u) : sp; // NaN: sign and payload kept, quieted
+    return crm_u2f((ux - 1u >= 0x7F7FFFFFu) ? sp : gen);
 }

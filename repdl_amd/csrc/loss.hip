@@ -13,7 +13,9 @@
 namespace
 {
 __device__ const uint64_t g_exp_tab2[256] = CRM_EXP_TAB_INIT;
-__device__ const double g_log_tab2[512] = CRM_LOG_TAB_INIT;
+__device__ const float g_log_invc2[128] = CRM_LOG_INVC_INIT;
+__device__ const double g_log_hi2[128] = CRM_LOG_HI_INIT;
+__device__ const float g_log_lo2[128] = CRM_LOG_LO_INIT;
 
 constexpr int CH = 256; // columns staged per pass
 
@@ -99,13 +101,18 @@ __global__ __launch_bounds__(64) void cross_entropy_rows_kernel(const float *__r
                                                                 int64_t N)
 {
     __shared__ uint64_t exp_tab[256];
-    __shared__ uint64_t log_tab[512];
+    __shared__ double log_hi[128];
+    __shared__ float log_invc[128], log_lo[128];
     __shared__ float stage[CH];
     const int lane = threadIdx.x;
     for (int i = lane; i < 256; i += 64)
         exp_tab[i] = g_exp_tab2[i];
-    for (int i = lane; i < 512; i += 64)
-        log_tab[i] = crm_d2u(g_log_tab2[i]);
+    for (int i = lane; i < 128; i += 64)
+    {
+        log_hi[i] = g_log_hi2[i];
+        log_invc[i] = g_log_invc2[i];
+        log_lo[i] = g_log_lo2[i];
+    }
     __syncthreads();
     const int64_t row = blockIdx.x;
     const float *x = in + row * N;
@@ -113,7 +120,11 @@ __global__ __launch_bounds__(64) void cross_entropy_rows_kernel(const float *__r
     const float sum = row_exp_sum(x, nullptr, N, m, lane, stage, exp_tab);
     if (lane == 0)
     {
-        float l = crm_log(sum, reinterpret_cast<const double *>(log_tab));
+        crm_log_tables lt;
+        lt.invc = log_invc;
+        lt.logc_hi = log_hi;
+        lt.logc_lo = log_lo;
+        float l = crm_log(sum, lt);
         int64_t t = target[row];
         float shifted = (t >= 0 && t < N) ? x[t] - m : __builtin_nanf("");
         loss[row] = l - shifted;

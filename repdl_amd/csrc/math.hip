@@ -5,7 +5,7 @@
 // (div, sqrt: the IEEE binary32 results).  The arithmetic lives in crmath.h and
 // uses no approximate-function instruction and no '/' operator; this file only
 // streams the data: 16-byte non-temporal loads and stores, one small contiguous
-// chunk per workgroup, four loads in flight per lane; the exp/log tables (2 KiB / 4 KiB) are copied to LDS once per
+// chunk per workgroup, four loads in flight per lane; the exp/log tables (2 KiB each) are copied to LDS once per
 // workgroup.  All four are HBM-bound: 8 bytes per element (12 for tensor/tensor
 // division).
 #include "common.h"
@@ -14,7 +14,9 @@
 namespace
 {
 __device__ const uint64_t g_exp_tab[256] = CRM_EXP_TAB_INIT;
-__device__ const double g_log_tab[512] = CRM_LOG_TAB_INIT;
+__device__ const float g_log_invc[128] = CRM_LOG_INVC_INIT;
+__device__ const double g_log_hi[128] = CRM_LOG_HI_INIT;
+__device__ const float g_log_lo[128] = CRM_LOG_LO_INIT;
 
 constexpr int EW_THREADS = 256;
 constexpr int EW_UNROLL = 4;                     // 16-byte accesses in flight per lane
@@ -40,7 +42,7 @@ template <int OP>
 struct Ctx
 {
     const uint64_t *exp_tab;
-    const double *log_tab;
+    crm_log_tables log_tab;
     crm_divisor divisor;
     __device__ __forceinline__ float apply(float x) const
     {
@@ -68,10 +70,15 @@ __global__ __launch_bounds__(EW_THREADS) void unary_kernel(const float *__restri
                                                            float *__restrict__ out, int64_t n,
                                                            float scalar, int vec_ok)
 {
-    __shared__ __attribute__((aligned(16))) uint64_t tab[OP == OP_LOG ? 512 : 256];
+    // exp: 256 words (tail, sbits pairs); log: logc_hi[128] then invc[128], logc_lo[128] as floats
+    __shared__ __attribute__((aligned(16))) uint64_t tab[256];
     Ctx<OP> ctx;
     ctx.exp_tab = tab;
-    ctx.log_tab = reinterpret_cast<const double *>(tab);
+    double *lhi = reinterpret_cast<double *>(tab);
+    float *linvc = reinterpret_cast<float *>(tab + 128), *llo = linvc + 128;
+    ctx.log_tab.invc = linvc;
+    ctx.log_tab.logc_hi = lhi;
+    ctx.log_tab.logc_lo = llo;
     if (OP == OP_DIV_SCALAR)
         ctx.divisor = crm_divisor_make(scalar);
 
@@ -98,8 +105,12 @@ __global__ __launch_bounds__(EW_THREADS) void unary_kernel(const float *__restri
     }
     if (OP == OP_LOG)
     {
-        for (int i = threadIdx.x; i < 512; i += EW_THREADS)
-            tab[i] = crm_d2u(g_log_tab[i]);
+        if (threadIdx.x < 128)
+        {
+            lhi[threadIdx.x] = g_log_hi[threadIdx.x];
+            linvc[threadIdx.x] = g_log_invc[threadIdx.x];
+            llo[threadIdx.x] = g_log_lo[threadIdx.x];
+        }
         __syncthreads();
     }
     if (full)

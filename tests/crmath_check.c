@@ -14,7 +14,10 @@
 #include "../repdl_amd/csrc/crmath.h"
 
 static const uint64_t EXP_TAB[256] = CRM_EXP_TAB_INIT;
-static const double LOG_TAB[512] = CRM_LOG_TAB_INIT;
+static const float LOG_INVC[128] = CRM_LOG_INVC_INIT;
+static const double LOG_HI[128] = CRM_LOG_HI_INIT;
+static const float LOG_LO[128] = CRM_LOG_LO_INIT;
+static const crm_log_tables LOG_TAB = {LOG_INVC, LOG_HI, LOG_LO};
 
 #define API __attribute__((visibility("default")))
 
