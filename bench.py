@@ -31,6 +31,16 @@ sys.path.insert(0, ROOT)
 FP32_PEAK_TFLOPS = 157.3  # MI355X vendor fp32 figure (256 CU x 2.4 GHz x 256 flop/clk)
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch from two `rocprofv3 --pmc` runs (FETCH_SIZE, then WRITE_SIZE), each scaled by
+# what the same counter reads for a plain 1 GiB elementwise copy kernel (--copy-probe): FETCH_SIZE
+# reads 524300 for 1 GiB (factor 1.99995 KiB per count), WRITE_SIZE 1048576 (factor 1.0).  Summary:
+# profiles/hbm_traffic_counters.txt.  Valid for the default workload sizes only.
+MEASURED_TRAFFIC_BYTES = {
+    "mm": 3441648 * 1.99995 * 1024 + 262171 * 1024,       # 7.3e9: operand panels re-read through L2 misses
+    "exp": 524338 * 1.99995 * 1024 + 1048577 * 1024,      # 2.147e9 = the algorithmic 8 B/element
+    "sum2d_dim1": 524392 * 1.99995 * 1024 + 64 * 1024,    # 1.074e9 = the algorithmic 4 B/element
+}
+
 
 def sha(t) -> str:
     return hashlib.sha256(t.detach().cpu().contiguous().numpy().tobytes()).hexdigest()
@@ -57,7 +67,7 @@ def time_gpu(fn, steps: int, warmup: int):
     return wall, sum(ev) / len(ev), min(ev)
 
 
-def hbm_entry(name, workload, algo_bytes, fn, steps, warmup, parity=None, cpu=None):
+def hbm_entry(name, workload, algo_bytes, fn, steps, warmup, parity=None, cpu=None, traffic=None):
     wall, ev_mean, ev_min = time_gpu(fn, steps, warmup)
     gbs = algo_bytes / (ev_mean * 1e-3) / 1e9
     out = {
@@ -68,7 +78,7 @@ def hbm_entry(name, workload, algo_bytes, fn, steps, warmup, parity=None, cpu=No
         "ms_per_step": round(ev_mean, 4),
         "ms_min": round(ev_min, 4),
         "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic},
     }
     if parity is not None:
         out["parity"] = parity
@@ -182,7 +192,8 @@ def main() -> int:
         "config": {"workload": "repdl.ops.mm fp32 %dx%dx%d, transB (nn.Linear forward), configs[3]" % (S, S, S),
                    "device": props.name, "cus": props.multi_processor_count},
         "roofline": {"bound": "mfma", "achieved": round(kern_tflops, 3), "peak": FP32_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(kern_tflops / FP32_PEAK_TFLOPS, 4), "traffic": None,
+                     "unit": "TFLOP/s", "frac": round(kern_tflops / FP32_PEAK_TFLOPS, 4),
+                     "traffic": round(MEASURED_TRAFFIC_BYTES["mm"]) if S == 8192 else None,
                      "kernel": "mm_kernel<NT>", "kernel_ms": round(ev_ms, 4), "kernel_ms_min": round(ev_min, 4),
                      "note": "fp32 compute peak; the kernel issues scalar v_fma_f32 only (no MFMA, packed "
                              "fp32 disabled), whose issue-rate ceiling is half of this peak"},
@@ -210,7 +221,8 @@ def main() -> int:
             cpu = {"value": round(2048 * R * 4 / dt / 1e9, 3), "unit": "GB/s", "cores": oracle.threads(),
                    "kind": kind, "sample": "first 2048 rows"}
             result["also"].append(hbm_entry("sum2d_dim1", "row sums of 16384x16384 N(0,1)*2^U(-20,20)", 4.0 * R * R + 4 * R,
-                                            f, args.steps, args.warmup, par, cpu))
+                                            f, args.steps, args.warmup, par, cpu,
+                                            round(MEASURED_TRAFFIC_BYTES["sum2d_dim1"])))
             del m_d, m_h, hold
 
         if want("sum1d"):
@@ -260,7 +272,8 @@ def main() -> int:
                     par = {"equal_on_first_2^24": sha(y_gpu_s) == sha(y_cpu_s)}
                     cpu = {"value": round(nbytes / n * sample / dt / 1e9, 3), "unit": "GB/s",
                            "cores": oracle.threads(), "kind": "port", "sample": "first 2^24 elements"}
-                    result["also"].append(hbm_entry(name, wl, nbytes, f, args.steps, args.warmup, par, cpu))
+                    result["also"].append(hbm_entry(name, wl, nbytes, f, args.steps, args.warmup, par, cpu,
+                                                    round(MEASURED_TRAFFIC_BYTES["exp"]) if name == "exp" else None))
                     hold.clear()
 
         if want("conv"):
