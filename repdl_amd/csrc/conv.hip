@@ -510,40 +510,34 @@ __device__ __forceinline__ float lane_value(float v, int k)
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), k));
 }
 
-// One step of a chain, written as an instruction pair so that the broadcast for step
-// k+16 is issued next to the FMA of step k: v_readlane_b32 has a long latency before
-// its SGPR result can feed a VALU operand (about 12 clocks measured), short enough to
-// hide behind sixteen dependent FMAs but not behind one.
-#define REPDL_WG_STEP(u)                                                                                     \
-    asm volatile("v_readlane_b32 %0, %2, %3\n\tv_fmac_f32_e32 %1, %4, %5"                                    \
-                 : "=&s"(gn[u]), "+v"(acc)                                                                   \
-                 : "v"(g), "n"(K0 + 16 + (u)), "s"(gc[u]), "v"(xv[u]))
-#define REPDL_WG_LAST(u) asm volatile("v_fmac_f32_e32 %0, %1, %2" : "+v"(acc) : "s"(gc[u]), "v"(xv[u]))
-
-// sixteen steps K0..K0+15 of a piece; gc = broadcast values of these steps, gn receives
-// those of the next sixteen (when there are any)
-template <int K0, bool MORE>
-__device__ __forceinline__ float wgrad_steps16(int g, const int (&gc)[16], int (&gn)[16], const float (&xv)[16],
-                                               float acc)
+// A step of a chain is an instruction pair: the FMA of this step and, next to it, the
+// broadcast for the step eight ahead.  v_readlane_b32 has a long latency before its SGPR
+// result can feed a VALU operand (about 12 clocks measured), short enough to hide behind
+// eight dependent FMAs but not behind one.
+// Eight steps as ONE asm block (the compiler pads every separate asm statement with an
+// s_nop, which would cost a third issue slot per step): FMAs with the broadcast values gc
+// and the taps xv[XO..XO+7]; meanwhile gn receives lanes LANE0..LANE0+7 of gsrc, the
+// broadcast values of the eight steps after.
+template <int LANE0, int XO>
+__device__ __forceinline__ float wgrad_steps8(int gsrc, const int (&gc)[8], int (&gn)[8], const float (&xv)[16],
+                                              float acc)
 {
-    if (MORE)
-    {
-        REPDL_WG_STEP(0); REPDL_WG_STEP(1); REPDL_WG_STEP(2); REPDL_WG_STEP(3);
-        REPDL_WG_STEP(4); REPDL_WG_STEP(5); REPDL_WG_STEP(6); REPDL_WG_STEP(7);
-        REPDL_WG_STEP(8); REPDL_WG_STEP(9); REPDL_WG_STEP(10); REPDL_WG_STEP(11);
-        REPDL_WG_STEP(12); REPDL_WG_STEP(13); REPDL_WG_STEP(14); REPDL_WG_STEP(15);
-    }
-    else
-    {
-        REPDL_WG_LAST(0); REPDL_WG_LAST(1); REPDL_WG_LAST(2); REPDL_WG_LAST(3);
-        REPDL_WG_LAST(4); REPDL_WG_LAST(5); REPDL_WG_LAST(6); REPDL_WG_LAST(7);
-        REPDL_WG_LAST(8); REPDL_WG_LAST(9); REPDL_WG_LAST(10); REPDL_WG_LAST(11);
-        REPDL_WG_LAST(12); REPDL_WG_LAST(13); REPDL_WG_LAST(14); REPDL_WG_LAST(15);
-    }
+    asm volatile("v_readlane_b32 %0, %9, %10\n\tv_fmac_f32_e32 %8, %18, %26\n\t"
+                 "v_readlane_b32 %1, %9, %11\n\tv_fmac_f32_e32 %8, %19, %27\n\t"
+                 "v_readlane_b32 %2, %9, %12\n\tv_fmac_f32_e32 %8, %20, %28\n\t"
+                 "v_readlane_b32 %3, %9, %13\n\tv_fmac_f32_e32 %8, %21, %29\n\t"
+                 "v_readlane_b32 %4, %9, %14\n\tv_fmac_f32_e32 %8, %22, %30\n\t"
+                 "v_readlane_b32 %5, %9, %15\n\tv_fmac_f32_e32 %8, %23, %31\n\t"
+                 "v_readlane_b32 %6, %9, %16\n\tv_fmac_f32_e32 %8, %24, %32\n\t"
+                 "v_readlane_b32 %7, %9, %17\n\tv_fmac_f32_e32 %8, %25, %33"
+                 : "=&s"(gn[0]), "=&s"(gn[1]), "=&s"(gn[2]), "=&s"(gn[3]), "=&s"(gn[4]), "=&s"(gn[5]), "=&s"(gn[6]),
+                   "=&s"(gn[7]), "+v"(acc)
+                 : "v"(gsrc), "n"(LANE0 + 0), "n"(LANE0 + 1), "n"(LANE0 + 2), "n"(LANE0 + 3), "n"(LANE0 + 4),
+                   "n"(LANE0 + 5), "n"(LANE0 + 6), "n"(LANE0 + 7), "s"(gc[0]), "s"(gc[1]), "s"(gc[2]), "s"(gc[3]),
+                   "s"(gc[4]), "s"(gc[5]), "s"(gc[6]), "s"(gc[7]), "v"(xv[XO + 0]), "v"(xv[XO + 1]), "v"(xv[XO + 2]),
+                   "v"(xv[XO + 3]), "v"(xv[XO + 4]), "v"(xv[XO + 5]), "v"(xv[XO + 6]), "v"(xv[XO + 7]));
     return acc;
 }
-#undef REPDL_WG_STEP
-#undef REPDL_WG_LAST
 
 template <bool UNIT>
 __device__ __forceinline__ void wgrad_read16(const float *__restrict__ xr, int k0, int sW, float (&xv)[16])
@@ -553,30 +547,71 @@ __device__ __forceinline__ void wgrad_read16(const float *__restrict__ xr, int k
         xv[u] = UNIT ? xr[k0 + u] : xr[(k0 + u) * sW];
 }
 
-// PIECE steps of one chain: the taps come from LDS sixteen at a time (the next sixteen
-// are read before the FMAs of the current ones), the grad_output values from lane k of g.
+// The software pipeline across the pieces of a chunk.  Invariant on entry to a piece: sa
+// holds the broadcast values of its steps 0..7 and xa the taps of its steps 0..15; on exit
+// the same holds for the next piece (g1 / x1).  Within the piece the taps are read sixteen
+// steps ahead and the broadcasts eight steps ahead of their use.
 template <int PIECE, bool UNIT>
-__device__ __forceinline__ float wgrad_piece(float gf, const float *__restrict__ xr, int sW, float acc)
+struct WgradPipe
 {
-    const int g = __float_as_int(gf);
-    int ga[16], gb[16];
+    int sa[8], sb[8];
     float xa[16], xb[16];
+
+    __device__ __forceinline__ void prime(int g0, const float *x0, int sW)
+    {
 #pragma unroll
-    for (int u = 0; u < 16; u++)
-        ga[u] = __builtin_amdgcn_readlane(g, u);
-    wgrad_read16<UNIT>(xr, 0, sW, xa);
-    if (PIECE == 16)
-        return wgrad_steps16<0, false>(g, ga, gb, xa, acc);
-    wgrad_read16<UNIT>(xr, 16, sW, xb);
-    acc = wgrad_steps16<0, true>(g, ga, gb, xa, acc);
-    if (PIECE == 32)
-        return wgrad_steps16<16, false>(g, gb, ga, xb, acc);
-    wgrad_read16<UNIT>(xr, 32, sW, xa);
-    acc = wgrad_steps16<16, true>(g, gb, ga, xb, acc);
-    wgrad_read16<UNIT>(xr, 48, sW, xb);
-    acc = wgrad_steps16<32, true>(g, ga, gb, xa, acc);
-    return wgrad_steps16<48, false>(g, gb, ga, xb, acc);
-}
+        for (int u = 0; u < 8; u++)
+            sa[u] = __builtin_amdgcn_readlane(g0, u);
+        wgrad_read16<UNIT>(x0, 0, sW, xa);
+    }
+
+    // PIECE = 32 or 64
+    __device__ __forceinline__ float piece(int g, const float *x, int g1, const float *x1, int sW, float acc)
+    {
+        if (PIECE == 64)
+        {
+            wgrad_read16<UNIT>(x, 16, sW, xb);
+            acc = wgrad_steps8<8, 0>(g, sa, sb, xa, acc);
+            acc = wgrad_steps8<16, 8>(g, sb, sa, xa, acc);
+            wgrad_read16<UNIT>(x, 32, sW, xa);
+            acc = wgrad_steps8<24, 0>(g, sa, sb, xb, acc);
+            acc = wgrad_steps8<32, 8>(g, sb, sa, xb, acc);
+            wgrad_read16<UNIT>(x, 48, sW, xb);
+            acc = wgrad_steps8<40, 0>(g, sa, sb, xa, acc);
+            acc = wgrad_steps8<48, 8>(g, sb, sa, xa, acc);
+            wgrad_read16<UNIT>(x1, 0, sW, xa);
+            acc = wgrad_steps8<56, 0>(g, sa, sb, xb, acc);
+            acc = wgrad_steps8<0, 8>(g1, sb, sa, xb, acc);
+        }
+        else
+        {
+            wgrad_read16<UNIT>(x, 16, sW, xb);
+            acc = wgrad_steps8<8, 0>(g, sa, sb, xa, acc);
+            acc = wgrad_steps8<16, 8>(g, sb, sa, xa, acc);
+            wgrad_read16<UNIT>(x1, 0, sW, xa);
+            acc = wgrad_steps8<24, 0>(g, sa, sb, xb, acc);
+            acc = wgrad_steps8<0, 8>(g1, sb, sa, xb, acc);
+        }
+        return acc;
+    }
+
+    // PIECE = 16: two pieces at a time (the second may be a dummy that only prefetches), so
+    // that the tap registers are back in xa at the end
+    __device__ __forceinline__ float pair16(int g, const float *x, int g1, const float *x1, int g2,
+                                            const float *x2, bool second, int sW, float acc)
+    {
+        wgrad_read16<UNIT>(x1, 0, sW, xb);
+        acc = wgrad_steps8<8, 0>(g, sa, sb, xa, acc);
+        acc = wgrad_steps8<0, 8>(g1, sb, sa, xa, acc);
+        if (second)
+        {
+            wgrad_read16<UNIT>(x2, 0, sW, xa);
+            acc = wgrad_steps8<8, 0>(g1, sa, sb, xb, acc);
+            acc = wgrad_steps8<0, 8>(g2, sb, sa, xb, acc);
+        }
+        return acc;
+    }
+};
 
 constexpr int WG_SLOTS = 16; // float4 staging slots per thread (16 rows x 64 floats per pass)
 constexpr int WG_Q = 16;    // row pieces per chunk (one register of grad_output each)
@@ -716,22 +751,54 @@ __global__ __launch_bounds__(256) void conv_wgrad_kernel(const float *__restrict
         {
             const int nq = ((d.OH - oh0 < R) ? d.OH - oh0 : R) * NP;
             const float *xs = lds + buf * bufsz + lane_off;
-            int r = 0, pc = 0;
-#pragma unroll
-            for (int q = 0; q < WG_Q; q++)
+            // tap pointer of piece q (row q / NP, piece q % NP of that row), clamped to the last
+            // real piece so that the prefetch past the end stays inside the staged rows
+            auto xptr = [&](int q) {
+                const int qq = q < nq ? q : nq - 1;
+                const int r = qq / NP, pc = qq - r * NP;
+                return xs + r * d.sH * Wp + pc * PIECE * d.sW;
+            };
+            const int sW = d.sW;
+            if (sW == 1)
             {
-                if (q < nq)
+                WgradPipe<PIECE, true> pipe;
+                pipe.prime(__float_as_int(gcur[0]), xptr(0), 1);
+                if (PIECE == 16)
                 {
-                    const float *xr = xs + r * d.sH * Wp + pc * PIECE * d.sW;
-                    if (d.sW == 1)
-                        acc = wgrad_piece<PIECE, true>(gcur[q], xr, 1, acc);
-                    else
-                        acc = wgrad_piece<PIECE, false>(gcur[q], xr, d.sW, acc);
+#pragma unroll
+                    for (int q = 0; q < WG_Q; q += 2)
+                        if (q < nq)
+                            acc = pipe.pair16(__float_as_int(gcur[q]), xptr(q), __float_as_int(gcur[q + 1]), xptr(q + 1),
+                                              __float_as_int(gcur[q + 2 < WG_Q ? q + 2 : q]), xptr(q + 2), q + 1 < nq, 1, acc);
                 }
-                if (++pc == NP)
+                else
                 {
-                    pc = 0;
-                    r++;
+#pragma unroll
+                    for (int q = 0; q < WG_Q; q++)
+                        if (q < nq)
+                            acc = pipe.piece(__float_as_int(gcur[q]), xptr(q), __float_as_int(gcur[q + 1 < WG_Q ? q + 1 : q]),
+                                             xptr(q + 1), 1, acc);
+                }
+            }
+            else
+            {
+                WgradPipe<PIECE, false> pipe;
+                pipe.prime(__float_as_int(gcur[0]), xptr(0), sW);
+                if (PIECE == 16)
+                {
+#pragma unroll
+                    for (int q = 0; q < WG_Q; q += 2)
+                        if (q < nq)
+                            acc = pipe.pair16(__float_as_int(gcur[q]), xptr(q), __float_as_int(gcur[q + 1]), xptr(q + 1),
+                                              __float_as_int(gcur[q + 2 < WG_Q ? q + 2 : q]), xptr(q + 2), q + 1 < nq, sW, acc);
+                }
+                else
+                {
+#pragma unroll
+                    for (int q = 0; q < WG_Q; q++)
+                        if (q < nq)
+                            acc = pipe.piece(__float_as_int(gcur[q]), xptr(q), __float_as_int(gcur[q + 1 < WG_Q ? q + 1 : q]),
+                                             xptr(q + 1), sW, acc);
                 }
             }
         }
