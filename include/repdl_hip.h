@@ -19,7 +19,8 @@
  *     repdl_hip_error_string() describes either kind.
  *   - Arithmetic contract: binary32, round to nearest even, subnormals kept;
  *     one accumulator per output element starting at +0.0f, updated by single
- *     fused multiply-adds in the loop order of RepDL's CPU backend; results are
+ *     fused multiply-adds in the loop order of RepDL's CPU backend (whether a
+ *     v_fma_f32 or a matrix instruction performs them, see "Matrix path"); results are
  *     bit-identical to that backend for finite data.  (When a NaN is produced
  *     inside a multiply-accumulate chain its sign and payload are unspecified;
  *     the elementwise operators below define NaN bits exactly.)
@@ -41,6 +42,26 @@ extern "C" {
 
 const char *repdl_hip_error_string(int code);
 int repdl_hip_abi_version(void);
+
+/* Matrix path.  No counterpart in the reference: its CUDA kernels use one FMA per
+ * term (backend/cuda/matrix_multiplication.cu:18-60, convolution.cu:62-151).
+ * mm and the three convolutions have two implementations of the same chains: one on
+ * the binary32 matrix instructions of gfx950 (v_mfma_f32_32x32x2_f32 /
+ * v_mfma_f32_16x16x4_f32) and one on v_fma_f32.  The matrix instructions are used
+ * only after a check on the device itself has found them bit-identical to chains of
+ * single-rounding FMAs, k ascending (the first GEMM-shaped call on a device runs
+ * about a million comparisons, synchronously, once).
+ *   repdl_hip_mfma_selftest: runs waves*trials further comparisons of each
+ *     instruction (operand classes cycle with the trial number) and writes the
+ *     number of differing results to mismatches[0] (32x32x2) and mismatches[1]
+ *     (16x16x4), HOST memory.  Synchronous.
+ *   repdl_hip_set_matrix_path: -1 = decide by the check (default), 0 = always the
+ *     v_fma_f32 kernels, 1 = always the matrix kernels.  Process-wide.
+ *   repdl_hip_matrix_path: 1 if GEMM-shaped calls on the current device now take the
+ *     matrix kernels, else 0 (runs the check if it has not run yet). */
+int repdl_hip_mfma_selftest(int64_t waves, int64_t trials, uint64_t seed, uint64_t *mismatches);
+int repdl_hip_set_matrix_path(int mode);
+int repdl_hip_matrix_path(void);
 
 /* mm -- backend/cuda/matrix_multiplication.cu:234-260 (bound at :267);
  * semantics backend/cpu/matrix_multiplication.cpp:12-36.

@@ -35,6 +35,8 @@ SIGNATURES = {
     "repdl_hip_div_scalar": [_P, _F32, _P, _I64, _P],
     "repdl_hip_softmax": [_P, _P, _I64, _I64, _P],
     "repdl_hip_cross_entropy": [_P, _P, _P, _I64, _I64, _P, _P],
+    "repdl_hip_mfma_selftest": [_I64, _I64, ctypes.c_uint64, ctypes.POINTER(ctypes.c_uint64)],
+    "repdl_hip_set_matrix_path": [_INT],
 }
 
 _lib = None
@@ -61,6 +63,8 @@ def lib() -> ctypes.CDLL:
         handle.repdl_hip_error_string.restype = ctypes.c_char_p
         handle.repdl_hip_sum1d_workspace_bytes.argtypes = [_I64]
         handle.repdl_hip_sum1d_workspace_bytes.restype = ctypes.c_size_t
+        handle.repdl_hip_matrix_path.argtypes = []
+        handle.repdl_hip_matrix_path.restype = _INT
         handle.repdl_hip_abi_version.argtypes = []
         handle.repdl_hip_abi_version.restype = _INT
         _lib = handle

@@ -32,6 +32,11 @@ static inline hipStream_t repdl_stream(void *s) { return reinterpret_cast<hipStr
 
 static inline int64_t repdl_cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// True when the binary32 matrix instructions of the current device were checked (or forced,
+// see repdl_hip_set_matrix_path) to evaluate k-ascending chains of single-rounding FMAs;
+// the GEMM-shaped operators then use them, otherwise their v_fma_f32 kernels.
+bool repdl_mfma_exact();
+
 __device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
 __device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
 

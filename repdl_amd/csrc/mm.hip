@@ -4,16 +4,22 @@
 // element owns one accumulator that starts at +0.0f and receives exactly one
 // fused multiply-add per k, k ascending.  Tiling over M and N and the way the
 // operands are staged are free; the order along K is not, so K is never split
-// across threads, there is no K padding (the last partial K tile runs a shorter
-// loop) and MFMA is not used (its internal accumulation is not a sequence of
-// single-rounding FMAs).
+// across threads.
 //
-// Layout: a workgroup of 256 threads computes a 128x128 tile of C; each thread
+// Two kernels implement it.  mm_mfma_kernel feeds v_mfma_f32_32x32x2_f32, which on
+// gfx950 evaluates exactly such a chain (two k per instruction, ascending; checked
+// on the device before first use, see mfma_check.hip).  mm_kernel is the same
+// computation with one v_fma_f32 per term; it runs when that check fails or the
+// matrix path is switched off.
+//
+// mm_kernel layout: a workgroup of 256 threads computes a 128x128 tile of C; each thread
 // an 8x8 micro-tile held in registers (rows ty*4+{0..3} and 64+ty*4+{0..3},
 // columns tx*4+{0..3} and 64+tx*4+{0..3}).  Both operands are staged through LDS
 // k-major (As[k][m], Bs[k][n]) so the inner loop reads its 8+8 operands with
 // four ds_read_b128 and issues 64 v_fma_f32.  Global loads for tile t+1 are
 // issued before the FMAs of tile t (register prefetch, two LDS buffers).
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace
@@ -229,6 +235,252 @@ __global__ __launch_bounds__(NT) void mm_kernel(const float *__restrict__ A,
     }
 }
 
+// ---------------------------------------------------------------------------
+// Matrix-core kernel.  A workgroup of WGM x WGN waves computes a (32 FM WGM) x
+// (32 FN WGN) tile of C; each wave FM x FN blocks of 32x32, one
+// v_mfma_f32_32x32x2_f32 per block and pair of k.  The instruction takes from lane l
+// the A element of row l%32 and the B element of column l%32, both at k = l/32, and
+// adds the k = 0 product to the accumulator first.  Operand tiles sit in LDS k-major
+// exactly as in mm_kernel, so an operand register is one ds_read_b32: lanes 0..31
+// read 32 consecutive rows at k, lanes 32..63 the same rows at k+1.
+//
+// K tail: positions k >= K are filled with -0.0f in the A tile and +0.0f in the B
+// tile.  Their product is -0, and x + (-0) = x for every x (both zeros, infinities
+// and NaN included), so a padded step leaves every accumulator bit for bit
+// unchanged.
+// ---------------------------------------------------------------------------
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+template <int R, int NTH>
+struct TileFrag
+{
+    float4 v[R * BK / 4 / NTH];
+};
+
+// Same two memory layouts as load_tile above, for an R x BK tile and NTH threads; k >= K
+// (and rows beyond Rlim, whose products are never stored) read as `pad`.
+template <bool KC, int R, int NTH>
+__device__ __forceinline__ void load_tile_pad(const float *__restrict__ X, int64_t ld, int64_t Rlim, int64_t K,
+                                              int64_t r0, int64_t k0, bool vec_ok, int tid, float pad,
+                                              TileFrag<R, NTH> &f)
+{
+    constexpr int NV = R * BK / 4 / NTH;
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+    {
+        const int idx = tid + NTH * i;
+        float4 v = make_float4(pad, pad, pad, pad);
+        if (KC)
+        {
+            const int64_t r = r0 + (idx >> 2), k = k0 + ((idx & 3) << 2);
+            if (r < Rlim)
+            {
+                const float *p = X + r * ld + k;
+                if (vec_ok && k + 3 < K)
+                    v = *reinterpret_cast<const float4 *>(p);
+                else
+                {
+                    if (k + 0 < K) v.x = p[0];
+                    if (k + 1 < K) v.y = p[1];
+                    if (k + 2 < K) v.z = p[2];
+                    if (k + 3 < K) v.w = p[3];
+                }
+            }
+        }
+        else
+        {
+            const int64_t k = k0 + idx / (R / 4), r = r0 + (idx % (R / 4)) * 4;
+            if (k < K)
+            {
+                const float *p = X + k * ld + r;
+                if (vec_ok && r + 3 < Rlim)
+                    v = *reinterpret_cast<const float4 *>(p);
+                else
+                {
+                    if (r + 0 < Rlim) v.x = p[0];
+                    if (r + 1 < Rlim) v.y = p[1];
+                    if (r + 2 < Rlim) v.z = p[2];
+                    if (r + 3 < Rlim) v.w = p[3];
+                }
+            }
+        }
+        f.v[i] = v;
+    }
+}
+
+template <bool KC, int R, int NTH>
+__device__ __forceinline__ void store_tile_pad(float *__restrict__ S, int tid, const TileFrag<R, NTH> &f)
+{
+    constexpr int NV = R * BK / 4 / NTH, LD = R + 4;
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+    {
+        const int idx = tid + NTH * i;
+        if (KC)
+        {
+            const int r = idx >> 2, k = (idx & 3) << 2;
+            S[(k + 0) * LD + r] = f.v[i].x;
+            S[(k + 1) * LD + r] = f.v[i].y;
+            S[(k + 2) * LD + r] = f.v[i].z;
+            S[(k + 3) * LD + r] = f.v[i].w;
+        }
+        else
+        {
+            const int k = idx / (R / 4), r = (idx % (R / 4)) * 4;
+            *reinterpret_cast<float4 *>(&S[k * LD + r]) = f.v[i];
+        }
+    }
+}
+
+template <bool TA, bool TB, int FM, int FN, int WGM, int WGN>
+__global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_kernel(const float *__restrict__ A, const float *__restrict__ B,
+                                                                float *__restrict__ C, int64_t M, int64_t N, int64_t K,
+                                                                int avec, int bvec, int64_t gx, int64_t gy,
+                                                                int64_t ntiles8)
+{
+    constexpr int NTH = 64 * WGM * WGN;
+    constexpr int TM = 32 * FM * WGM, TN = 32 * FN * WGN;
+    constexpr int LDA_ = TM + 4, LDB_ = TN + 4;
+    constexpr bool A_KC = !TA, B_KC = TB;
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    float *const As = smem;                 // [2][BK * LDA_]
+    float *const Bs = smem + 2 * BK * LDA_; // [2][BK * LDB_]
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave % WGM, wn = wave / WGM;
+    const int l32 = lane & 31, half = lane >> 5;
+
+    // tile order: see mm_kernel
+    int64_t tile = blockIdx.x;
+    if (tile < ntiles8)
+        tile = (tile & 7) * (ntiles8 >> 3) + (tile >> 3);
+    const int64_t group_sz = (int64_t)GROUP_M * gx;
+    const int64_t group = tile / group_sz;
+    const int64_t first_row = group * GROUP_M;
+    const int64_t rows_here = (gy - first_row < GROUP_M) ? gy - first_row : GROUP_M;
+    const int64_t in_group = tile - group * group_sz;
+    const int64_t trow = first_row + in_group % rows_here, tcol = in_group / rows_here;
+    const int64_t m0 = trow * TM, n0 = tcol * TN;
+    const int64_t lda = TA ? M : K, ldb = TB ? K : N;
+
+    f16v acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[i][j][r] = 0.0f;
+
+    const int a_off = half * LDA_ + wm * 32 * FM + l32;
+    const int b_off = half * LDB_ + wn * 32 * FN + l32;
+    const int64_t nkt = (K + BK - 1) / BK;
+    TileFrag<TM, NTH> fa;
+    TileFrag<TN, NTH> fb;
+    if (nkt > 0)
+    {
+        load_tile_pad<A_KC, TM, NTH>(A, lda, M, K, m0, 0, avec, tid, -0.0f, fa);
+        load_tile_pad<B_KC, TN, NTH>(B, ldb, N, K, n0, 0, bvec, tid, 0.0f, fb);
+        store_tile_pad<A_KC, TM, NTH>(As, tid, fa);
+        store_tile_pad<B_KC, TN, NTH>(Bs, tid, fb);
+    }
+    __syncthreads();
+
+    for (int64_t kt = 0; kt < nkt; kt++)
+    {
+        const int cur = (int)(kt & 1);
+        const bool more = kt + 1 < nkt;
+        if (more)
+        {
+            load_tile_pad<A_KC, TM, NTH>(A, lda, M, K, m0, (kt + 1) * BK, avec, tid, -0.0f, fa);
+            load_tile_pad<B_KC, TN, NTH>(B, ldb, N, K, n0, (kt + 1) * BK, bvec, tid, 0.0f, fb);
+        }
+        // Every k-tile runs all BK / 2 instructions per block (the tail of K is padded, see
+        // above): one code path keeps the accumulators in place.  All operand registers of
+        // the tile are read before the first instruction is issued.
+        const float *as = As + cur * BK * LDA_ + a_off, *bs = Bs + cur * BK * LDB_ + b_off;
+        float a[BK / 2][FM], b[BK / 2][FN];
+#pragma unroll
+        for (int kp = 0; kp < BK / 2; kp++)
+        {
+#pragma unroll
+            for (int i = 0; i < FM; i++)
+                a[kp][i] = as[2 * kp * LDA_ + 32 * i];
+#pragma unroll
+            for (int j = 0; j < FN; j++)
+                b[kp][j] = bs[2 * kp * LDB_ + 32 * j];
+        }
+#pragma unroll
+        for (int kp = 0; kp < BK / 2; kp++)
+#pragma unroll
+            for (int i = 0; i < FM; i++)
+#pragma unroll
+                for (int j = 0; j < FN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kp][i], b[kp][j], acc[i][j], 0, 0, 0);
+        if (more)
+        {
+            store_tile_pad<A_KC, TM, NTH>(As + (cur ^ 1) * BK * LDA_, tid, fa);
+            store_tile_pad<B_KC, TN, NTH>(Bs + (cur ^ 1) * BK * LDB_, tid, fb);
+        }
+        __syncthreads();
+    }
+
+    // register r of a block is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+        {
+            const int64_t m = m0 + wm * 32 * FM + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3);
+            if (m >= M)
+                continue;
+#pragma unroll
+            for (int j = 0; j < FN; j++)
+            {
+                const int64_t n = n0 + wn * 32 * FN + 32 * j + l32;
+                if (n < N)
+                    C[m * N + n] = acc[i][j][r];
+            }
+        }
+}
+
+template <bool TA, bool TB, int FM, int FN, int WGM, int WGN>
+int launch_mfma_t(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int avec, int bvec,
+                  hipStream_t s)
+{
+    constexpr int TM = 32 * FM * WGM, TN = 32 * FN * WGN;
+    constexpr size_t shmem = (size_t)2 * BK * (TM + 4 + TN + 4) * sizeof(float);
+    const int64_t gx = repdl_cdiv(N, TN), gy = repdl_cdiv(M, TM);
+    if (gx * gy > REPDL_I32_MAX)
+        return REPDL_E_ARG;
+    const int64_t ntiles8 = (gx * gy) & ~(int64_t)7;
+    auto kern = &mm_mfma_kernel<TA, TB, FM, FN, WGM, WGN>;
+    if (shmem > 48 * 1024)
+    {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)shmem);
+        if (e != hipSuccess)
+            return (int)e;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)(gx * gy)), dim3(64 * WGM * WGN), shmem, s, A, B, C, M, N, K, avec, bvec, gx, gy,
+                       ntiles8);
+    return repdl_launch_status();
+}
+
+template <int FM, int FN, int WGM, int WGN>
+int launch_mfma(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int transA, int transB,
+                int avec, int bvec, hipStream_t s)
+{
+    if (!transA && !transB)
+        return launch_mfma_t<false, false, FM, FN, WGM, WGN>(A, B, C, M, N, K, avec, bvec, s);
+    if (transA && !transB)
+        return launch_mfma_t<true, false, FM, FN, WGM, WGN>(A, B, C, M, N, K, avec, bvec, s);
+    if (!transA && transB)
+        return launch_mfma_t<false, true, FM, FN, WGM, WGN>(A, B, C, M, N, K, avec, bvec, s);
+    return launch_mfma_t<true, true, FM, FN, WGM, WGN>(A, B, C, M, N, K, avec, bvec, s);
+}
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 } // namespace
 
@@ -240,15 +492,40 @@ REPDL_API int repdl_hip_mm(const float *A, const float *B, float *C, int64_t M, 
         return REPDL_OK;
     REPDL_REQUIRE(C != nullptr);
     REPDL_REQUIRE(K == 0 || (A != nullptr && B != nullptr));
-    const int64_t gx = repdl_cdiv(N, BN), gy = repdl_cdiv(M, BM);
-    REPDL_REQUIRE(gx * gy <= REPDL_I32_MAX);
-    const int64_t ntiles8 = (gx * gy) & ~(int64_t)7; // tiles covered by whole rounds over the 8 XCDs
     const int64_t lda = transA ? M : K, ldb = transB ? K : N;
     const int avec = aligned16(A) && (lda % 4 == 0);
     const int bvec = aligned16(B) && (ldb % 4 == 0);
+    hipStream_t s = repdl_stream(stream);
+    if (repdl_mfma_exact())
+    {
+        // the largest tile that still gives every CU several workgroups
+        int cfg = 0;
+        const int64_t target = 2 * 256;
+        if (repdl_cdiv(M, 256) * repdl_cdiv(N, 256) >= target)
+            cfg = 3;
+        else if (repdl_cdiv(M, 128) * repdl_cdiv(N, 128) >= target)
+            cfg = 1;
+        if (const char *e = getenv("REPDL_HIP_MM_TILE"))
+            cfg = atoi(e);
+        switch (cfg)
+        {
+        case 0:
+            return launch_mfma<1, 1, 2, 2>(A, B, C, M, N, K, transA, transB, avec, bvec, s);
+        case 1:
+            return launch_mfma<2, 2, 2, 2>(A, B, C, M, N, K, transA, transB, avec, bvec, s);
+        case 2:
+            return launch_mfma<4, 2, 2, 2>(A, B, C, M, N, K, transA, transB, avec, bvec, s);
+        case 3:
+            return launch_mfma<4, 2, 2, 4>(A, B, C, M, N, K, transA, transB, avec, bvec, s);
+        default:
+            return launch_mfma<4, 4, 2, 2>(A, B, C, M, N, K, transA, transB, avec, bvec, s);
+        }
+    }
+    const int64_t gx = repdl_cdiv(N, BN), gy = repdl_cdiv(M, BM);
+    REPDL_REQUIRE(gx * gy <= REPDL_I32_MAX);
+    const int64_t ntiles8 = (gx * gy) & ~(int64_t)7; // tiles covered by whole rounds over the 8 XCDs
     const int cvec = aligned16(C) && (N % 4 == 0);
     dim3 grid((unsigned)(gx * gy)), block(NT);
-    hipStream_t s = repdl_stream(stream);
     if (!transA && !transB)
         hipLaunchKernelGGL((mm_kernel<false, false>), grid, block, 0, s, A, B, C, M, N, K, avec, bvec, cvec, gx, gy, ntiles8);
     else if (transA && !transB)

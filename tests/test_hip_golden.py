@@ -11,8 +11,13 @@ from oracle import api as oracle
 pytestmark = pytest.mark.gpu
 
 
+GEMM_SHAPED = ("mm", "conv2d")
+
+
 @pytest.mark.parametrize("case", cases.CASES, ids=[c["name"] for c in cases.CASES])
-def test_hip_matches_reference_digest(case, golden):
+def test_hip_matches_reference_digest(case, golden, matrix_path):
+    if matrix_path == "fma" and not case["name"].startswith(GEMM_SHAPED):
+        pytest.skip("only one implementation of this operator")
     from hipbackend import backend
 
     g = golden[case["name"]]

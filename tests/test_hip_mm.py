@@ -6,7 +6,7 @@ import torch
 import gen
 from oracle import api as oracle
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("matrix_path")]
 
 SHAPES = [(128, 128, 16), (127, 129, 15), (257, 130, 1000), (1, 513, 77), (640, 1, 3), (384, 256, 2049), (2, 2, 2)]
 
@@ -58,3 +58,44 @@ def test_determinism():
     a, b = gen.normal_like(5, 700, 900).cuda(), gen.normal_like(6, 900, 500).cuda()
     h = {gen.sha256(ops.mm(a, b)) for _ in range(5)}
     assert len(h) == 1
+
+
+def _same_bits_or_both_nan(got, want):
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(got), nan)
+    return torch.equal(got.view(torch.int32)[~nan], want.view(torch.int32)[~nan])
+
+
+@pytest.mark.parametrize("tA,tB", [(0, 1), (1, 0)])
+def test_special_values(tA, tB):
+    """Zeros of both signs, subnormals, products that underflow or overflow, infinities:
+    the chains must still agree bit for bit (NaN results only have to be NaN)."""
+    from repdl_amd import ops
+
+    M, N, K = 200, 136, 333
+    a = gen.elementwise_mix(11, M * K).view((K, M) if tA else (M, K))
+    b = gen.elementwise_mix(12, N * K).view((N, K) if tB else (K, N))
+    a = torch.where(torch.isnan(a), torch.zeros_like(a), a)
+    b = torch.where(torch.isnan(b), torch.full_like(b, -0.0), b)
+    got = ops.mm(a.cuda(), b.cuda(), bool(tA), bool(tB)).cpu()
+    assert _same_bits_or_both_nan(got, oracle.mm(a, b, bool(tA), bool(tB)))
+    # tiny magnitudes: every product is subnormal or underflows, sums of signed zeros
+    a = gen.scaled_normal(13, M, K, lo=-90, hi=-70)
+    b = gen.scaled_normal(14, K, N, lo=-80, hi=-60) * gen.relu_like(15, K, N).sign()
+    got = ops.mm(a.cuda(), b.cuda()).cpu()
+    want = oracle.mm(a, b)
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+    assert (want.abs() < 2.0 ** -126).all() and (want != 0).any()
+
+
+@pytest.mark.parametrize("K", [1, 2, 3, 15, 16, 17, 31, 33])
+def test_k_tails_keep_negative_zero(K):
+    """A K that does not fill the last tile must not disturb an accumulator that is -0."""
+    from repdl_amd import ops
+
+    a = torch.full((70, K), -1e-30)
+    b = torch.full((K, 40), 1e-30)  # every product rounds to -0, so every result is -0
+    got = ops.mm(a.cuda(), b.cuda()).cpu()
+    want = oracle.mm(a, b)
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+    assert (want.view(torch.int32) == -(2 ** 31)).all()
