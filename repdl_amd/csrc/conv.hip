@@ -178,7 +178,9 @@ __device__ __forceinline__ void kpos_advance(KPos &p, const KStep &s, int KH, in
     p.c += s.dc;
 }
 
-template <int BM, int MODE>
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+template <int BM, int MODE, bool MFMA>
 __global__ __launch_bounds__(2 * BM) void conv_gemm_kernel(const float *__restrict__ Xg, // gathered operand: input (FWD) / grad_output (DGRAD)
                                                            const float *__restrict__ Wt, // kernel
                                                            float *__restrict__ Out, ConvDims d, int wvec,
@@ -268,11 +270,13 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_kernel(const float *__restri
 
     float4 fa[NA], fb[NB];
 
+    // Positions k >= K hold -0.0f here and +0.0f in the gathered operand: the product is -0
+    // and x + (-0) = x for every x, so the matrix kernel can run whole k-tiles.
     auto load_a = [&](int k0) {
 #pragma unroll
         for (int i = 0; i < NA; i++)
         {
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            float4 v = make_float4(-0.0f, -0.0f, -0.0f, -0.0f);
             if (MODE == MODE_FWD)
             {
                 const int idx = tid + NT * i;
@@ -384,100 +388,188 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_kernel(const float *__restri
         }
     };
 
-    float acc[8][8];
+    float *Oimg = Out + (int64_t)n * (MODE == MODE_FWD ? d.OC : d.IC) * P;
+    const int nkt = (K + BK - 1) / BK;
+    if constexpr (MFMA)
+    {
+        // Matrix-instruction form: each wave owns 64 rows x 64 pixels as 2 x 2 blocks of
+        // v_mfma_f32_32x32x2_f32 (lane l supplies row / pixel l%32 at k = l/32, the k = 0
+        // product is added first).  BM = 64: two waves side by side; BM = 128: 2 x 2 waves.
+        const int lane = tid & 63, l32 = lane & 31, half = lane >> 5;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int wm = BM == 64 ? 0 : (wave & 1), wn = BM == 64 ? wave : (wave >> 1);
+        f16v acc[2][2];
 #pragma unroll
-    for (int i = 0; i < 8; i++)
+        for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 8; j++)
-            acc[i][j] = 0.0f;
-
-    auto fma_step = [&](const float *A, const float *B, int kk) {
-        const float4 a0 = *reinterpret_cast<const float4 *>(&A[kk * LDA + ty * 4]);
-        const float4 a1 = *reinterpret_cast<const float4 *>(&A[kk * LDA + BM / 2 + ty * 4]);
-        const float4 b0 = *reinterpret_cast<const float4 *>(&B[kk * LDB + tx * 4]);
-        const float4 b1 = *reinterpret_cast<const float4 *>(&B[kk * LDB + 64 + tx * 4]);
-        const float a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
-        const float b[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    acc[i][j][r] = 0.0f;
+        const int a_off = half * LDA + wm * 64 + l32, b_off = half * LDB + wn * 64 + l32;
+        if (nkt > 0)
+        {
+            load_a(0);
+            load_b();
+            store_a(As[0]);
+            store_b(Bs[0]);
+        }
+        __syncthreads();
+        for (int kt = 0; kt < nkt; kt++)
+        {
+            const int cur = kt & 1;
+            const bool more = kt + 1 < nkt;
+            if (more)
+            {
+                load_a((kt + 1) * BK);
+                load_b();
+            }
+            const float *as = As[cur] + a_off, *bs = Bs[cur] + b_off;
+            float a[BK / 2][2], b[BK / 2][2];
+#pragma unroll
+            for (int kp = 0; kp < BK / 2; kp++)
+            {
+                a[kp][0] = as[2 * kp * LDA];
+                a[kp][1] = as[2 * kp * LDA + 32];
+                b[kp][0] = bs[2 * kp * LDB];
+                b[kp][1] = bs[2 * kp * LDB + 32];
+            }
+#pragma unroll
+            for (int kp = 0; kp < BK / 2; kp++)
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kp][i], b[kp][j], acc[i][j], 0, 0, 0);
+            if (more)
+            {
+                store_a(As[cur ^ 1]);
+                store_b(Bs[cur ^ 1]);
+            }
+            __syncthreads();
+        }
+        // register r of a block: row 8*(r/4) + 4*(lane/32) + r%4, pixel lane%32
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+            {
+                const int m = m0 + wm * 64 + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3);
+                if (m >= M)
+                    continue;
+                const int ch = MODE == MODE_FWD ? g * OCg + m : m;
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                {
+                    const int pix = p0 + wn * 64 + 32 * j + l32;
+                    if (pix >= P)
+                        continue;
+                    float v = acc[i][j][r];
+                    if (((__float_as_uint(v) << 1) == 0u) || (v != v))
+                    {
+                        const int ph = pix / PW, pw = pix - ph * PW;
+                        v = MODE == MODE_FWD ? conv2d_exact(Xg, Wt, d, n, ch, ph, pw)
+                                             : conv2d_grad_input_exact(Xg, Wt, d, n, ch, ph, pw);
+                    }
+                    Oimg[(int64_t)ch * P + pix] = v;
+                }
+            }
+    }
+    else
+    {
+        float acc[8][8];
 #pragma unroll
         for (int i = 0; i < 8; i++)
 #pragma unroll
             for (int j = 0; j < 8; j++)
-                acc[i][j] = __fmaf_rn(a[i], b[j], acc[i][j]);
-    };
+                acc[i][j] = 0.0f;
 
-    const int nkt = (K + BK - 1) / BK;
-    if (nkt > 0)
-    {
-        load_a(0);
-        load_b();
-        store_a(As[0]);
-        store_b(Bs[0]);
-    }
-    __syncthreads();
-    for (int kt = 0; kt < nkt; kt++)
-    {
-        const int cur = kt & 1;
-        const bool more = kt + 1 < nkt;
-        if (more)
-        {
-            load_a((kt + 1) * BK);
-            load_b();
-        }
-        const int krem = K - kt * BK;
-        if (krem >= BK)
-        {
+        auto fma_step = [&](const float *A, const float *B, int kk) {
+            const float4 a0 = *reinterpret_cast<const float4 *>(&A[kk * LDA + ty * 4]);
+            const float4 a1 = *reinterpret_cast<const float4 *>(&A[kk * LDA + BM / 2 + ty * 4]);
+            const float4 b0 = *reinterpret_cast<const float4 *>(&B[kk * LDB + tx * 4]);
+            const float4 b1 = *reinterpret_cast<const float4 *>(&B[kk * LDB + 64 + tx * 4]);
+            const float a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+            const float b[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
 #pragma unroll
-            for (int kk = 0; kk < BK; kk++)
-                fma_step(As[cur], Bs[cur], kk);
-        }
-        else
+            for (int i = 0; i < 8; i++)
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    acc[i][j] = __fmaf_rn(a[i], b[j], acc[i][j]);
+        };
+
+        if (nkt > 0)
         {
-            for (int kk = 0; kk < krem; kk++)
-                fma_step(As[cur], Bs[cur], kk);
-        }
-        if (more)
-        {
-            store_a(As[cur ^ 1]);
-            store_b(Bs[cur ^ 1]);
+            load_a(0);
+            load_b();
+            store_a(As[0]);
+            store_b(Bs[0]);
         }
         __syncthreads();
-    }
-
-    // ---- epilogue: exact recompute of +-0 / NaN results, then store ----
-    float *Oimg = Out + (int64_t)n * (MODE == MODE_FWD ? d.OC : d.IC) * P;
-#pragma unroll
-    for (int i = 0; i < 8; i++)
-    {
-        const int m = m0 + ty * 4 + (i & 3) + (i >> 2) * (BM / 2);
-        if (m >= M)
-            continue;
-        const int ch = MODE == MODE_FWD ? g * OCg + m : m; // output channel (FWD) / input channel (DGRAD)
-#pragma unroll
-        for (int jh = 0; jh < 2; jh++)
+        for (int kt = 0; kt < nkt; kt++)
         {
-            const int pix = p0 + tx * 4 + jh * 64;
-            float v[4];
-#pragma unroll
-            for (int j = 0; j < 4; j++)
+            const int cur = kt & 1;
+            const bool more = kt + 1 < nkt;
+            if (more)
             {
-                v[j] = acc[i][jh * 4 + j];
-                const bool suspect = ((__float_as_uint(v[j]) << 1) == 0u) || (v[j] != v[j]);
-                if (suspect && pix + j < P)
-                {
-                    const int ph = (pix + j) / PW, pw = (pix + j) - ph * PW;
-                    v[j] = MODE == MODE_FWD ? conv2d_exact(Xg, Wt, d, n, ch, ph, pw)
-                                            : conv2d_grad_input_exact(Xg, Wt, d, n, ch, ph, pw);
-                }
+                load_a((kt + 1) * BK);
+                load_b();
             }
-            float *p = Oimg + (int64_t)ch * P + pix;
-            if (ovec && pix + 3 < P)
-                *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+            const int krem = K - kt * BK;
+            if (krem >= BK)
+            {
+#pragma unroll
+                for (int kk = 0; kk < BK; kk++)
+                    fma_step(As[cur], Bs[cur], kk);
+            }
             else
             {
+                for (int kk = 0; kk < krem; kk++)
+                    fma_step(As[cur], Bs[cur], kk);
+            }
+            if (more)
+            {
+                store_a(As[cur ^ 1]);
+                store_b(Bs[cur ^ 1]);
+            }
+            __syncthreads();
+        }
+
+        // ---- epilogue: exact recompute of +-0 / NaN results, then store ----
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+        {
+            const int m = m0 + ty * 4 + (i & 3) + (i >> 2) * (BM / 2);
+            if (m >= M)
+                continue;
+            const int ch = MODE == MODE_FWD ? g * OCg + m : m; // output channel (FWD) / input channel (DGRAD)
+#pragma unroll
+            for (int jh = 0; jh < 2; jh++)
+            {
+                const int pix = p0 + tx * 4 + jh * 64;
+                float v[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++)
-                    if (pix + j < P)
-                        p[j] = v[j];
+                {
+                    v[j] = acc[i][jh * 4 + j];
+                    const bool suspect = ((__float_as_uint(v[j]) << 1) == 0u) || (v[j] != v[j]);
+                    if (suspect && pix + j < P)
+                    {
+                        const int ph = (pix + j) / PW, pw = (pix + j) - ph * PW;
+                        v[j] = MODE == MODE_FWD ? conv2d_exact(Xg, Wt, d, n, ch, ph, pw)
+                                                : conv2d_grad_input_exact(Xg, Wt, d, n, ch, ph, pw);
+                    }
+                }
+                float *p = Oimg + (int64_t)ch * P + pix;
+                if (ovec && pix + 3 < P)
+                    *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+                else
+                {
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        if (pix + j < P)
+                            p[j] = v[j];
+                }
             }
         }
     }
@@ -819,6 +911,256 @@ __global__ __launch_bounds__(256) void conv_wgrad_kernel(const float *__restrict
     }
 }
 
+// ---------------------------------------------------------------------------
+// grad-kernel on the matrix instruction v_mfma_f32_16x16x4_f32 (four k per
+// instruction, ascending, each a single-rounding FMA; see mfma_check.hip).
+// A wave owns ONE 16 (oc) x 16 (columns) block: the chains are as long as the batch
+// and cannot be split, so what counts is the time per step of a chain, and a
+// dependent sequence of these instructions advances 256 chains by four steps in 32
+// clocks with two operand registers per instruction.  While a matrix instruction
+// runs, the SIMD issues no vector ALU instruction of any wave (measured), so every
+// VALU instruction on that SIMD lengthens the chain: the work is split by wave.
+//
+// A workgroup is four waves, one workgroup per CU, one wave per SIMD.  Waves 0 and 1
+// compute (2 x 16 oc over the same 16 columns): LDS reads and matrix instructions,
+// next to no VALU.  Waves 2 and 3 stage: per chunk (R output rows of one image) they
+// bring
+//   * grad_output[n][oc0..oc0+31][oh0..oh0+R)[*]: R*OW consecutive floats per oc, at
+//     pitch GP (GP = 4 mod 32: the 64 lanes of an operand read hit every bank twice);
+//   * the input rows the 16 columns touch, zero-padded left and right as in
+//     conv_wgrad_kernel, so that a tap is an LDS word at a fixed per-lane offset
+// into the LDS buffer that is not being computed from, and then issue the global
+// loads of the chunk after, which stay in flight across the barrier.  Staging slots
+// beyond the data load word 0 of the chunk and store nothing.
+// Lane l of a computing wave supplies, for the four steps ow..ow+3 of one
+// instruction, grad_output of oc l%16 and the tap of column l%16, both at step l/16.
+// Operands are read a piece (QP instructions) ahead.  Out-of-image taps read staged
+// zeros, so +-0 / NaN results are recomputed with the literal chain, as everywhere
+// in this file.  Requires OW % (4 QP) == 0, OH % R == 0 and 16-byte aligned
+// grad_output; other shapes take conv_wgrad_kernel.
+// ---------------------------------------------------------------------------
+typedef float f4v __attribute__((ext_vector_type(4)));
+constexpr int MW_GS = 16; // float4 staging slots of grad_output per staging thread
+constexpr int MW_XS = 8;  // float4 staging slots of input per staging thread
+constexpr int MW_OC = 32; // oc per workgroup
+constexpr int MW_ST = 128; // staging threads
+
+template <int QP, bool UNIT> // QP: instructions per piece
+__global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__restrict__ GO,
+                                                              const float *__restrict__ X,
+                                                              float *__restrict__ GK, ConvDims d, int R, int NP,
+                                                              int GP, int Wp, int CP, int hrows, int xoff, int bufsz,
+                                                              int xvec)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int tid = threadIdx.x;
+    const bool stager = __builtin_amdgcn_readfirstlane(tid >> 7) != 0;
+    const int KHW = d.KH * d.KW, NC = d.IC * KHW;
+    const int c0 = blockIdx.x * 16;
+    const int ic_first = c0 / KHW;
+    const int oc0 = blockIdx.y * MW_OC;
+    const int OWp = 4 * QP * NP; // = OW
+    const int nchunks = d.N * (d.OH / R);
+
+    for (int i = tid; i < 2 * bufsz; i += 256)
+        lds[i] = 0.0f;
+    __syncthreads();
+
+    if (stager)
+    {
+        const int st = tid & (MW_ST - 1);
+        const int last_col = (c0 + 15 < NC) ? c0 + 15 : NC - 1;
+        const int nic = last_col / KHW - ic_first + 1;
+        // slots, fixed for the whole kernel.  Input: slot = (staged row, 4 floats of it).
+        const int nw4 = (d.W + 3) >> 2;
+        const int nxs = nic * hrows * nw4;
+        int x_goff[MW_XS], x_hr[MW_XS], x_w[MW_XS], x_loff[MW_XS];
+#pragma unroll
+        for (int i = 0; i < MW_XS; i++)
+        {
+            const int s = st + MW_ST * i;
+            const bool on = s < nxs;
+            const int row = s / nw4, w = (s - row * nw4) << 2;
+            const int icl = row / hrows, hr = row - icl * hrows;
+            x_goff[i] = on ? (ic_first + icl) * d.H * d.W + w : 0;
+            x_hr[i] = hr;
+            x_w[i] = on ? w : 0;
+            x_loff[i] = on ? xoff + icl * CP + hr * Wp + d.pW + w : -1;
+        }
+        // grad_output: slot = (oc, 4 consecutive steps of the chunk)
+        const int spo = (R * d.OW) >> 2; // float4 per oc and chunk
+        uint32_t g_goff[MW_GS];
+        int g_loff[MW_GS];
+#pragma unroll
+        for (int i = 0; i < MW_GS; i++)
+        {
+            const int s = st + MW_ST * i;
+            const bool on = s < MW_OC * spo;
+            const int o = s / spo, t = (s - o * spo) << 2;
+            const int oc = oc0 + o < d.OC ? oc0 + o : d.OC - 1; // rows of missing oc repeat the last one
+            g_goff[i] = on ? (uint32_t)((oc - oc0) * d.OH * d.OW + t) * 4u : 0u;
+            g_loff[i] = on ? 64 + o * GP + t : -1;
+        }
+        f4v xst[MW_XS], gst[MW_GS]; // plain vectors: they must stay in registers
+        auto chunk_load = [&](int n, int oh0) {
+            const float *Xn = X + (int64_t)n * d.IC * d.H * d.W;
+            const int hbase = oh0 * d.sH - d.pH;
+#pragma unroll
+            for (int i = 0; i < MW_XS; i++)
+            {
+                const int h = hbase + x_hr[i];
+                const bool ok = h >= 0 && h < d.H;
+                const int hc = h < 0 ? 0 : (h >= d.H ? d.H - 1 : h);
+                const float *p = Xn + x_goff[i] + hc * d.W;
+                f4v v;
+                if (xvec)
+                    v = *reinterpret_cast<const f4v *>(p); // W % 4 == 0: whole float4 inside the row
+                else
+                {
+                    v.x = p[0];
+                    v.y = x_w[i] + 1 < d.W ? p[1] : 0.0f;
+                    v.z = x_w[i] + 2 < d.W ? p[2] : 0.0f;
+                    v.w = x_w[i] + 3 < d.W ? p[3] : 0.0f;
+                }
+                xst[i].x = ok ? v.x : 0.0f;
+                xst[i].y = ok ? v.y : 0.0f;
+                xst[i].z = ok ? v.z : 0.0f;
+                xst[i].w = ok ? v.w : 0.0f;
+            }
+            const char *Gn = reinterpret_cast<const char *>(GO + (((int64_t)n * d.OC + oc0) * d.OH + oh0) * d.OW);
+#pragma unroll
+            for (int i = 0; i < MW_GS; i++)
+                gst[i] = *reinterpret_cast<const f4v *>(Gn + g_goff[i]);
+        };
+        auto stage_store = [&](int buf) {
+            float *base = lds + buf * bufsz;
+#pragma unroll
+            for (int i = 0; i < MW_XS; i++)
+                if (x_loff[i] >= 0)
+                {
+                    float *p = base + x_loff[i];
+                    p[0] = xst[i].x;
+                    p[1] = xst[i].y;
+                    p[2] = xst[i].z;
+                    p[3] = xst[i].w;
+                }
+#pragma unroll
+            for (int i = 0; i < MW_GS; i++)
+                if (g_loff[i] >= 0)
+                    *reinterpret_cast<f4v *>(base + g_loff[i]) = gst[i];
+        };
+        int n1 = 0, oh1 = 0; // the chunk the next chunk_load fetches
+        auto advance = [&]() {
+            oh1 += R;
+            if (oh1 >= d.OH)
+            {
+                oh1 = 0;
+                n1++;
+            }
+        };
+        if (nchunks > 0)
+        {
+            chunk_load(n1, oh1);
+            advance();
+            stage_store(0);
+        }
+        if (nchunks > 1)
+        {
+            chunk_load(n1, oh1);
+            advance();
+        }
+        __syncthreads();
+        for (int c = 0; c < nchunks; c++)
+        {
+            // registers hold chunk c + 1; buffer (c + 1) & 1 was last read in iteration c - 1
+            if (c + 1 < nchunks)
+                stage_store((c + 1) & 1);
+            if (c + 2 < nchunks)
+            {
+                chunk_load(n1, oh1);
+                advance();
+            }
+            __syncthreads();
+        }
+        return;
+    }
+
+    // ---- computing waves ----
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col = c0 + (lane & 15);
+    const int colc = col < NC ? col : NC - 1;
+    const int ic = colc / KHW;
+    const int rem = colc - ic * KHW;
+    const int kh = rem / d.KW, kw = rem - kh * d.KW;
+    const int q = lane >> 4;
+    const int sW = UNIT ? 1 : d.sW;
+    const int a_lane = 64 + (wave * 16 + (lane & 15)) * GP + q; // 64 zero words lead each buffer
+    const int x_lane = xoff + (ic - ic_first) * CP + kh * Wp + kw + q * sW;
+    const int npieces = R * NP;
+
+    f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    __syncthreads(); // chunk 0 is staged
+    for (int c = 0; c < nchunks; c++)
+    {
+        const int buf = c & 1;
+        const float *ab = lds + buf * bufsz + a_lane;
+        const float *xb = lds + buf * bufsz + x_lane;
+        // A piece is QP consecutive instructions of an output row.  The operands of the next
+        // piece are read before the current one runs.  The loop is free of conditions so that
+        // the reads stay where they are written: an odd number of pieces is made even by a
+        // dummy piece whose grad_output operand comes from the 64 zero words in front of the
+        // buffer (products of zero only matter to results that are recomputed anyway).
+        const float *zb = lds + buf * bufsz + q;
+        int rr = 0, rp = 0; // piece the next read fetches (row, piece of the row)
+        auto read_piece = [&](float (&a)[QP], float (&b)[QP]) {
+            const bool dummy = rr >= R;
+            const int xr = dummy ? 0 : rr;
+            const float *ap = dummy ? zb : ab + rr * OWp + 4 * QP * rp;
+            const float *xp = xb + xr * d.sH * Wp + 4 * QP * rp * sW;
+#pragma unroll
+            for (int u = 0; u < QP; u++)
+            {
+                a[u] = ap[4 * u];
+                b[u] = xp[4 * u * sW];
+            }
+            if (++rp == NP)
+            {
+                rp = 0;
+                rr++;
+            }
+        };
+        auto run_piece = [&](const float (&a)[QP], const float (&b)[QP]) {
+#pragma unroll
+            for (int u = 0; u < QP; u++)
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u], b[u], acc, 0, 0, 0);
+        };
+        float a0[QP], b0[QP], a1[QP], b1[QP];
+        read_piece(a0, b0);
+        for (int p = 0; p < npieces; p += 2)
+        {
+            read_piece(a1, b1);
+            run_piece(a0, b0);
+            read_piece(a0, b0);
+            run_piece(a1, b1);
+        }
+        __syncthreads();
+    }
+    // register r of the block: oc 4*(lane/16) + r of the wave's 16, column lane%16
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+    {
+        const int oc = oc0 + wave * 16 + 4 * q + r;
+        if (oc < d.OC && col < NC)
+        {
+            float v = acc[r];
+            if (((__float_as_uint(v) << 1) == 0u) || (v != v))
+                v = conv2d_grad_kernel_exact(GO, X, d, oc, ic, kh, kw);
+            GK[(int64_t)oc * NC + col] = v;
+        }
+    }
+}
+
 inline bool fits_i32(int64_t v) { return v >= 0 && v <= REPDL_I32_MAX; }
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
@@ -835,16 +1177,23 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
     const int wvec = MODE == MODE_FWD && aligned16(kernel) && (K % 4 == 0);
     const int ovec = aligned16(out) && (P % 4 == 0);
     hipStream_t s = repdl_stream(stream);
+    const bool mfma = repdl_mfma_exact();
     if (M <= 64)
     {
         dim3 grid((unsigned)gx, (unsigned)repdl_cdiv(M, 64), (unsigned)gz);
-        hipLaunchKernelGGL((conv_gemm_kernel<64, MODE>), grid, dim3(128), 0, s, gathered, kernel, out, d, wvec, ovec);
+        if (mfma)
+            hipLaunchKernelGGL((conv_gemm_kernel<64, MODE, true>), grid, dim3(128), 0, s, gathered, kernel, out, d, wvec, ovec);
+        else
+            hipLaunchKernelGGL((conv_gemm_kernel<64, MODE, false>), grid, dim3(128), 0, s, gathered, kernel, out, d, wvec, ovec);
     }
     else
     {
         dim3 grid((unsigned)gx, (unsigned)repdl_cdiv(M, 128), (unsigned)gz);
         REPDL_REQUIRE(grid.y <= 65535);
-        hipLaunchKernelGGL((conv_gemm_kernel<128, MODE>), grid, dim3(256), 0, s, gathered, kernel, out, d, wvec, ovec);
+        if (mfma)
+            hipLaunchKernelGGL((conv_gemm_kernel<128, MODE, true>), grid, dim3(256), 0, s, gathered, kernel, out, d, wvec, ovec);
+        else
+            hipLaunchKernelGGL((conv_gemm_kernel<128, MODE, false>), grid, dim3(256), 0, s, gathered, kernel, out, d, wvec, ovec);
     }
     return repdl_launch_status();
 }
@@ -909,6 +1258,94 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
     ConvDims d{(int)N, (int)IC, (int)H, (int)W, (int)OC, (int)KH, (int)KW, (int)OH,
                (int)OW, (int)sH, (int)sW, (int)pH, (int)pW, 1};
     hipStream_t s = repdl_stream(stream);
+
+    // Matrix-instruction kernel: geometry of a chunk (see conv_wgrad_mfma_kernel).
+    if (repdl_mfma_exact() && OW % 4 == 0 && sW <= 16 && aligned16(grad_output))
+    {
+        const int64_t KHW = KH * KW, NC = IC * KHW;
+        // instructions per piece: the largest candidate that divides a row of OW / 4 instructions
+        const int64_t nqr = OW / 4;
+        int64_t QP = 0, NP = 0;
+        for (int64_t qp : {16, 14, 7, 4})
+            if (QP == 0 && nqr % qp == 0)
+            {
+                QP = qp;
+                NP = nqr / qp;
+            }
+        const int64_t OWp = 4 * QP * NP;
+        int64_t Wp = pW + (W + 3) / 4 * 4;
+        const int64_t reach = (OWp - 1) * sW + KW; // the taps of the padded steps must be staged zeros
+        if (reach > Wp)
+            Wp = reach;
+        while (Wp % 32 != KW % 32)
+            Wp++;
+        const int64_t span = (15 + KHW - 1) / KHW + 1; // channels a 16-column block can span
+        const int64_t nic_max = span < IC ? span : IC;
+        const int64_t nw4 = (W + 3) / 4;
+        int64_t R = 0, hrows = 0, GP = 0, CP = 0;
+        for (int64_t r = OH; r >= 1 && QP > 0; r--)
+        {
+            if (OH % r != 0)
+                continue; // whole chunks only
+            const int64_t hr = (r - 1) * sH + KH;
+            int64_t gp = r * OWp;
+            while (gp % 32 != 4)
+                gp++;
+            int64_t cp = hr * Wp;
+            while (cp % 32 != KHW % 32)
+                cp++;
+            if (MW_OC * r * OW <= 4 * MW_ST * MW_GS && nic_max * hr * nw4 <= MW_ST * MW_XS &&
+                2 * (64 + MW_OC * gp + nic_max * cp + 3) * 4 <= 150 * 1024)
+            {
+                R = r;
+                hrows = hr;
+                GP = gp;
+                CP = cp;
+                break;
+            }
+        }
+        if (R > 0 && N * (OH / R) <= REPDL_I32_MAX)
+        {
+            const int64_t xoff = 64 + MW_OC * GP; // 64 zero words, then the grad_output rows, then the input rows
+            const int64_t bufsz = (xoff + nic_max * CP + 3) / 4 * 4; // float4 stores into either buffer
+            const int xvec = aligned16(input) && (W % 4 == 0);
+            const int64_t gx = repdl_cdiv(NC, 16), gy = repdl_cdiv(OC, MW_OC);
+            REPDL_REQUIRE(fits_i32(gx) && gy <= 65535);
+            size_t shmem = (size_t)(2 * bufsz * 4);
+            if (shmem < 84 * 1024)
+                shmem = 84 * 1024; // one workgroup per CU: every wave has a SIMD to itself
+#define REPDL_WGRAD_MFMA(Q, U)                                                                                     \
+    do                                                                                                            \
+    {                                                                                                             \
+        hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_wgrad_mfma_kernel<Q, U>),        \
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);              \
+        if (e_ != hipSuccess)                                                                                     \
+            return (int)e_;                                                                                       \
+        hipLaunchKernelGGL((conv_wgrad_mfma_kernel<Q, U>), dim3((unsigned)gx, (unsigned)gy), dim3(256), shmem, s, \
+                           grad_output, input, grad_kernel, d, (int)R, (int)NP, (int)GP, (int)Wp, (int)CP,        \
+                           (int)hrows, (int)xoff, (int)bufsz, xvec);                                              \
+    } while (0)
+#define REPDL_WGRAD_MFMA_Q(Q)          \
+    do                                 \
+    {                                  \
+        if (sW == 1)                   \
+            REPDL_WGRAD_MFMA(Q, true); \
+        else                           \
+            REPDL_WGRAD_MFMA(Q, false); \
+    } while (0)
+            if (QP == 16)
+                REPDL_WGRAD_MFMA_Q(16);
+            else if (QP == 14)
+                REPDL_WGRAD_MFMA_Q(14);
+            else if (QP == 7)
+                REPDL_WGRAD_MFMA_Q(7);
+            else
+                REPDL_WGRAD_MFMA_Q(4);
+#undef REPDL_WGRAD_MFMA_Q
+#undef REPDL_WGRAD_MFMA
+            return repdl_launch_status();
+        }
+    }
 
     // Geometry.  A row of OW outputs is cut into NP pieces of PIECE (16/32/64) steps;
     // steps past the end of the row must read zeros, so the staged row pitch Wp covers
