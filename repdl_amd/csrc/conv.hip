@@ -1113,36 +1113,45 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
         // buffer (products of zero only matter to results that are recomputed anyway).
         const float *zb = lds + buf * bufsz + q;
         int rr = 0, rp = 0; // piece the next read fetches (row, piece of the row)
-        auto read_piece = [&](float (&a)[QP], float (&b)[QP]) {
+        const float *ap, *xp;
+        auto next_piece = [&]() {
             const bool dummy = rr >= R;
             const int xr = dummy ? 0 : rr;
-            const float *ap = dummy ? zb : ab + rr * OWp + 4 * QP * rp;
-            const float *xp = xb + xr * d.sH * Wp + 4 * QP * rp * sW;
-#pragma unroll
-            for (int u = 0; u < QP; u++)
-            {
-                a[u] = ap[4 * u];
-                b[u] = xp[4 * u * sW];
-            }
+            ap = dummy ? zb : ab + rr * OWp + 4 * QP * rp;
+            xp = xb + xr * d.sH * Wp + 4 * QP * rp * sW;
             if (++rp == NP)
             {
                 rp = 0;
                 rr++;
             }
         };
-        auto run_piece = [&](const float (&a)[QP], const float (&b)[QP]) {
+        // runs the piece in (ca, cb) and reads the next one into (na, nb): one pair of reads
+        // behind every instruction, pinned there (left alone, the scheduler moves the reads
+        // behind the last instructions of the piece, too late for the next one)
+        auto step_piece = [&](const float (&ca)[QP], const float (&cb)[QP], float (&na)[QP], float (&nb)[QP]) {
+            next_piece();
 #pragma unroll
             for (int u = 0; u < QP; u++)
-                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u], b[u], acc, 0, 0, 0);
+            {
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ca[u], cb[u], acc, 0, 0, 0);
+                na[u] = ap[4 * u];
+                nb[u] = xp[4 * u * sW];
+                __builtin_amdgcn_sched_barrier(0);
+            }
         };
         float a0[QP], b0[QP], a1[QP], b1[QP];
-        read_piece(a0, b0);
+        next_piece();
+#pragma unroll
+        for (int u = 0; u < QP; u++)
+        {
+            a0[u] = ap[4 * u];
+            b0[u] = xp[4 * u * sW];
+        }
+        __builtin_amdgcn_sched_barrier(0);
         for (int p = 0; p < npieces; p += 2)
         {
-            read_piece(a1, b1);
-            run_piece(a0, b0);
-            read_piece(a0, b0);
-            run_piece(a1, b1);
+            step_piece(a0, b0, a1, b1);
+            step_piece(a1, b1, a0, b0);
         }
         __syncthreads();
     }

@@ -445,6 +445,193 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_kernel(const float *__r
         }
 }
 
+// The same kernel for the common case that needs no bounds checks: M, N multiples of the
+// tile, K a multiple of BK, 16-byte aligned operands.  While a matrix instruction runs, its
+// SIMD issues no vector ALU instruction of any wave (measured), so address arithmetic in the
+// loop costs matrix time one for one.  Here the loop has none: a global load is a uniform
+// base (advanced per k-tile on the scalar unit) plus a per-thread byte offset that never
+// changes; LDS addresses are per-thread constants plus the buffer offset plus immediates.
+template <bool TA, bool TB, int FM, int FN, int WGM, int WGN>
+__global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_fast_kernel(const float *__restrict__ A,
+                                                                     const float *__restrict__ B,
+                                                                     float *__restrict__ C, int64_t M, int64_t N,
+                                                                     int64_t K, int64_t gx, int64_t gy, int64_t ntiles8)
+{
+    constexpr int NTH = 64 * WGM * WGN;
+    constexpr int TM = 32 * FM * WGM, TN = 32 * FN * WGN;
+    constexpr int LDA_ = TM + 4, LDB_ = TN + 4;
+    constexpr int NVA = TM * BK / 4 / NTH, NVB = TN * BK / 4 / NTH;
+    constexpr bool A_KC = !TA, B_KC = TB;
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    float *const As = smem;                 // [2][BK * LDA_]
+    float *const Bs = smem + 2 * BK * LDA_; // [2][BK * LDB_]
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave % WGM, wn = wave / WGM;
+    const int l32 = lane & 31, half = lane >> 5;
+
+    int64_t tile = blockIdx.x;
+    if (tile < ntiles8)
+        tile = (tile & 7) * (ntiles8 >> 3) + (tile >> 3);
+    const int64_t group_sz = (int64_t)GROUP_M * gx;
+    const int64_t group = tile / group_sz;
+    const int64_t first_row = group * GROUP_M;
+    const int64_t rows_here = (gy - first_row < GROUP_M) ? gy - first_row : GROUP_M;
+    const int64_t in_group = tile - group * group_sz;
+    const int64_t trow = first_row + in_group % rows_here, tcol = in_group / rows_here;
+    const int64_t m0 = trow * TM, n0 = tcol * TN;
+    const int64_t lda = TA ? M : K, ldb = TB ? K : N;
+
+    // per-thread constants: byte offset of each float4 slot inside the operand tile, and the
+    // LDS word it goes to
+    uint32_t a_voff[NVA], b_voff[NVB];
+    int a_st[NVA], b_st[NVB];
+#pragma unroll
+    for (int i = 0; i < NVA; i++)
+    {
+        const int idx = tid + NTH * i;
+        if (A_KC)
+        {
+            const int r = idx >> 2, k = (idx & 3) << 2;
+            a_voff[i] = (uint32_t)((int64_t)r * lda + k) * 4u;
+            a_st[i] = k * LDA_ + r;
+        }
+        else
+        {
+            const int k = idx / (TM / 4), r = (idx % (TM / 4)) * 4;
+            a_voff[i] = (uint32_t)((int64_t)k * lda + r) * 4u;
+            a_st[i] = k * LDA_ + r;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NVB; i++)
+    {
+        const int idx = tid + NTH * i;
+        if (B_KC)
+        {
+            const int r = idx >> 2, k = (idx & 3) << 2;
+            b_voff[i] = (uint32_t)((int64_t)r * ldb + k) * 4u;
+            b_st[i] = k * LDB_ + r;
+        }
+        else
+        {
+            const int k = idx / (TN / 4), r = (idx % (TN / 4)) * 4;
+            b_voff[i] = (uint32_t)((int64_t)k * ldb + r) * 4u;
+            b_st[i] = k * LDB_ + r;
+        }
+    }
+    // uniform tile bases, advanced by one k-tile per iteration
+    const char *a_base = reinterpret_cast<const char *>(A_KC ? A + m0 * lda : A + m0);
+    const char *b_base = reinterpret_cast<const char *>(B_KC ? B + n0 * ldb : B + n0);
+    const int64_t a_step = (A_KC ? (int64_t)BK : (int64_t)BK * lda) * 4;
+    const int64_t b_step = (B_KC ? (int64_t)BK : (int64_t)BK * ldb) * 4;
+
+    f16v acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[i][j][r] = 0.0f;
+
+    v4f fa[NVA], fb[NVB];
+    auto load_tiles = [&]() {
+#pragma unroll
+        for (int i = 0; i < NVA; i++)
+            fa[i] = *reinterpret_cast<const v4f *>(a_base + a_voff[i]);
+#pragma unroll
+        for (int i = 0; i < NVB; i++)
+            fb[i] = *reinterpret_cast<const v4f *>(b_base + b_voff[i]);
+        a_base += a_step;
+        b_base += b_step;
+    };
+    auto store_tiles = [&](int buf) {
+        float *as = As + buf * BK * LDA_, *bs = Bs + buf * BK * LDB_;
+#pragma unroll
+        for (int i = 0; i < NVA; i++)
+        {
+            if (A_KC)
+            {
+                as[a_st[i] + 0 * LDA_] = fa[i][0];
+                as[a_st[i] + 1 * LDA_] = fa[i][1];
+                as[a_st[i] + 2 * LDA_] = fa[i][2];
+                as[a_st[i] + 3 * LDA_] = fa[i][3];
+            }
+            else
+                *reinterpret_cast<v4f *>(&as[a_st[i]]) = fa[i];
+        }
+#pragma unroll
+        for (int i = 0; i < NVB; i++)
+        {
+            if (B_KC)
+            {
+                bs[b_st[i] + 0 * LDB_] = fb[i][0];
+                bs[b_st[i] + 1 * LDB_] = fb[i][1];
+                bs[b_st[i] + 2 * LDB_] = fb[i][2];
+                bs[b_st[i] + 3 * LDB_] = fb[i][3];
+            }
+            else
+                *reinterpret_cast<v4f *>(&bs[b_st[i]]) = fb[i];
+        }
+    };
+    const int a_off = half * LDA_ + wm * 32 * FM + l32;
+    const int b_off = half * LDB_ + wn * 32 * FN + l32;
+    auto compute = [&](int buf) {
+        const float *as = As + buf * BK * LDA_ + a_off, *bs = Bs + buf * BK * LDB_ + b_off;
+        float a[BK / 2][FM], b[BK / 2][FN];
+#pragma unroll
+        for (int kp = 0; kp < BK / 2; kp++)
+        {
+#pragma unroll
+            for (int i = 0; i < FM; i++)
+                a[kp][i] = as[2 * kp * LDA_ + 32 * i];
+#pragma unroll
+            for (int j = 0; j < FN; j++)
+                b[kp][j] = bs[2 * kp * LDB_ + 32 * j];
+        }
+#pragma unroll
+        for (int kp = 0; kp < BK / 2; kp++)
+#pragma unroll
+            for (int i = 0; i < FM; i++)
+#pragma unroll
+                for (int j = 0; j < FN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kp][i], b[kp][j], acc[i][j], 0, 0, 0);
+    };
+
+    const int64_t nkt = K / BK;
+    if (nkt > 0)
+    {
+        load_tiles();
+        store_tiles(0);
+    }
+    __syncthreads();
+    for (int64_t kt = 0; kt < nkt; kt++)
+    {
+        const int cur = (int)(kt & 1);
+        const bool more = kt + 1 < nkt;
+        if (more)
+            load_tiles();
+        compute(cur);
+        if (more)
+            store_tiles(cur ^ 1);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+        {
+            const int64_t m = m0 + wm * 32 * FM + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3);
+#pragma unroll
+            for (int j = 0; j < FN; j++)
+                C[m * N + n0 + wn * 32 * FN + 32 * j + l32] = acc[i][j][r];
+        }
+}
+
 template <bool TA, bool TB, int FM, int FN, int WGM, int WGN>
 int launch_mfma_t(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int avec, int bvec,
                   hipStream_t s)
@@ -455,6 +642,24 @@ int launch_mfma_t(const float *A, const float *B, float *C, int64_t M, int64_t N
     if (gx * gy > REPDL_I32_MAX)
         return REPDL_E_ARG;
     const int64_t ntiles8 = (gx * gy) & ~(int64_t)7;
+    const int64_t lda = TA ? M : K, ldb = TB ? K : N;
+    // no bounds checks needed, and every in-tile byte offset fits 32 bits
+    const bool regular = M % TM == 0 && N % TN == 0 && K % BK == 0 && avec && bvec &&
+                         (int64_t)(TM + BK) * lda * 4 < (1LL << 32) && (int64_t)(TN + BK) * ldb * 4 < (1LL << 32);
+    if (regular)
+    {
+        auto kern = &mm_mfma_fast_kernel<TA, TB, FM, FN, WGM, WGN>;
+        if (shmem > 48 * 1024)
+        {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+            if (e != hipSuccess)
+                return (int)e;
+        }
+        hipLaunchKernelGGL(kern, dim3((unsigned)(gx * gy)), dim3(64 * WGM * WGN), shmem, s, A, B, C, M, N, K, gx, gy,
+                           ntiles8);
+        return repdl_launch_status();
+    }
     auto kern = &mm_mfma_kernel<TA, TB, FM, FN, WGM, WGN>;
     if (shmem > 48 * 1024)
     {
