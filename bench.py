@@ -36,7 +36,7 @@ HBM_PEAK_GBS = 8000.0
 # reads 524300 for 1 GiB (factor 1.99995 KiB per count), WRITE_SIZE 1048576 (factor 1.0).  Summary:
 # profiles/hbm_traffic_counters.txt.  Valid for the default workload sizes only.
 MEASURED_TRAFFIC_BYTES = {
-    "mm": 3441648 * 1.99995 * 1024 + 262171 * 1024,       # 7.3e9: operand panels re-read through L2 misses
+    "mm": None,
     "exp": 524338 * 1.99995 * 1024 + 1048577 * 1024,      # 2.147e9 = the algorithmic 8 B/element
     "sum2d_dim1": 524392 * 1.99995 * 1024 + 64 * 1024,    # 1.074e9 = the algorithmic 4 B/element
 }
@@ -120,7 +120,7 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 1
     import repdl_amd
-    from repdl_amd import ops
+    from repdl_amd import _lib, ops
 
     from oracle import api as oracle  # checker / baseline legs only
     from oracle import ref as oracle_ref
@@ -176,6 +176,14 @@ def main() -> int:
     }
     del x_d, w_d, y_gpu, out_holder
 
+    if _lib.lib().repdl_hip_matrix_path() == 1:
+        kernel_name = "mm_mfma_fast_kernel<NT, 256x256x16 tile, 512 threads>"
+        kernel_note = ("fp32 matrix-instruction peak; v_mfma_f32_32x32x2_f32, checked on this device to be a "
+                       "k-ascending chain of single-rounding FMAs before use")
+    else:
+        kernel_name = "mm_kernel<NT>"
+        kernel_note = ("fp32 compute peak; the matrix-instruction check failed on this device, so the kernel issues "
+                       "v_fma_f32 only, whose issue-rate ceiling is half of this peak")
     result = {
         "metric": "bit-exact fp32 mm GFLOP/s at 8192^3",
         "value": round(gflops, 1),
@@ -193,10 +201,9 @@ def main() -> int:
                    "device": props.name, "cus": props.multi_processor_count},
         "roofline": {"bound": "mfma", "achieved": round(kern_tflops, 3), "peak": FP32_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(kern_tflops / FP32_PEAK_TFLOPS, 4),
-                     "traffic": round(MEASURED_TRAFFIC_BYTES["mm"]) if S == 8192 else None,
-                     "kernel": "mm_kernel<NT>", "kernel_ms": round(ev_ms, 4), "kernel_ms_min": round(ev_min, 4),
-                     "note": "fp32 compute peak; the kernel issues scalar v_fma_f32 only (no MFMA, packed "
-                             "fp32 disabled), whose issue-rate ceiling is half of this peak"},
+                     "traffic": round(MEASURED_TRAFFIC_BYTES["mm"]) if S == 8192 and MEASURED_TRAFFIC_BYTES["mm"] else None,
+                     "kernel": kernel_name, "kernel_ms": round(ev_ms, 4), "kernel_ms_min": round(ev_min, 4),
+                     "note": kernel_note},
         "cpu_baseline": cpu_baseline,
         "parity": parity,
         "also": [],
