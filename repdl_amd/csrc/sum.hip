@@ -44,7 +44,7 @@ __global__ __launch_bounds__(RT) void rowchain_kernel(const float *__restrict__ 
     constexpr int RLD = RC + 4;    // padded LDS row: keeps 16-byte alignment, shifts banks by 4
     constexpr int C4 = RC / 4;     // float4 per tile row
     constexpr int RV = RTILE / 4 / RT; // float4 per thread and tile
-    __shared__ __attribute__((aligned(16))) float tile[RR * RLD];
+    __shared__ __attribute__((aligned(16))) float tile[RR * RLD + 64]; // + 64: the walk reads ahead past the last row
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int walker = blockIdx.x % (RT / 64);
@@ -106,23 +106,48 @@ __global__ __launch_bounds__(RT) void rowchain_kernel(const float *__restrict__ 
             const int64_t sgm = t / tiles_per_seg, c0 = (t - sgm * tiles_per_seg) * RC;
             const int64_t rem = seglen - c0;
             const float *row = &tile[lane * RLD];
-            if (rem >= RC)
+            // 8*WB elements per step, the next ones read from LDS before the adds of the current
+            // ones: with few chains per workgroup the walk is the critical path, and it should
+            // cost one dependent v_add_f32 per element and little else.  Elements past the end
+            // of a short tile are walked one by one (they must not be added at all: -0 + 0 = +0).
+            constexpr int WB = RC < 64 ? RC / 8 : 8; // float4 per half step
+            const int here = rem >= RC ? RC : (int)rem;
+            const int nfull = here - here % (8 * WB);
+            if (nfull > 0)
             {
-#pragma unroll 8
-                for (int c = 0; c < RC; c += 4)
+                v4f va[WB], vb[WB];
+#pragma unroll
+                for (int u = 0; u < WB; u++)
+                    va[u] = *reinterpret_cast<const v4f *>(&row[4 * u]);
+                for (int c = 0; c < nfull; c += 8 * WB)
                 {
-                    const v4f v = *reinterpret_cast<const v4f *>(&row[c]);
-                    acc = acc + v.x;
-                    acc = acc + v.y;
-                    acc = acc + v.z;
-                    acc = acc + v.w;
+#pragma unroll
+                    for (int u = 0; u < WB; u++)
+                        vb[u] = *reinterpret_cast<const v4f *>(&row[c + 4 * WB + 4 * u]);
+#pragma unroll
+                    for (int u = 0; u < WB; u++)
+                    {
+                        acc = acc + va[u].x;
+                        acc = acc + va[u].y;
+                        acc = acc + va[u].z;
+                        acc = acc + va[u].w;
+                    }
+                    // the last step reads 4*WB floats past the row: inside the tile or its pad
+#pragma unroll
+                    for (int u = 0; u < WB; u++)
+                        va[u] = *reinterpret_cast<const v4f *>(&row[c + 8 * WB + 4 * u]);
+#pragma unroll
+                    for (int u = 0; u < WB; u++)
+                    {
+                        acc = acc + vb[u].x;
+                        acc = acc + vb[u].y;
+                        acc = acc + vb[u].z;
+                        acc = acc + vb[u].w;
+                    }
                 }
             }
-            else
-            {
-                for (int c = 0; c < (int)rem; c++)
-                    acc = acc + row[c];
-            }
+            for (int c = nfull; c < here; c++)
+                acc = acc + row[c];
         }
         __syncthreads(); // the walk of tile t is over: the buffer may be overwritten
         if (more)
@@ -134,34 +159,113 @@ __global__ __launch_bounds__(RT) void rowchain_kernel(const float *__restrict__ 
 }
 
 // ---------------------------------------------------------------------------
-// Column chains: out[j] = chain over i of in[i*N + j] (sum2d_dim0).  One lane
-// per column, rows consumed in order; loads are issued UNROLL rows ahead.
+// Column chains: out[j] = chain over i of in[i*N + j] (sum2d_dim0).  Same scheme
+// as the row chains, turned: a workgroup owns CW adjacent columns (64, 32 or 16,
+// fewer when columns are scarce so that the CUs still get several workgroups each)
+// and moves down in tiles of (RTILE / CW) rows x CW columns = 32 KiB.  All waves
+// stream the next tile into registers (16-byte non-temporal loads; a row of the
+// tile is CW*4 contiguous bytes) while one wave walks the current tile in LDS,
+// lane = column, one ds_read_b32 and one dependent v_add_f32 per row.
 // ---------------------------------------------------------------------------
-constexpr int CU_UNROLL = 16;
-
-__global__ __launch_bounds__(64) void colchain_kernel(const float *__restrict__ in,
-                                                      float *__restrict__ out, int64_t M, int64_t N,
-                                                      float factor)
+template <int CW, bool VEC>
+__global__ __launch_bounds__(256) void coltile_kernel(const float *__restrict__ in, float *__restrict__ out,
+                                                      int64_t M, int64_t N, float factor)
 {
-    const int64_t j = (int64_t)blockIdx.x * 64 + threadIdx.x;
-    if (j >= N)
-        return;
-    const float *p = in + j;
+    constexpr int TR = RTILE / CW;      // rows per tile
+    constexpr int C4 = CW / 4;          // float4 per tile row
+    constexpr int RV = RTILE / 4 / 256; // float4 per thread and tile
+    __shared__ __attribute__((aligned(16))) float tile[RTILE];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int walker = blockIdx.x % 4;
+    const int64_t col0 = (int64_t)blockIdx.x * CW;
+    const int64_t ntiles = (M + TR - 1) / TR;
+
     float acc = 0.0f;
-    int64_t i = 0;
-    for (; i + CU_UNROLL <= M; i += CU_UNROLL)
+    v4f stage[RV];
+    auto load = [&](int64_t t) {
+#pragma unroll
+        for (int i = 0; i < RV; i++)
+        {
+            const int idx = tid + 256 * i;
+            const int64_t r = t * TR + idx / C4;
+            const int64_t c = col0 + ((idx % C4) << 2);
+            v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (r < M)
+            {
+                const float *p = in + r * N + c;
+                if (VEC && c + 3 < N)
+                    v = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(p));
+                else
+                {
+                    if (c + 0 < N) v.x = p[0];
+                    if (c + 1 < N) v.y = p[1];
+                    if (c + 2 < N) v.z = p[2];
+                    if (c + 3 < N) v.w = p[3];
+                }
+            }
+            stage[i] = v;
+        }
+    };
+    auto store = [&]() {
+#pragma unroll
+        for (int i = 0; i < RV; i++)
+            *reinterpret_cast<v4f *>(&tile[(tid + 256 * i) << 2]) = stage[i]; // [row][column], CW floats per row
+    };
+
+    if (ntiles > 0)
     {
-        float v[CU_UNROLL];
-#pragma unroll
-        for (int u = 0; u < CU_UNROLL; u++)
-            v[u] = p[(i + u) * N];
-#pragma unroll
-        for (int u = 0; u < CU_UNROLL; u++)
-            acc = acc + v[u];
+        load(0);
+        store();
     }
-    for (; i < M; i++)
-        acc = acc + p[i * N];
-    out[j] = factor * acc;
+    __syncthreads();
+    for (int64_t t = 0; t < ntiles; t++)
+    {
+        const bool more = t + 1 < ntiles;
+        if (more)
+            load(t + 1);
+        if (wave == walker && lane < CW)
+        {
+            const int64_t rem = M - t * TR; // rows of this tile that exist; the rest must not be added
+            const float *colp = &tile[lane];
+            if (rem >= TR)
+            {
+                float va[16], vb[16];
+#pragma unroll
+                for (int u = 0; u < 16; u++)
+                    va[u] = colp[u * CW];
+                for (int r = 0; r < TR; r += 32)
+                {
+#pragma unroll
+                    for (int u = 0; u < 16; u++)
+                        vb[u] = colp[(r + 16 + u) * CW];
+#pragma unroll
+                    for (int u = 0; u < 16; u++)
+                        acc = acc + va[u];
+                    if (r + 32 < TR)
+                    {
+#pragma unroll
+                        for (int u = 0; u < 16; u++)
+                            va[u] = colp[(r + 32 + u) * CW];
+                    }
+#pragma unroll
+                    for (int u = 0; u < 16; u++)
+                        acc = acc + vb[u];
+                }
+            }
+            else
+            {
+                for (int r = 0; r < (int)rem; r++)
+                    acc = acc + colp[r * CW];
+            }
+        }
+        __syncthreads(); // the walk of tile t is over: the buffer may be overwritten
+        if (more)
+            store();
+        __syncthreads();
+    }
+    if (wave == walker && lane < CW && col0 + lane < N)
+        out[col0 + lane] = factor * acc;
 }
 } // namespace
 
@@ -230,9 +334,27 @@ REPDL_API int repdl_hip_sum2d_dim0(const float *in, float *out, int64_t M, int64
     REPDL_REQUIRE(M >= 0 && N >= 0 && (N == 0 || out != nullptr) && (M * N == 0 || in != nullptr));
     if (N == 0)
         return REPDL_OK;
-    const int64_t grid = repdl_cdiv(N, 64);
+    const bool vec = (reinterpret_cast<uintptr_t>(in) & 15) == 0 && N % 4 == 0;
+    const int cw = N >= 65536 ? 64 : N >= 8192 ? 32 : 16; // 32 columns = one 128-byte line per row
+    const int64_t grid = repdl_cdiv(N, cw);
     REPDL_REQUIRE(grid <= REPDL_I32_MAX);
-    hipLaunchKernelGGL(colchain_kernel, dim3((unsigned)grid), dim3(64), 0, repdl_stream(stream), in, out, M,
-                       N, repdl_sum_factor(average, M));
+    const dim3 g((unsigned)grid);
+    hipStream_t st = repdl_stream(stream);
+    const float factor = repdl_sum_factor(average, M);
+#define REPDL_COLTILE(CWv)                                                                               \
+    do                                                                                                  \
+    {                                                                                                   \
+        if (vec)                                                                                        \
+            hipLaunchKernelGGL((coltile_kernel<CWv, true>), g, dim3(256), 0, st, in, out, M, N, factor); \
+        else                                                                                            \
+            hipLaunchKernelGGL((coltile_kernel<CWv, false>), g, dim3(256), 0, st, in, out, M, N, factor); \
+    } while (0)
+    if (cw == 64)
+        REPDL_COLTILE(64);
+    else if (cw == 32)
+        REPDL_COLTILE(32);
+    else
+        REPDL_COLTILE(16);
+#undef REPDL_COLTILE
     return repdl_launch_status();
 }
