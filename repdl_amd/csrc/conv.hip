@@ -576,6 +576,239 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_kernel(const float *__restri
 }
 
 // ---------------------------------------------------------------------------
+// Implicit GEMM without address arithmetic in the loop (matrix path, the common
+// shapes).  While a matrix instruction runs, its SIMD issues no vector ALU
+// instruction of any wave, so the index arithmetic and bounds checks of a gather are
+// paid in matrix time.  Here the gathered operand is first copied into a zero-padded
+// workspace tensor ([C][Hp][Wp] per image, by conv_pad_kernel; skipped when there is
+// nothing to pad), after which the element of k-row k at pixel p sits at
+//     image base + tab[k] + pix_off[p]
+// with tab[k] depending only on k = (channel, kh, kw) (a table written once per call
+// by conv_ktab_kernel, read with scalar loads) and pix_off[p] only on the pixel (one
+// per-thread constant).  A load is then: scalar base, constant vector offset.
+//   forward     tab[k] = c*Hp*Wp + kh*Wp + kw,                  pix_off = oh*sH*Wp + ow*sW
+//   grad-input  tab[k] = oc*Hp*Wp + (pH+PT-kh)*Wp + (pW+PL-kw), pix_off = h*Wp + w      (stride 1)
+// The kernel operand of grad-input is a strided gather too: W[(oc*IC + ic)*KHW + kh*KW + kw]
+// = tabA[k] + ic*KHW.  Lanes map to pixels (or input channels), k-rows to instructions,
+// so every table entry is wave-uniform.  Requires K % 16 == 0 and M % BM == 0; pixels
+// past the end of the image repeat the last pixel and are not stored.  The padded
+// zeros play the role of the skipped taps exactly as in conv_gemm_kernel, with the same
+// epilogue.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void conv_pad_kernel(const float *__restrict__ src, float *__restrict__ dst,
+                                                       int64_t total, int H, int W, int Hp, int Wp, int PT, int PL)
+{
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total)
+        return;
+    const int wp = (int)(idx % Wp);
+    const int64_t t = idx / Wp;
+    const int hp = (int)(t % Hp);
+    const int64_t pl = t / Hp;
+    const int h = hp - PT, w = wp - PL;
+    dst[idx] = (h >= 0 && h < H && w >= 0 && w < W) ? src[(pl * H + h) * W + w] : 0.0f;
+}
+
+__global__ __launch_bounds__(256) void conv_ktab_kernel(int *__restrict__ tabB, int *__restrict__ tabA, int K, int KH,
+                                                        int KW, int plane, int Wp, int mode, int IC, int baseH,
+                                                        int baseW)
+{
+    const int k = blockIdx.x * 256 + threadIdx.x;
+    if (k >= K)
+        return;
+    const int KHW = KH * KW;
+    const int c = k / KHW, rem = k - c * KHW;
+    const int kh = rem / KW, kw = rem - kh * KW;
+    if (mode == MODE_FWD)
+        tabB[k] = c * plane + kh * Wp + kw;
+    else
+    {
+        tabB[k] = c * plane + (baseH - kh) * Wp + (baseW - kw);
+        tabA[k] = c * IC * KHW + kh * KW + kw;
+    }
+}
+
+template <int BM, int MODE>
+__global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__restrict__ Gp,   // padded gathered operand
+                                                                const float *__restrict__ Xg,   // the original one (epilogue)
+                                                                const float *__restrict__ Wt, float *__restrict__ Out,
+                                                                ConvDims d, const int *__restrict__ tabB,
+                                                                const int *__restrict__ tabA, int plane, int Wp,
+                                                                int64_t img_stride)
+{
+    constexpr int NT = 2 * BM;
+    constexpr int LDA = BM + 4;
+    constexpr int NKR = BM == 64 ? 16 : 8; // k-rows of the gathered tile per wave
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    __shared__ __attribute__((aligned(16))) float As[2][BK * LDA];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int KHW = d.KH * d.KW;
+    const int ICg = d.IC / d.groups, OCg = d.OC / d.groups;
+    const int M = MODE == MODE_FWD ? OCg : d.IC;
+    const int K = (MODE == MODE_FWD ? ICg : d.OC) * KHW;
+    const int P = MODE == MODE_FWD ? d.OH * d.OW : d.H * d.W;
+    const int PW = MODE == MODE_FWD ? d.OW : d.W;
+    const int n = MODE == MODE_FWD ? blockIdx.z / d.groups : blockIdx.z;
+    const int g = MODE == MODE_FWD ? blockIdx.z % d.groups : 0;
+    const int m0 = blockIdx.y * BM, p0 = blockIdx.x * BN;
+
+    // gathered operand: this lane's pixel, this wave's k-rows
+    const int b_half = BM == 64 ? wave : (wave & 1);
+    const int b_kr0 = BM == 64 ? 0 : 8 * (wave >> 1);
+    const int pix_local = 64 * b_half + lane;
+    const int pixc = p0 + pix_local < P ? p0 + pix_local : P - 1;
+    const int pph = pixc / PW, ppw = pixc - pph * PW;
+    const int pix_off = MODE == MODE_FWD ? pph * d.sH * Wp + ppw * d.sW : pph * Wp + ppw;
+    const float *Gimg = Gp + (int64_t)n * img_stride + (MODE == MODE_FWD ? (int64_t)g * ICg * plane : 0);
+    // kernel operand
+    const float *Wg = MODE == MODE_FWD ? Wt + (int64_t)g * OCg * K : Wt;
+    uint32_t a_voff[2]; // FWD: byte offsets of this thread's two float4 slots in the [BM][K] panel
+    int a_st[2];
+    const int a_half = BM == 64 ? 0 : (wave & 1); // DGRAD: this lane's input channel, this wave's 8 k-rows
+    const int a_kr0 = BM == 64 ? 8 * wave : 8 * (wave >> 1);
+    const int a_m = 64 * a_half + lane;
+    if (MODE == MODE_FWD)
+    {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+        {
+            const int idx = tid + NT * i;
+            const int r = idx >> 2, k4 = (idx & 3) << 2;
+            a_voff[i] = (uint32_t)(r * K + k4) * 4u;
+            a_st[i] = k4 * LDA + r;
+        }
+    }
+    const int a_ch_off = (m0 + a_m) * KHW; // DGRAD
+
+    v4f fa4[2];
+    float fa1[8], fb[NKR];
+    auto load_tiles = [&](int kt) {
+        const int *tb = tabB + kt * BK + b_kr0;
+#pragma unroll
+        for (int j = 0; j < NKR; j++)
+        {
+            const float *rowp = Gimg + tb[j];
+            fb[j] = rowp[pix_off];
+        }
+        if (MODE == MODE_FWD)
+        {
+            const char *ab = reinterpret_cast<const char *>(Wg + (int64_t)m0 * K + kt * BK);
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+                fa4[i] = *reinterpret_cast<const v4f *>(ab + a_voff[i]);
+        }
+        else
+        {
+            const int *ta = tabA + kt * BK + a_kr0;
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+            {
+                const float *wp = Wg + ta[j];
+                fa1[j] = wp[a_ch_off];
+            }
+        }
+    };
+    auto store_tiles = [&](int buf) {
+        float *as = As[buf], *bs = Bs[buf];
+#pragma unroll
+        for (int j = 0; j < NKR; j++)
+            bs[(b_kr0 + j) * LDB + pix_local] = fb[j];
+        if (MODE == MODE_FWD)
+        {
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+            {
+                as[a_st[i] + 0 * LDA] = fa4[i][0];
+                as[a_st[i] + 1 * LDA] = fa4[i][1];
+                as[a_st[i] + 2 * LDA] = fa4[i][2];
+                as[a_st[i] + 3 * LDA] = fa4[i][3];
+            }
+        }
+        else
+        {
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                as[(a_kr0 + j) * LDA + a_m] = fa1[j];
+        }
+    };
+
+    const int l32 = lane & 31, half = lane >> 5;
+    const int wm = BM == 64 ? 0 : (wave & 1), wn = BM == 64 ? wave : (wave >> 1);
+    f16v acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[i][j][r] = 0.0f;
+    const int a_off = half * LDA + wm * 64 + l32, b_off = half * LDB + wn * 64 + l32;
+
+    const int nkt = K / BK;
+    if (nkt > 0)
+    {
+        load_tiles(0);
+        store_tiles(0);
+    }
+    __syncthreads();
+    for (int kt = 0; kt < nkt; kt++)
+    {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < nkt;
+        if (more)
+            load_tiles(kt + 1);
+        const float *as = As[cur] + a_off, *bs = Bs[cur] + b_off;
+        float a[BK / 2][2], b[BK / 2][2];
+#pragma unroll
+        for (int kp = 0; kp < BK / 2; kp++)
+        {
+            a[kp][0] = as[2 * kp * LDA];
+            a[kp][1] = as[2 * kp * LDA + 32];
+            b[kp][0] = bs[2 * kp * LDB];
+            b[kp][1] = bs[2 * kp * LDB + 32];
+        }
+#pragma unroll
+        for (int kp = 0; kp < BK / 2; kp++)
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kp][i], b[kp][j], acc[i][j], 0, 0, 0);
+        if (more)
+            store_tiles(cur ^ 1);
+        __syncthreads();
+    }
+
+    float *Oimg = Out + (int64_t)n * (MODE == MODE_FWD ? d.OC : d.IC) * P;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+        {
+            const int m = m0 + wm * 64 + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3);
+            const int ch = MODE == MODE_FWD ? g * OCg + m : m;
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+            {
+                const int pix = p0 + wn * 64 + 32 * j + l32;
+                if (pix >= P)
+                    continue;
+                float v = acc[i][j][r];
+                if (((__float_as_uint(v) << 1) == 0u) || (v != v))
+                {
+                    const int ph = pix / PW, pw = pix - ph * PW;
+                    v = MODE == MODE_FWD ? conv2d_exact(Xg, Wt, d, n, ch, ph, pw)
+                                         : conv2d_grad_input_exact(Xg, Wt, d, n, ch, ph, pw);
+                }
+                Oimg[(int64_t)ch * P + pix] = v;
+            }
+        }
+}
+
+// ---------------------------------------------------------------------------
 // grad-kernel.  GK[oc][ic][kh][kw] is a chain over k = (n, oh, ow): there are
 // only OC*IC*KH*KW chains and K = N*OH*OW cannot be split, so one LANE owns one
 // chain (one dependent v_fma_f32 per k) and the kernel is shaped to make a k
@@ -1187,6 +1420,48 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
     const int ovec = aligned16(out) && (P % 4 == 0);
     hipStream_t s = repdl_stream(stream);
     const bool mfma = repdl_mfma_exact();
+    // Fast path: whole tiles of channels, whole k-tiles, grad-input only at stride 1.
+    const int bm = M <= 64 ? 64 : 128;
+    if (mfma && K % BK == 0 && M % bm == 0 && (MODE == MODE_FWD || (d.sH == 1 && d.sW == 1)))
+    {
+        const int C = MODE == MODE_FWD ? d.IC : d.OC;                 // channels of the gathered tensor
+        const int GH = MODE == MODE_FWD ? d.H : d.OH, GW = MODE == MODE_FWD ? d.W : d.OW;
+        const int PT = MODE == MODE_FWD ? d.pH : (d.KH - 1 - d.pH > 0 ? d.KH - 1 - d.pH : 0);
+        const int PL = MODE == MODE_FWD ? d.pW : (d.KW - 1 - d.pW > 0 ? d.KW - 1 - d.pW : 0);
+        const int64_t Hp = GH + 2 * (int64_t)PT, Wp = GW + 2 * (int64_t)PL;
+        const int64_t plane = Hp * Wp, img = (int64_t)C * plane;
+        if (img * 4 < (1LL << 31) && (int64_t)M * K * 4 < (1LL << 31))
+        {
+            const bool pad = PT > 0 || PL > 0;
+            const size_t tab_bytes = ((size_t)2 * K * sizeof(int) + 255) / 256 * 256;
+            const size_t ws_bytes = tab_bytes + (pad ? (size_t)d.N * img * sizeof(float) : 0);
+            char *ws = nullptr;
+            hipError_t e = hipMallocAsync(reinterpret_cast<void **>(&ws), ws_bytes, s);
+            if (e != hipSuccess)
+                return (int)e;
+            int *tabB = reinterpret_cast<int *>(ws), *tabA = tabB + K;
+            float *Gp = reinterpret_cast<float *>(ws + tab_bytes);
+            hipLaunchKernelGGL(conv_ktab_kernel, dim3((unsigned)repdl_cdiv(K, 256)), dim3(256), 0, s, tabB, tabA, (int)K,
+                               d.KH, d.KW, (int)plane, (int)Wp, MODE, d.IC, d.pH + PT, d.pW + PL);
+            if (pad)
+            {
+                const int64_t total = (int64_t)d.N * img;
+                hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)repdl_cdiv(total, 256)), dim3(256), 0, s, gathered, Gp,
+                                   total, GH, GW, (int)Hp, (int)Wp, PT, PL);
+            }
+            const float *src = pad ? Gp : gathered;
+            dim3 grid((unsigned)gx, (unsigned)(M / bm), (unsigned)gz);
+            if (bm == 64)
+                hipLaunchKernelGGL((conv_gemm_fast_kernel<64, MODE>), grid, dim3(128), 0, s, src, gathered, kernel, out, d, tabB,
+                                   tabA, (int)plane, (int)Wp, img);
+            else
+                hipLaunchKernelGGL((conv_gemm_fast_kernel<128, MODE>), grid, dim3(256), 0, s, src, gathered, kernel, out, d,
+                                   tabB, tabA, (int)plane, (int)Wp, img);
+            const int rc = repdl_launch_status();
+            e = hipFreeAsync(ws, s);
+            return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
+        }
+    }
     if (M <= 64)
     {
         dim3 grid((unsigned)gx, (unsigned)repdl_cdiv(M, 64), (unsigned)gz);
