@@ -1,0 +1,94 @@
+"""GPU parity of the three convolutions against the oracle beyond the golden cases: shapes
+that take the matrix-instruction kernels' fast paths (whole channel tiles, K a multiple of
+16, padded-workspace gather; grad-kernel with OW a multiple of 16 or 28) and shapes that
+fall back, strides, paddings larger and smaller than the kernel reach, groups, pixels that
+do not fill the last tile, and data that forces the exact recomputation of zero / NaN
+results (ReLU zeros, signed zeros, infinities)."""
+import pytest
+import torch
+
+import gen
+from oracle import api as oracle
+
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("matrix_path")]
+
+# (N, IC, H, W, OC, KH, KW, sH, sW, pH, pW, groups)
+FWD = [
+    (2, 32, 20, 24, 64, 3, 3, 1, 1, 1, 1, 1),    # fast path, 480 pixels (3.75 tiles)
+    (3, 16, 17, 13, 64, 1, 1, 1, 1, 0, 0, 1),    # fast path, no padding workspace
+    (2, 64, 19, 19, 128, 3, 3, 2, 2, 1, 1, 2),   # fast path, groups, stride 2
+    (1, 16, 12, 40, 128, 5, 5, 1, 2, 1, 3, 1),   # fast path, BM = 128, asymmetric stride / padding
+    (2, 16, 9, 9, 64, 1, 1, 1, 1, 1, 1, 1),      # padding beyond the kernel reach
+    (2, 8, 14, 14, 24, 3, 3, 1, 1, 1, 1, 1),     # K = 72: general kernel
+    (1, 12, 10, 11, 70, 3, 2, 2, 1, 0, 1, 1),    # ragged everything
+]
+
+
+def _data(shape, seed, special):
+    N, IC, H, W, OC, KH, KW, sH, sW, pH, pW, g = shape
+    x = gen.relu_like(seed, N, IC, H, W)
+    w = gen.normal_like(seed + 1, OC, IC // g, KH, KW)
+    if special:
+        x.view(-1)[::97] = float("inf")
+        x.view(-1)[5::211] = -0.0
+        w.view(-1)[::53] = 0.0
+        w.view(-1)[7::59] = -0.0
+    return x, w
+
+
+def _same(got, want):
+    nan = torch.isnan(want)
+    return torch.equal(torch.isnan(got), nan) and torch.equal(got.view(torch.int32)[~nan], want.view(torch.int32)[~nan])
+
+
+@pytest.mark.parametrize("special", [False, True], ids=["plain", "special"])
+@pytest.mark.parametrize("shape", FWD, ids=[str(s) for s in FWD])
+def test_forward(shape, special):
+    from repdl_amd import ops
+
+    N, IC, H, W, OC, KH, KW, sH, sW, pH, pW, g = shape
+    x, w = _data(shape, 100, special)
+    got = ops.conv2d(x.cuda(), w.cuda(), (sH, sW), (pH, pW), g).cpu()
+    assert _same(got, oracle.conv2d(x, w, sH, sW, pH, pW, g))
+
+
+@pytest.mark.parametrize("special", [False, True], ids=["plain", "special"])
+@pytest.mark.parametrize("shape", [s for s in FWD if s[-1] == 1], ids=[str(s) for s in FWD if s[-1] == 1])
+def test_grad_input(shape, special):
+    from repdl_amd import ops
+
+    N, IC, H, W, OC, KH, KW, sH, sW, pH, pW, g = shape
+    OH, OW = (H + 2 * pH - KH) // sH + 1, (W + 2 * pW - KW) // sW + 1
+    go = gen.normal_like(7, N, OC, OH, OW) * gen.relu_like(8, N, OC, OH, OW).sign()
+    w = gen.normal_like(9, OC, IC, KH, KW)
+    if special:
+        go.view(-1)[::101] = float("-inf")
+        w.view(-1)[3::41] = -0.0
+    got = ops.conv2d_grad_input((N, IC, H, W), w.cuda(), go.cuda(), (sH, sW), (pH, pW)).cpu()
+    assert _same(got, oracle.conv2d_grad_input(go, w, H, W, sH, sW, pH, pW))
+
+
+WGRAD = [
+    (3, 20, 18, 16, 40, 3, 3, 1, 1, 1, 1),   # OW = 16: one piece of 4 instructions
+    (2, 8, 30, 28, 70, 3, 3, 1, 1, 1, 1),    # OW = 28: pieces of 7, OH = 30 -> chunks of several rows
+    (2, 16, 16, 64, 16, 1, 1, 1, 1, 0, 0),   # OW = 64: pieces of 16, 1x1
+    (2, 6, 33, 65, 33, 3, 3, 2, 2, 1, 1),    # stride 2, OW = 33: v_fma_f32 kernel
+    (2, 5, 11, 12, 9, 2, 3, 1, 1, 0, 1),     # ragged
+]
+
+
+@pytest.mark.parametrize("special", [False, True], ids=["plain", "special"])
+@pytest.mark.parametrize("shape", WGRAD, ids=[str(s) for s in WGRAD])
+def test_grad_kernel(shape, special):
+    from repdl_amd import ops
+
+    N, IC, H, W, OC, KH, KW, sH, sW, pH, pW = shape
+    OH, OW = (H + 2 * pH - KH) // sH + 1, (W + 2 * pW - KW) // sW + 1
+    x = gen.relu_like(21, N, IC, H, W)
+    go = gen.normal_like(22, N, OC, OH, OW)
+    if special:
+        x.view(-1)[::89] = float("inf")
+        go.view(-1)[::61] = 0.0
+        go[:, 0] = 0.0  # a whole output channel of zero gradients: results are exact zeros
+    got = ops.conv2d_grad_kernel(x.cuda(), (OC, IC, KH, KW), go.cuda(), (sH, sW), (pH, pW)).cpu()
+    assert _same(got, oracle.conv2d_grad_kernel(go, x, KH, KW, sH, sW, pH, pW))
