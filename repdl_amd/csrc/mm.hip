@@ -18,8 +18,6 @@
 // k-major (As[k][m], Bs[k][n]) so the inner loop reads its 8+8 operands with
 // four ds_read_b128 and issues 64 v_fma_f32.  Global loads for tile t+1 are
 // issued before the FMAs of tile t (register prefetch, two LDS buffers).
-#include <stdlib.h>
-
 #include "common.h"
 
 namespace
@@ -628,7 +626,7 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_fast_kernel(const float
             const int64_t m = m0 + wm * 32 * FM + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3);
 #pragma unroll
             for (int j = 0; j < FN; j++)
-                C[m * N + n0 + wn * 32 * FN + 32 * j + l32] = acc[i][j][r];
+                __builtin_nontemporal_store(acc[i][j][r], &C[m * N + n0 + wn * 32 * FN + 32 * j + l32]);
         }
 }
 
@@ -710,20 +708,14 @@ REPDL_API int repdl_hip_mm(const float *A, const float *B, float *C, int64_t M, 
             cfg = 3;
         else if (repdl_cdiv(M, 128) * repdl_cdiv(N, 128) >= target)
             cfg = 1;
-        if (const char *e = getenv("REPDL_HIP_MM_TILE"))
-            cfg = atoi(e);
         switch (cfg)
         {
         case 0:
             return launch_mfma<1, 1, 2, 2>(A, B, C, M, N, K, transA, transB, avec, bvec, s);
         case 1:
             return launch_mfma<2, 2, 2, 2>(A, B, C, M, N, K, transA, transB, avec, bvec, s);
-        case 2:
-            return launch_mfma<4, 2, 2, 2>(A, B, C, M, N, K, transA, transB, avec, bvec, s);
-        case 3:
-            return launch_mfma<4, 2, 2, 4>(A, B, C, M, N, K, transA, transB, avec, bvec, s);
         default:
-            return launch_mfma<4, 4, 2, 2>(A, B, C, M, N, K, transA, transB, avec, bvec, s);
+            return launch_mfma<4, 2, 2, 4>(A, B, C, M, N, K, transA, transB, avec, bvec, s);
         }
     }
     const int64_t gx = repdl_cdiv(N, BN), gy = repdl_cdiv(M, BM);
