@@ -1163,22 +1163,21 @@ __global__ __launch_bounds__(256) void conv_wgrad_kernel(const float *__restrict
 //   * the input rows the 16 columns touch, zero-padded left and right as in
 //     conv_wgrad_kernel, so that a tap is an LDS word at a fixed per-lane offset
 // into the LDS buffer that is not being computed from, and then issue the global
-// loads of the chunk after, which stay in flight across the barrier.  Staging slots
-// beyond the data load word 0 of the chunk and store nothing.
+// loads of the chunk after, which stay in flight across the barrier.
 // Lane l of a computing wave supplies, for the four steps ow..ow+3 of one
 // instruction, grad_output of oc l%16 and the tap of column l%16, both at step l/16.
 // Operands are read a piece (QP instructions) ahead.  Out-of-image taps read staged
 // zeros, so +-0 / NaN results are recomputed with the literal chain, as everywhere
-// in this file.  Requires OW % (4 QP) == 0, OH % R == 0 and 16-byte aligned
-// grad_output; other shapes take conv_wgrad_kernel.
+// in this file.  Requires OW % (4 QP) == 0, OH % R == 0, W % 4 == 0 and 16-byte aligned
+// grad_output and input; other shapes take conv_wgrad_kernel.
 // ---------------------------------------------------------------------------
 typedef float f4v __attribute__((ext_vector_type(4)));
 constexpr int MW_GS = 16; // float4 staging slots of grad_output per staging thread
-constexpr int MW_XS = 8;  // float4 staging slots of input per staging thread
+constexpr int MW_XS = 8;  // most float4 staging slots of input per staging thread
 constexpr int MW_OC = 32; // oc per workgroup
 constexpr int MW_ST = 128; // staging threads
 
-template <int QP, bool UNIT> // QP: instructions per piece
+template <int QP, bool UNIT, int XS> // QP: instructions per piece; XS: input staging slots per thread
 __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__restrict__ GO,
                                                               const float *__restrict__ X,
                                                               float *__restrict__ GK, ConvDims d, int R, int NP,
@@ -1204,21 +1203,23 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
         const int st = tid & (MW_ST - 1);
         const int last_col = (c0 + 15 < NC) ? c0 + 15 : NC - 1;
         const int nic = last_col / KHW - ic_first + 1;
-        // slots, fixed for the whole kernel.  Input: slot = (staged row, 4 floats of it).
-        const int nw4 = (d.W + 3) >> 2;
+        // Slots, fixed for the whole kernel.  Slots past the data repeat the last slot (same words,
+        // same values), so that no load or store sits behind a branch or a mask (the compiler waits
+        // for every outstanding load where branches that contain loads merge).
+        // Input: slot = (staged row, 4 floats of it); W % 4 == 0 and 16-byte alignment are given.
+        const int nw4 = d.W >> 2;
         const int nxs = nic * hrows * nw4;
-        int x_goff[MW_XS], x_hr[MW_XS], x_w[MW_XS], x_loff[MW_XS];
+        int x_goff[XS], x_hr[XS], x_loff[XS];
 #pragma unroll
-        for (int i = 0; i < MW_XS; i++)
+        for (int i = 0; i < XS; i++)
         {
-            const int s = st + MW_ST * i;
-            const bool on = s < nxs;
+            int s = st + MW_ST * i;
+            s = s < nxs ? s : nxs - 1;
             const int row = s / nw4, w = (s - row * nw4) << 2;
             const int icl = row / hrows, hr = row - icl * hrows;
-            x_goff[i] = on ? (ic_first + icl) * d.H * d.W + w : 0;
+            x_goff[i] = (ic_first + icl) * d.H * d.W + w;
             x_hr[i] = hr;
-            x_w[i] = on ? w : 0;
-            x_loff[i] = on ? xoff + icl * CP + hr * Wp + d.pW + w : -1;
+            x_loff[i] = xoff + icl * CP + hr * Wp + d.pW + w;
         }
         // grad_output: slot = (oc, 4 consecutive steps of the chunk)
         const int spo = (R * d.OW) >> 2; // float4 per oc and chunk
@@ -1227,39 +1228,29 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
 #pragma unroll
         for (int i = 0; i < MW_GS; i++)
         {
-            const int s = st + MW_ST * i;
-            const bool on = s < MW_OC * spo;
+            int s = st + MW_ST * i;
+            s = s < MW_OC * spo ? s : MW_OC * spo - 1;
             const int o = s / spo, t = (s - o * spo) << 2;
             const int oc = oc0 + o < d.OC ? oc0 + o : d.OC - 1; // rows of missing oc repeat the last one
-            g_goff[i] = on ? (uint32_t)((oc - oc0) * d.OH * d.OW + t) * 4u : 0u;
-            g_loff[i] = on ? 64 + o * GP + t : -1;
+            g_goff[i] = (uint32_t)((oc - oc0) * d.OH * d.OW + t) * 4u;
+            g_loff[i] = 64 + o * GP + t;
         }
-        f4v xst[MW_XS], gst[MW_GS]; // plain vectors: they must stay in registers
+        f4v xst[XS], gst[MW_GS]; // plain vectors: they must stay in registers
         auto chunk_load = [&](int n, int oh0) {
             const float *Xn = X + (int64_t)n * d.IC * d.H * d.W;
             const int hbase = oh0 * d.sH - d.pH;
 #pragma unroll
-            for (int i = 0; i < MW_XS; i++)
-            {
-                const int h = hbase + x_hr[i];
-                const bool ok = h >= 0 && h < d.H;
-                const int hc = h < 0 ? 0 : (h >= d.H ? d.H - 1 : h);
-                const float *p = Xn + x_goff[i] + hc * d.W;
-                f4v v;
-                if (xvec)
-                    v = *reinterpret_cast<const f4v *>(p); // W % 4 == 0: whole float4 inside the row
-                else
+            for (int i = 0; i < XS; i++)
                 {
-                    v.x = p[0];
-                    v.y = x_w[i] + 1 < d.W ? p[1] : 0.0f;
-                    v.z = x_w[i] + 2 < d.W ? p[2] : 0.0f;
-                    v.w = x_w[i] + 3 < d.W ? p[3] : 0.0f;
+                    const int h = hbase + x_hr[i];
+                    const bool ok = h >= 0 && h < d.H;
+                    const int hc = h < 0 ? 0 : (h >= d.H ? d.H - 1 : h);
+                    const f4v v = *reinterpret_cast<const f4v *>(Xn + x_goff[i] + hc * d.W);
+                    xst[i][0] = ok ? v[0] : 0.0f;
+                    xst[i][1] = ok ? v[1] : 0.0f;
+                    xst[i][2] = ok ? v[2] : 0.0f;
+                    xst[i][3] = ok ? v[3] : 0.0f;
                 }
-                xst[i].x = ok ? v.x : 0.0f;
-                xst[i].y = ok ? v.y : 0.0f;
-                xst[i].z = ok ? v.z : 0.0f;
-                xst[i].w = ok ? v.w : 0.0f;
-            }
             const char *Gn = reinterpret_cast<const char *>(GO + (((int64_t)n * d.OC + oc0) * d.OH + oh0) * d.OW);
 #pragma unroll
             for (int i = 0; i < MW_GS; i++)
@@ -1268,19 +1259,17 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
         auto stage_store = [&](int buf) {
             float *base = lds + buf * bufsz;
 #pragma unroll
-            for (int i = 0; i < MW_XS; i++)
-                if (x_loff[i] >= 0)
+            for (int i = 0; i < XS; i++)
                 {
                     float *p = base + x_loff[i];
-                    p[0] = xst[i].x;
-                    p[1] = xst[i].y;
-                    p[2] = xst[i].z;
-                    p[3] = xst[i].w;
+                    p[0] = xst[i][0];
+                    p[1] = xst[i][1];
+                    p[2] = xst[i][2];
+                    p[3] = xst[i][3];
                 }
 #pragma unroll
             for (int i = 0; i < MW_GS; i++)
-                if (g_loff[i] >= 0)
-                    *reinterpret_cast<f4v *>(base + g_loff[i]) = gst[i];
+                *reinterpret_cast<f4v *>(base + g_loff[i]) = gst[i];
         };
         int n1 = 0, oh1 = 0; // the chunk the next chunk_load fetches
         auto advance = [&]() {
@@ -1362,11 +1351,12 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
         // behind every instruction, pinned there (left alone, the scheduler moves the reads
         // behind the last instructions of the piece, too late for the next one)
         auto step_piece = [&](const float (&ca)[QP], const float (&cb)[QP], float (&na)[QP], float (&nb)[QP]) {
-            next_piece();
 #pragma unroll
             for (int u = 0; u < QP; u++)
             {
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ca[u], cb[u], acc, 0, 0, 0);
+                if (u == 0)
+                    next_piece(); // the address arithmetic of the next piece runs under the first instruction
                 na[u] = ap[4 * u];
                 nb[u] = xp[4 * u * sW];
                 __builtin_amdgcn_sched_barrier(0);
@@ -1544,7 +1534,7 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
     hipStream_t s = repdl_stream(stream);
 
     // Matrix-instruction kernel: geometry of a chunk (see conv_wgrad_mfma_kernel).
-    if (repdl_mfma_exact() && OW % 4 == 0 && sW <= 16 && aligned16(grad_output))
+    if (repdl_mfma_exact() && OW % 4 == 0 && W % 4 == 0 && sW <= 16 && aligned16(grad_output) && aligned16(input))
     {
         const int64_t KHW = KH * KW, NC = IC * KHW;
         // instructions per piece: the largest candidate that divides a row of OW / 4 instructions
@@ -1598,24 +1588,29 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
             size_t shmem = (size_t)(2 * bufsz * 4);
             if (shmem < 84 * 1024)
                 shmem = 84 * 1024; // one workgroup per CU: every wave has a SIMD to itself
-#define REPDL_WGRAD_MFMA(Q, U)                                                                                     \
-    do                                                                                                            \
-    {                                                                                                             \
-        hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_wgrad_mfma_kernel<Q, U>),        \
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);              \
-        if (e_ != hipSuccess)                                                                                     \
-            return (int)e_;                                                                                       \
-        hipLaunchKernelGGL((conv_wgrad_mfma_kernel<Q, U>), dim3((unsigned)gx, (unsigned)gy), dim3(256), shmem, s, \
-                           grad_output, input, grad_kernel, d, (int)R, (int)NP, (int)GP, (int)Wp, (int)CP,        \
-                           (int)hrows, (int)xoff, (int)bufsz, xvec);                                              \
+            const bool few = nic_max * hrows * nw4 <= 2 * MW_ST; // input slots per staging thread: 2 or MW_XS
+#define REPDL_WGRAD_MFMA(Q, U, X)                                                                                    \
+    do                                                                                                              \
+    {                                                                                                               \
+        hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_wgrad_mfma_kernel<Q, U, X>),       \
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);                \
+        if (e_ != hipSuccess)                                                                                       \
+            return (int)e_;                                                                                         \
+        hipLaunchKernelGGL((conv_wgrad_mfma_kernel<Q, U, X>), dim3((unsigned)gx, (unsigned)gy), dim3(256), shmem, s, \
+                           grad_output, input, grad_kernel, d, (int)R, (int)NP, (int)GP, (int)Wp, (int)CP,          \
+                           (int)hrows, (int)xoff, (int)bufsz, xvec);                                                \
     } while (0)
-#define REPDL_WGRAD_MFMA_Q(Q)          \
-    do                                 \
-    {                                  \
-        if (sW == 1)                   \
-            REPDL_WGRAD_MFMA(Q, true); \
-        else                           \
-            REPDL_WGRAD_MFMA(Q, false); \
+#define REPDL_WGRAD_MFMA_Q(Q)                     \
+    do                                            \
+    {                                             \
+        if (sW == 1 && few)                       \
+            REPDL_WGRAD_MFMA(Q, true, 2);         \
+        else if (sW == 1)                         \
+            REPDL_WGRAD_MFMA(Q, true, MW_XS);     \
+        else if (few)                             \
+            REPDL_WGRAD_MFMA(Q, false, 2);        \
+        else                                      \
+            REPDL_WGRAD_MFMA(Q, false, MW_XS);    \
     } while (0)
             if (QP == 16)
                 REPDL_WGRAD_MFMA_Q(16);
