@@ -1334,17 +1334,23 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
         // dummy piece whose grad_output operand comes from the 64 zero words in front of the
         // buffer (products of zero only matter to results that are recomputed anyway).
         const float *zb = lds + buf * bufsz + q;
-        int rr = 0, rp = 0; // piece the next read fetches (row, piece of the row)
+        // the piece the next read fetches: number q (row q / NP, piece q % NP of the row).  Its
+        // grad_output words start at 4*QP*q (rows follow each other without a gap), its taps at
+        // xrow + 4*QP*sW*(q % NP); everything advances by additions on the scalar unit.
+        int q_next = 0, rp = 0, aoff = 0, xrow = 0, xoff_p = 0;
         const float *ap, *xp;
         auto next_piece = [&]() {
-            const bool dummy = rr >= R;
-            const int xr = dummy ? 0 : rr;
-            ap = dummy ? zb : ab + rr * OWp + 4 * QP * rp;
-            xp = xb + xr * d.sH * Wp + 4 * QP * rp * sW;
+            const bool dummy = q_next >= npieces;
+            ap = dummy ? zb : ab + aoff;
+            xp = xb + (dummy ? 0 : xoff_p);
+            q_next++;
+            aoff += 4 * QP;
+            xoff_p += 4 * QP * sW;
             if (++rp == NP)
             {
                 rp = 0;
-                rr++;
+                xrow += d.sH * Wp;
+                xoff_p = xrow;
             }
         };
         // runs the piece in (ca, cb) and reads the next one into (na, nb): one pair of reads
