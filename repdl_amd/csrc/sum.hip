@@ -121,9 +121,12 @@ __global__ __launch_bounds__(RT) void rowchain_kernel(const float *__restrict__ 
                     va[u] = *reinterpret_cast<const v4f *>(&row[4 * u]);
                 for (int c = 0; c < nfull; c += 8 * WB)
                 {
+                    // (the barriers keep the scheduler from gathering all reads in one place, which
+                    // would leave the adds waiting for reads issued just before them)
 #pragma unroll
                     for (int u = 0; u < WB; u++)
                         vb[u] = *reinterpret_cast<const v4f *>(&row[c + 4 * WB + 4 * u]);
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int u = 0; u < WB; u++)
                     {
@@ -132,10 +135,12 @@ __global__ __launch_bounds__(RT) void rowchain_kernel(const float *__restrict__ 
                         acc = acc + va[u].z;
                         acc = acc + va[u].w;
                     }
+                    __builtin_amdgcn_sched_barrier(0);
                     // the last step reads 4*WB floats past the row: inside the tile or its pad
 #pragma unroll
                     for (int u = 0; u < WB; u++)
                         va[u] = *reinterpret_cast<const v4f *>(&row[c + 8 * WB + 4 * u]);
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int u = 0; u < WB; u++)
                     {
@@ -144,6 +149,7 @@ __global__ __launch_bounds__(RT) void rowchain_kernel(const float *__restrict__ 
                         acc = acc + vb[u].z;
                         acc = acc + vb[u].w;
                     }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
             for (int c = nfull; c < here; c++)
