@@ -54,6 +54,40 @@ def build(verbose: bool = False) -> str:
     return LIB
 
 
+EXT_NAME = "_hip_ext"
+
+
+def ext_path() -> str:
+    import sysconfig
+
+    return os.path.join(HERE, "backend", EXT_NAME + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_ext(verbose: bool = False) -> str:
+    """Builds ``repdl_amd/backend/_hip_ext``: csrc/bind.cpp, the PyTorch C++ extension module
+    with the function list of RepDL's backend/cuda/bind.cpp, over librepdl_hip.so.  Host C++
+    only (g++ against the PyTorch and HIP headers); needs build() first."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    out = ext_path()
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+           "-DTORCH_EXTENSION_NAME=" + EXT_NAME, "-DTORCH_API_INCLUDE_EXTENSION_H", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI), "-Wno-deprecated-declarations"]
+    for inc in ce.include_paths() + [sysconfig.get_paths()["include"], "/opt/rocm/include"]:
+        cmd += ["-isystem", inc]
+    cmd += [os.path.join(CSRC, "bind.cpp"), "-o", out, "-L" + tlib, "-L" + HERE, "-lrepdl_hip", "-lc10", "-lc10_hip",
+            "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python", "-Wl,-rpath,$ORIGIN/..", "-Wl,-rpath," + tlib]
+    _run(cmd)
+    if verbose:
+        print(out)
+    return out
+
+
 if __name__ == "__main__":
     build(verbose=True)
+    build_ext(verbose=True)
     sys.exit(0)

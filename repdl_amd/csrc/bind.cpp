@@ -1,0 +1,246 @@
+// repdl_amd.backend._hip_ext -- the compiled counterpart of RepDL's repdl.backend.cuda
+// (backend/cuda/bind.cpp:6-19): a PyTorch C++ extension module that exports the same ten
+// functions with the same positional signatures (matrix_multiplication.cu:234-235, 267;
+// convolution.cu:153-155, 259-262, 359-362, 385-387; summation.cu:149-155;
+// softmax.cpp:15, 28; cross_entropy.cpp:15, 31), plus exp / log / sqrt / div / div_scalar.
+// It is the only file of this library that knows about PyTorch: every function checks its
+// tensors, allocates the output on the input's device, and hands raw pointers and the current
+// stream to the C ABI of include/repdl_hip.h.  Host C++ only; built with the host compiler
+// against the PyTorch headers (repdl_amd/build.py, build_ext).
+#include <torch/extension.h>
+
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+
+#include "../../include/repdl_hip.h"
+
+namespace repdl
+{
+namespace hip
+{
+namespace
+{
+// PyTorch-ROCm presents HIP devices and streams under the CUDA names.
+using DeviceGuard = c10::hip::HIPGuardMasqueradingAsCUDA;
+
+void *current_stream() { return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream(); }
+
+torch::Tensor checked(const torch::Tensor &t, const char *name, int64_t dim, c10::ScalarType dtype = torch::kFloat)
+{
+    TORCH_CHECK(t.is_cuda(), name, " must be on the GPU (this backend has no CPU path)");
+    TORCH_CHECK(t.scalar_type() == dtype, name, " must be ", dtype, ", got ", t.scalar_type());
+    TORCH_CHECK(dim < 0 || t.dim() == dim, name, " must have ", dim, " dimensions, got ", t.dim());
+    return t.contiguous();
+}
+
+void same_device(const torch::Tensor &a, const torch::Tensor &b)
+{
+    TORCH_CHECK(a.device() == b.device(), "tensors are on different devices: ", a.device(), " and ", b.device());
+}
+
+void ok(int rc, const char *what) { TORCH_CHECK(rc == 0, what, " failed with code ", rc, ": ", repdl_hip_error_string(rc)); }
+} // namespace
+
+torch::Tensor mm(const torch::Tensor &input, const torch::Tensor &mat2, bool transA, bool transB)
+{
+    const auto a = checked(input, "input", 2), b = checked(mat2, "mat2", 2);
+    same_device(a, b);
+    const int64_t M = !transA ? a.size(0) : a.size(1), K = !transA ? a.size(1) : a.size(0);
+    const int64_t N = !transB ? b.size(1) : b.size(0), Kb = !transB ? b.size(0) : b.size(1);
+    TORCH_CHECK(K == Kb, "mm: inner dimensions differ (", K, " vs ", Kb, ")");
+    const DeviceGuard guard(a.device());
+    auto out = torch::empty({M, N}, a.options());
+    ok(repdl_hip_mm(a.data_ptr<float>(), b.data_ptr<float>(), out.data_ptr<float>(), M, N, K, transA, transB,
+                    current_stream()),
+       "repdl_hip_mm");
+    return out;
+}
+
+torch::Tensor conv2d(const torch::Tensor &input, const torch::Tensor &kernel, int64_t sH, int64_t sW, int64_t pH,
+                     int64_t pW, int64_t groups)
+{
+    const auto x = checked(input, "input", 4), k = checked(kernel, "kernel", 4);
+    same_device(x, k);
+    const int64_t N = x.size(0), IC = x.size(1), H = x.size(2), W = x.size(3);
+    const int64_t OC = k.size(0), ICg = k.size(1), KH = k.size(2), KW = k.size(3);
+    TORCH_CHECK(groups > 0 && IC % groups == 0 && OC % groups == 0 && ICg == IC / groups, "conv2d: channels (", IC,
+                " in, ", OC, " out, kernel ", ICg, ") do not match groups=", groups);
+    TORCH_CHECK(sH > 0 && sW > 0 && pH >= 0 && pW >= 0, "conv2d: bad stride or padding");
+    TORCH_CHECK(H + 2 * pH >= KH && W + 2 * pW >= KW, "conv2d: kernel larger than padded input");
+    const int64_t OH = (H + 2 * pH - KH) / sH + 1, OW = (W + 2 * pW - KW) / sW + 1;
+    const DeviceGuard guard(x.device());
+    auto out = torch::empty({N, OC, OH, OW}, x.options());
+    ok(repdl_hip_conv2d(x.data_ptr<float>(), k.data_ptr<float>(), out.data_ptr<float>(), N, IC, H, W, OC, KH, KW, sH,
+                        sW, pH, pW, groups, current_stream()),
+       "repdl_hip_conv2d");
+    return out;
+}
+
+torch::Tensor conv2d_grad_input(const torch::Tensor &grad_output, const torch::Tensor &kernel, int64_t H, int64_t W,
+                                int64_t sH, int64_t sW, int64_t pH, int64_t pW)
+{
+    const auto go = checked(grad_output, "grad_output", 4), k = checked(kernel, "kernel", 4);
+    same_device(go, k);
+    const int64_t N = go.size(0), OC = go.size(1), OH = go.size(2), OW = go.size(3);
+    const int64_t IC = k.size(1), KH = k.size(2), KW = k.size(3);
+    TORCH_CHECK(k.size(0) == OC, "conv2d_grad_input: grad_output has ", OC, " channels, kernel has ", k.size(0));
+    const DeviceGuard guard(go.device());
+    auto out = torch::empty({N, IC, H, W}, go.options());
+    ok(repdl_hip_conv2d_grad_input(go.data_ptr<float>(), k.data_ptr<float>(), out.data_ptr<float>(), N, OC, OH, OW, IC,
+                                   KH, KW, H, W, sH, sW, pH, pW, current_stream()),
+       "repdl_hip_conv2d_grad_input");
+    return out;
+}
+
+torch::Tensor conv2d_grad_kernel(const torch::Tensor &grad_output, const torch::Tensor &input, int64_t KH, int64_t KW,
+                                 int64_t sH, int64_t sW, int64_t pH, int64_t pW)
+{
+    const auto go = checked(grad_output, "grad_output", 4), x = checked(input, "input", 4);
+    same_device(go, x);
+    const int64_t N = x.size(0), IC = x.size(1), H = x.size(2), W = x.size(3);
+    const int64_t OC = go.size(1), OH = go.size(2), OW = go.size(3);
+    TORCH_CHECK(go.size(0) == N, "conv2d_grad_kernel: batch sizes differ (", N, " vs ", go.size(0), ")");
+    const DeviceGuard guard(x.device());
+    auto out = torch::empty({OC, IC, KH, KW}, x.options());
+    ok(repdl_hip_conv2d_grad_kernel(go.data_ptr<float>(), x.data_ptr<float>(), out.data_ptr<float>(), N, IC, H, W, OC,
+                                    OH, OW, KH, KW, sH, sW, pH, pW, current_stream()),
+       "repdl_hip_conv2d_grad_kernel");
+    return out;
+}
+
+torch::Tensor sum1d(const torch::Tensor &input, bool average)
+{
+    const auto x = checked(input, "input", 1);
+    const int64_t n = x.size(0);
+    const DeviceGuard guard(x.device());
+    auto out = torch::empty({}, x.options());
+    const size_t nbytes = repdl_hip_sum1d_workspace_bytes(n);
+    // scratch for the parallel evaluation of the sequential chain, from PyTorch's allocator
+    auto work = torch::empty({(int64_t)nbytes}, x.options().dtype(torch::kUInt8));
+    ok(repdl_hip_sum1d_ws(x.data_ptr<float>(), out.data_ptr<float>(), n, average, nbytes ? work.data_ptr() : nullptr,
+                          nbytes, current_stream()),
+       "repdl_hip_sum1d_ws");
+    return out;
+}
+
+torch::Tensor sum2d_dim0(const torch::Tensor &input, bool keepdim, bool average)
+{
+    const auto x = checked(input, "input", 2);
+    const DeviceGuard guard(x.device());
+    auto out = torch::empty({1, x.size(1)}, x.options());
+    ok(repdl_hip_sum2d_dim0(x.data_ptr<float>(), out.data_ptr<float>(), x.size(0), x.size(1), average, current_stream()),
+       "repdl_hip_sum2d_dim0");
+    return keepdim ? out : out.squeeze();
+}
+
+torch::Tensor sum2d_dim1(const torch::Tensor &input, bool keepdim, bool average)
+{
+    const auto x = checked(input, "input", 2);
+    const DeviceGuard guard(x.device());
+    auto out = torch::empty({x.size(0), 1}, x.options());
+    ok(repdl_hip_sum2d_dim1(x.data_ptr<float>(), out.data_ptr<float>(), x.size(0), x.size(1), average, current_stream()),
+       "repdl_hip_sum2d_dim1");
+    return keepdim ? out : out.squeeze();
+}
+
+torch::Tensor sum4d_dim023(const torch::Tensor &input, bool keepdim, bool average)
+{
+    const auto x = checked(input, "input", 4);
+    const DeviceGuard guard(x.device());
+    auto out = torch::empty({1, x.size(1), 1, 1}, x.options());
+    ok(repdl_hip_sum4d_dim023(x.data_ptr<float>(), out.data_ptr<float>(), x.size(0), x.size(1), x.size(2), x.size(3),
+                              average, current_stream()),
+       "repdl_hip_sum4d_dim023");
+    return keepdim ? out : out.squeeze();
+}
+
+namespace
+{
+template <typename F>
+torch::Tensor unary(const torch::Tensor &input, F fn, const char *what)
+{
+    const auto x = checked(input, "input", -1);
+    const DeviceGuard guard(x.device());
+    auto out = torch::empty_like(x);
+    ok(fn(x.data_ptr<float>(), out.data_ptr<float>(), x.numel(), current_stream()), what);
+    return out;
+}
+} // namespace
+
+torch::Tensor exp(const torch::Tensor &input) { return unary(input, repdl_hip_exp, "repdl_hip_exp"); }
+torch::Tensor log(const torch::Tensor &input) { return unary(input, repdl_hip_log, "repdl_hip_log"); }
+torch::Tensor sqrt(const torch::Tensor &input) { return unary(input, repdl_hip_sqrt, "repdl_hip_sqrt"); }
+
+torch::Tensor div_scalar(const torch::Tensor &input, double other)
+{
+    const auto x = checked(input, "input", -1);
+    const DeviceGuard guard(x.device());
+    auto out = torch::empty_like(x);
+    ok(repdl_hip_div_scalar(x.data_ptr<float>(), (float)other, out.data_ptr<float>(), x.numel(), current_stream()),
+       "repdl_hip_div_scalar");
+    return out;
+}
+
+// input / other elementwise; `other` is broadcast to the common shape; a 0-dim `other` goes
+// through the scalar entry point (repdl/ops.py:98-103 divides by Python numbers and tensors alike)
+torch::Tensor div(const torch::Tensor &input, const torch::Tensor &other)
+{
+    if (other.dim() == 0)
+        return div_scalar(input, other.item<double>());
+    auto x = checked(input, "input", -1), y = checked(other, "other", -1);
+    same_device(x, y);
+    const auto shape = at::infer_size(x.sizes(), y.sizes());
+    x = x.expand(shape).contiguous();
+    y = y.expand(shape).contiguous();
+    const DeviceGuard guard(x.device());
+    auto out = torch::empty(shape, x.options());
+    ok(repdl_hip_div(x.data_ptr<float>(), y.data_ptr<float>(), out.data_ptr<float>(), out.numel(), current_stream()),
+       "repdl_hip_div");
+    return out;
+}
+
+torch::Tensor softmax(const torch::Tensor &input)
+{
+    const auto x = checked(input, "input", 2);
+    const DeviceGuard guard(x.device());
+    auto out = torch::empty_like(x);
+    ok(repdl_hip_softmax(x.data_ptr<float>(), out.data_ptr<float>(), x.size(0), x.size(1), current_stream()),
+       "repdl_hip_softmax");
+    return out;
+}
+
+torch::Tensor cross_entropy(const torch::Tensor &input, const torch::Tensor &target)
+{
+    const auto x = checked(input, "input", 2), t = checked(target, "target", 1, torch::kLong);
+    same_device(x, t);
+    TORCH_CHECK(t.size(0) == x.size(0), "cross_entropy: ", x.size(0), " rows but ", t.size(0), " targets");
+    const DeviceGuard guard(x.device());
+    auto out = torch::empty({}, x.options());
+    auto work = torch::empty({std::max<int64_t>(x.size(0), 1)}, x.options());
+    ok(repdl_hip_cross_entropy(x.data_ptr<float>(), t.data_ptr<int64_t>(), out.data_ptr<float>(), x.size(0), x.size(1),
+                               work.data_ptr<float>(), current_stream()),
+       "repdl_hip_cross_entropy");
+    return out;
+}
+} // namespace hip
+} // namespace repdl
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
+{
+    namespace h = repdl::hip;
+    m.def("conv2d", &h::conv2d);
+    m.def("conv2d_grad_input", &h::conv2d_grad_input);
+    m.def("conv2d_grad_kernel", &h::conv2d_grad_kernel);
+    m.def("cross_entropy", &h::cross_entropy);
+    m.def("mm", &h::mm);
+    m.def("softmax", &h::softmax);
+    m.def("sum1d", &h::sum1d, py::arg("input"), py::arg("average") = false);
+    m.def("sum2d_dim0", &h::sum2d_dim0, py::arg("input"), py::arg("keepdim") = false, py::arg("average") = false);
+    m.def("sum2d_dim1", &h::sum2d_dim1, py::arg("input"), py::arg("keepdim") = false, py::arg("average") = false);
+    m.def("sum4d_dim023", &h::sum4d_dim023, py::arg("input"), py::arg("keepdim") = false, py::arg("average") = false);
+    m.def("exp", &h::exp);
+    m.def("log", &h::log);
+    m.def("sqrt", &h::sqrt);
+    m.def("div", &h::div);
+    m.def("div_scalar", &h::div_scalar);
+}

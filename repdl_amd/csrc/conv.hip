@@ -1426,7 +1426,7 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
         const int PL = MODE == MODE_FWD ? d.pW : (d.KW - 1 - d.pW > 0 ? d.KW - 1 - d.pW : 0);
         const int64_t Hp = GH + 2 * (int64_t)PT, Wp = GW + 2 * (int64_t)PL;
         const int64_t plane = Hp * Wp, img = (int64_t)C * plane;
-        if (img * 4 < (1LL << 31) && (int64_t)M * K * 4 < (1LL << 31))
+        if (img * 4 < (1LL << 31) && (int64_t)M * K * 4 < (1LL << 31) && (int64_t)d.N * img / 256 < REPDL_I32_MAX)
         {
             const bool pad = PT > 0 || PL > 0;
             const size_t tab_bytes = ((size_t)2 * K * sizeof(int) + 255) / 256 * 256;

@@ -9,8 +9,17 @@ from repdl_amd.backend import hip
 
 
 class _Adaptor:
+    def __init__(self, binding=None):
+        self._binding = binding  # None: whatever repdl_amd.backend.hip currently serves
+
     def __getattr__(self, name):
-        fn = getattr(hip, name)
+        if self._binding == "ext":
+            from repdl_amd.backend import _hip_ext as mod
+        elif self._binding == "ctypes":
+            from repdl_amd.backend import hip_ctypes as mod
+        else:
+            mod = hip
+        fn = getattr(mod, name)
 
         def call(*args):
             moved = [a.cuda() if isinstance(a, torch.Tensor) else a for a in args]
@@ -22,3 +31,5 @@ class _Adaptor:
 
 
 backend = _Adaptor()
+ext_backend = _Adaptor("ext")
+ctypes_backend = _Adaptor("ctypes")

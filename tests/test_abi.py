@@ -103,3 +103,17 @@ def test_get_hash_convention():
     h.update(lin.weight.detach().numpy().tobytes())
     h.update(lin.bias.detach().numpy().tobytes())
     assert repdl_amd.utils.get_hash(lin) == h.hexdigest()
+
+
+def test_compiled_binding_loads_when_built():
+    """If csrc/bind.cpp has been built, repdl_amd.backend.hip must serve it (an extension that
+    is there but does not import would otherwise go unnoticed behind the ctypes binding)."""
+    from repdl_amd import build
+    from repdl_amd.backend import hip
+
+    if os.path.exists(build.ext_path()):
+        assert hip.BINDING == "ext"
+        for fn in hip.FUNCTIONS:
+            assert callable(getattr(hip, fn))
+    else:
+        assert hip.BINDING == "ctypes"
