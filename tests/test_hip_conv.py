@@ -92,3 +92,24 @@ def test_grad_kernel(shape, special):
         go[:, 0] = 0.0  # a whole output channel of zero gradients: results are exact zeros
     got = ops.conv2d_grad_kernel(x.cuda(), (OC, IC, KH, KW), go.cuda(), (sH, sW), (pH, pW)).cpu()
     assert _same(got, oracle.conv2d_grad_kernel(go, x, KH, KW, sH, sW, pH, pW))
+
+
+@pytest.mark.parametrize("layer", [(64, 64, 56, 56, 64, 3, 1, 1), (64, 256, 56, 56, 64, 1, 1, 0)], ids=["3x3_64_64", "1x1_256_64"])
+def test_benchmark_layers_full_size(layer, matrix_path):
+    """The two convolution layers of the benchmark configuration at full size (batch 64, 56x56),
+    all three operators, every output bit against the oracle."""
+    from repdl_amd import ops
+
+    N, IC, H, W, OC, Kk, st, pd = layer
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(N, IC, H, W, generator=g).clamp_(min=0)
+    w = torch.randn(OC, IC, Kk, Kk, generator=g) * (2.0 / (IC * Kk * Kk)) ** 0.5
+    OH = (H + 2 * pd - Kk) // st + 1
+    go = torch.randn(N, OC, OH, OH, generator=g)
+    xd, wd, god = x.cuda(), w.cuda(), go.cuda()
+    assert gen.sha256(ops.conv2d(xd, wd, (st, st), (pd, pd), 1)) == gen.sha256(oracle.conv2d(x, w, st, st, pd, pd, 1))
+    assert gen.sha256(ops.conv2d_grad_input(x.shape, wd, god, (st, st), (pd, pd))) == gen.sha256(
+        oracle.conv2d_grad_input(go, w, H, W, st, st, pd, pd))
+    if matrix_path == "matrix":  # the v_fma_f32 grad-kernel needs seconds at this size; the golden cases cover it
+        assert gen.sha256(ops.conv2d_grad_kernel(xd, w.shape, god, (st, st), (pd, pd))) == gen.sha256(
+            oracle.conv2d_grad_kernel(go, x, Kk, Kk, st, st, pd, pd))

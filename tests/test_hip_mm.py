@@ -99,3 +99,30 @@ def test_k_tails_keep_negative_zero(K):
     want = oracle.mm(a, b)
     assert torch.equal(got.view(torch.int32), want.view(torch.int32))
     assert (want.view(torch.int32) == -(2 ** 31)).all()
+
+
+@pytest.mark.parametrize("shape", [(8192, 8192, 8192, 0, 1), (4096, 4096, 32768, 0, 0), (4096, 4096, 32768, 0, 1),
+                                   (4096, 4096, 65536, 1, 0)], ids=str)
+def test_full_size_shapes(shape):
+    """The Linear shapes at their full sizes (forward NT, the long-K products, the weight
+    gradient with the batch as K).  The CPU oracle needs minutes for one of these, so the whole
+    output is checked through a property -- the matrix-instruction kernel and the v_fma_f32 kernel,
+    two independent evaluations of the same chains, must agree in every bit -- and a slab of
+    rows is checked against the oracle itself."""
+    from repdl_amd import _lib, ops
+
+    M, N, K, tA, tB = shape
+    g = torch.Generator(device="cuda").manual_seed(M + N + K)
+    a = torch.randn((K, M) if tA else (M, K), generator=g, device="cuda")
+    b = torch.randn((N, K) if tB else (K, N), generator=g, device="cuda")
+    got = ops.mm(a, b, bool(tA), bool(tB))
+    mode = _lib.lib().repdl_hip_matrix_path()
+    _lib.call("repdl_hip_set_matrix_path", 0 if mode == 1 else -1)
+    other = ops.mm(a, b, bool(tA), bool(tB))
+    _lib.call("repdl_hip_set_matrix_path", 0 if mode == 0 else -1)
+    assert torch.equal(got.view(torch.int32), other.view(torch.int32))
+    del other
+    rows = 16
+    a_slab = (a[:, :rows] if tA else a[:rows]).contiguous().cpu()
+    want = oracle.mm(a_slab, b.cpu(), bool(tA), bool(tB))
+    assert torch.equal(got[:rows].cpu().view(torch.int32), want.view(torch.int32))
