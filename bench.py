@@ -111,7 +111,7 @@ def main() -> int:
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (every operator shards by outputs with no "
-              "cross-device arithmetic; see DESIGN.md); run with --gpus 1", file=sys.stderr)
+              "cross-device arithmetic, so a second GPU would only add an all-gather of outputs); run with --gpus 1", file=sys.stderr)
         return 2
 
     import torch
