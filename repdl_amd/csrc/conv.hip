@@ -1333,29 +1333,19 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
         const float *ab = lds + buf * bufsz + a_lane;
         const float *xb = lds + buf * bufsz + x_lane;
         // A piece is QP consecutive instructions of an output row.  The operands of the next
-        // piece are read before the current one runs.  The loop is free of conditions so that
-        // the reads stay where they are written: an odd number of pieces is made even by a
-        // dummy piece whose grad_output operand comes from the 64 zero words in front of the
-        // buffer (products of zero only matter to results that are recomputed anyway).
-        const float *zb = lds + buf * bufsz + q;
-        // the piece the next read fetches: number q (row q / NP, piece q % NP of the row).  Its
-        // grad_output words start at 4*QP*q (rows follow each other without a gap), its taps at
-        // xrow + 4*QP*sW*(q % NP); everything advances by additions on the scalar unit.
-        int q_next = 0, rp = 0, aoff = 0, xrow = 0, xoff_p = 0;
-        const float *ap, *xp;
-        auto next_piece = [&]() {
-            const bool dummy = q_next >= npieces;
-            ap = dummy ? zb : ab + aoff;
-            xp = xb + (dummy ? 0 : xoff_p);
-            q_next++;
-            aoff += 4 * QP;
-            xoff_p += 4 * QP * sW;
-            if (++rp == NP)
-            {
-                rp = 0;
-                xrow += d.sH * Wp;
-                xoff_p = xrow;
-            }
+        // piece are read while the current one runs; the pointers of the piece being read advance
+        // by one vector addition each: the grad_output words of consecutive pieces follow each
+        // other without a gap (4*QP per piece), the taps advance by 4*QP*sW inside a row and jump
+        // to the next staged row after the last piece of a row.  The read behind the last piece
+        // of the chunk fetches words that are never used (inside the buffer, or the slack behind it).
+        const float *ap = ab, *xp = xb;
+        int rp = 0;
+        const int xstep_in = 4 * QP * sW, xstep_row = d.sH * Wp - (NP - 1) * 4 * QP * sW;
+        auto advance_piece = [&]() {
+            ap += 4 * QP;
+            const bool last = ++rp == NP;
+            xp += last ? xstep_row : xstep_in;
+            rp = last ? 0 : rp;
         };
         // runs the piece in (ca, cb) and reads the next one into (na, nb): one pair of reads
         // behind every instruction, pinned there (left alone, the scheduler moves the reads
@@ -1366,14 +1356,13 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
             {
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ca[u], cb[u], acc, 0, 0, 0);
                 if (u == 0)
-                    next_piece(); // the address arithmetic of the next piece runs under the first instruction
+                    advance_piece(); // under the first instruction
                 na[u] = ap[4 * u];
                 nb[u] = xp[4 * u * sW];
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
         float a0[QP], b0[QP], a1[QP], b1[QP];
-        next_piece();
 #pragma unroll
         for (int u = 0; u < QP; u++)
         {
@@ -1381,10 +1370,16 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
             b0[u] = xp[4 * u * sW];
         }
         __builtin_amdgcn_sched_barrier(0);
-        for (int p = 0; p < npieces; p += 2)
+        for (int p = 0; p + 1 < npieces; p += 2)
         {
             step_piece(a0, b0, a1, b1);
             step_piece(a1, b1, a0, b0);
+        }
+        if (npieces & 1) // the operands of the last piece are in (a0, b0)
+        {
+#pragma unroll
+            for (int u = 0; u < QP; u++)
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[u], b0[u], acc, 0, 0, 0);
         }
         __syncthreads();
     }
@@ -1579,7 +1574,7 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
             while (cp % 32 != KHW % 32)
                 cp++;
             if (MW_OC * r * OW <= 4 * MW_ST * MW_GS && nic_max * hr * nw4 <= MW_ST * MW_XS &&
-                2 * (64 + MW_OC * gp + nic_max * cp + 3) * 4 <= 150 * 1024)
+                2 * (64 + MW_OC * gp + nic_max * cp + sH * Wp + 64 + 3) * 4 <= 150 * 1024)
             {
                 R = r;
                 hrows = hr;
@@ -1591,7 +1586,8 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
         if (R > 0 && N * (OH / R) <= REPDL_I32_MAX)
         {
             const int64_t xoff = 64 + MW_OC * GP; // 64 zero words, then the grad_output rows, then the input rows
-            const int64_t bufsz = (xoff + nic_max * CP + 3) / 4 * 4; // float4 stores into either buffer
+            // (+ a row of slack: the read behind the last piece of a chunk overshoots by one staged row)
+            const int64_t bufsz = (xoff + nic_max * CP + sH * Wp + 64 + 3) / 4 * 4; // multiple of 4: float4 stores
             const int xvec = aligned16(input) && (W % 4 == 0);
             const int64_t gx = repdl_cdiv(NC, 16), gy = repdl_cdiv(OC, MW_OC);
             REPDL_REQUIRE(fits_i32(gx) && gy <= 65535);
