@@ -449,7 +449,7 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_kernel(const float *__r
 // loop costs matrix time one for one.  Here the loop has none: a global load is a uniform
 // base (advanced per k-tile on the scalar unit) plus a per-thread byte offset that never
 // changes; LDS addresses are per-thread constants plus the buffer offset plus immediates.
-template <bool TA, bool TB, int FM, int FN, int WGM, int WGN>
+template <bool TA, bool TB, int FM, int FN, int WGM, int WGN, bool EDGE>
 __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_fast_kernel(const float *__restrict__ A,
                                                                      const float *__restrict__ B,
                                                                      float *__restrict__ C, int64_t M, int64_t N,
@@ -546,6 +546,101 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_fast_kernel(const float
         a_base += a_step;
         b_base += b_step;
     };
+    // EDGE variant: any M, N, K with 16-byte aligned operands.  A workgroup whose tile lies wholly
+    // inside C loads whole k-tiles as above; tiles on the lower or right edge, and the last
+    // partial k-tile of every workgroup, take predicated loads (rows past the edge are never
+    // stored; k positions past K hold -0.0f in the A tile and +0.0f in the B tile, a bit-exact
+    // no-op, see mm_mfma_kernel).
+    const bool interior = !EDGE || (m0 + TM <= M && n0 + TN <= N);
+    auto load_tiles_guarded = [&](int64_t kt) {
+        if constexpr (EDGE)
+        {
+#pragma unroll
+            for (int i = 0; i < NVA; i++)
+            {
+                const int idx = tid + NTH * i;
+                const int64_t r = m0 + (A_KC ? (idx >> 2) : (idx % (TM / 4)) * 4);
+                const int64_t k = kt * BK + (A_KC ? ((idx & 3) << 2) : idx / (TM / 4));
+                v4f v = {-0.0f, -0.0f, -0.0f, -0.0f};
+                if (A_KC)
+                {
+                    if (r < M)
+                    {
+                        const float *p = A + r * lda + k;
+                        if (k + 3 < K)
+                            v = *reinterpret_cast<const v4f *>(p);
+                        else
+                        {
+                            if (k + 0 < K) v[0] = p[0];
+                            if (k + 1 < K) v[1] = p[1];
+                            if (k + 2 < K) v[2] = p[2];
+                            if (k + 3 < K) v[3] = p[3];
+                        }
+                    }
+                }
+                else if (k < K)
+                {
+                    const float *p = A + k * lda + r;
+                    if (r + 3 < M)
+                        v = *reinterpret_cast<const v4f *>(p);
+                    else
+                    {
+                        if (r + 0 < M) v[0] = p[0];
+                        if (r + 1 < M) v[1] = p[1];
+                        if (r + 2 < M) v[2] = p[2];
+                        if (r + 3 < M) v[3] = p[3];
+                    }
+                }
+                fa[i] = v;
+            }
+#pragma unroll
+            for (int i = 0; i < NVB; i++)
+            {
+                const int idx = tid + NTH * i;
+                const int64_t r = n0 + (B_KC ? (idx >> 2) : (idx % (TN / 4)) * 4);
+                const int64_t k = kt * BK + (B_KC ? ((idx & 3) << 2) : idx / (TN / 4));
+                v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+                if (B_KC)
+                {
+                    if (r < N)
+                    {
+                        const float *p = B + r * ldb + k;
+                        if (k + 3 < K)
+                            v = *reinterpret_cast<const v4f *>(p);
+                        else
+                        {
+                            if (k + 0 < K) v[0] = p[0];
+                            if (k + 1 < K) v[1] = p[1];
+                            if (k + 2 < K) v[2] = p[2];
+                            if (k + 3 < K) v[3] = p[3];
+                        }
+                    }
+                }
+                else if (k < K)
+                {
+                    const float *p = B + k * ldb + r;
+                    if (r + 3 < N)
+                        v = *reinterpret_cast<const v4f *>(p);
+                    else
+                    {
+                        if (r + 0 < N) v[0] = p[0];
+                        if (r + 1 < N) v[1] = p[1];
+                        if (r + 2 < N) v[2] = p[2];
+                        if (r + 3 < N) v[3] = p[3];
+                    }
+                }
+                fb[i] = v;
+            }
+        }
+    };
+    // k-tile kt: whole and inside -> the cheap loads (which also step the bases), else predicated
+    const int64_t nkt_whole = K / BK;
+    auto load_any = [&](int64_t kt) {
+        if (!EDGE || (interior && kt < nkt_whole))
+            load_tiles();
+        else
+            load_tiles_guarded(kt);
+    };
     auto store_tiles = [&](int buf) {
         float *as = As + buf * BK * LDA_, *bs = Bs + buf * BK * LDB_;
 #pragma unroll
@@ -599,10 +694,10 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_fast_kernel(const float
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kp][i], b[kp][j], acc[i][j], 0, 0, 0);
     };
 
-    const int64_t nkt = K / BK;
+    const int64_t nkt = EDGE ? (K + BK - 1) / BK : K / BK;
     if (nkt > 0)
     {
-        load_tiles();
+        load_any(0);
         store_tiles(0);
     }
     __syncthreads();
@@ -611,7 +706,7 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_fast_kernel(const float
         const int cur = (int)(kt & 1);
         const bool more = kt + 1 < nkt;
         if (more)
-            load_tiles();
+            load_any(kt + 1);
         compute(cur);
         if (more)
             store_tiles(cur ^ 1);
@@ -624,9 +719,15 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_fast_kernel(const float
         for (int r = 0; r < 16; r++)
         {
             const int64_t m = m0 + wm * 32 * FM + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3);
+            if (EDGE && m >= M)
+                continue;
 #pragma unroll
             for (int j = 0; j < FN; j++)
-                __builtin_nontemporal_store(acc[i][j][r], &C[m * N + n0 + wn * 32 * FN + 32 * j + l32]);
+            {
+                const int64_t nn = n0 + wn * 32 * FN + 32 * j + l32;
+                if (!EDGE || nn < N)
+                    __builtin_nontemporal_store(acc[i][j][r], &C[m * N + nn]);
+            }
         }
 }
 
@@ -641,12 +742,16 @@ int launch_mfma_t(const float *A, const float *B, float *C, int64_t M, int64_t N
         return REPDL_E_ARG;
     const int64_t ntiles8 = (gx * gy) & ~(int64_t)7;
     const int64_t lda = TA ? M : K, ldb = TB ? K : N;
-    // no bounds checks needed, and every in-tile byte offset fits 32 bits
-    const bool regular = M % TM == 0 && N % TN == 0 && K % BK == 0 && avec && bvec &&
-                         (int64_t)(TM + BK) * lda * 4 < (1LL << 32) && (int64_t)(TN + BK) * ldb * 4 < (1LL << 32);
-    if (regular)
+    // aligned operands whose in-tile byte offsets fit 32 bits: the kernel without address arithmetic
+    // in the loop -- its plain form for whole-tile shapes, its EDGE form (edge tiles and the K tail
+    // predicated) for the rest
+    const bool aligned = avec && bvec && (int64_t)(TM + BK) * lda * 4 < (1LL << 32) &&
+                         (int64_t)(TN + BK) * ldb * 4 < (1LL << 32);
+    const bool whole = M % TM == 0 && N % TN == 0 && K % BK == 0;
+    if (aligned)
     {
-        auto kern = &mm_mfma_fast_kernel<TA, TB, FM, FN, WGM, WGN>;
+        auto kern = whole ? &mm_mfma_fast_kernel<TA, TB, FM, FN, WGM, WGN, false>
+                          : &mm_mfma_fast_kernel<TA, TB, FM, FN, WGM, WGN, true>;
         if (shmem > 48 * 1024)
         {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
