@@ -73,10 +73,13 @@ int repdl_hip_mm(const float *A, const float *B, float *C, int64_t M, int64_t N,
 /* conv2d -- backend/cuda/convolution.cu:153-183 (bound at :385); semantics
  * backend/cpu/convolution.cpp:12-52.  NCHW; kernel is [OC, IC/groups, KH, KW];
  * output is [N, OC, OH, OW] with OH = (H + 2 pH - KH) / sH + 1.
- * Scratch: on the matrix path, conv2d and conv2d_grad_input take a zero-padded copy
- * of their gathered operand plus two small offset tables from the stream-ordered
- * allocator (hipMallocAsync / hipFreeAsync on `stream`; at most the size of that
- * operand with its padding border).  The v_fma_f32 path allocates nothing. */
+ * Scratch: the three convolutions take scratch memory from the stream-ordered
+ * allocator (hipMallocAsync / hipFreeAsync on `stream`): 17 KiB whenever the geometry
+ * makes the reference skip taps (padding, strides of grad-input, kernels wider than one
+ * tap in grad-input); on the matrix path also a zero-padded copy of the gathered operand
+ * of conv2d / conv2d_grad_input with two small offset tables, and for conv2d_grad_kernel
+ * copies of grad_output / input with rows rounded up to a multiple of 4 floats when
+ * their widths are not one.  At most the size of the operands with their borders. */
 int repdl_hip_conv2d(const float *input, const float *kernel, float *output, int64_t N, int64_t IC,
                      int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t sH,
                      int64_t sW, int64_t pH, int64_t pW, int64_t groups, void *stream);

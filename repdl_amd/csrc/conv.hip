@@ -12,12 +12,12 @@
 //     grad-input  C[ic, pixel]  = sum_k W^T[ic, k] * col(GO)[k, pixel],     k = (oc, kh, kw)
 // with k running in exactly the reference's order.  The gathered operand holds a
 // zero where the reference skips a tap.  For finite data fma(0, w, acc) = acc
-// unless acc is -0.0f, and a zero sign can only survive to the end if the final
-// result is itself a zero; with non-finite data the padded product is a NaN that
-// sticks.  So a result that is neither zero nor NaN is already exactly the
-// reference's, and the epilogue recomputes the rare +-0 / NaN results with the
-// literal skip-the-tap chain (the *_exact functions below, which are also the
-// whole of the direct kernels).
+// unless acc is -0.0f, and a chain can hold -0.0f only after a product so small
+// that it rounds to zero; with non-finite data the padded product is a NaN that
+// sticks.  So the epilogue recomputes with the literal skip-the-tap chain (the
+// *_exact functions below, which are also the whole of the direct kernels) every NaN
+// result, and the zero results only when the operands can produce such a product
+// (see "the guard of the zero results" below).
 //
 // grad-kernel has only OC*IC*KH*KW outputs, each a chain as long as the batch
 // (N*OH*OW): it is limited by chain length and parallelism, not by FMA rate.
@@ -138,6 +138,142 @@ __global__ __launch_bounds__(64) void conv2d_grad_kernel_direct(const float *__r
 }
 
 // ---------------------------------------------------------------------------
+// The guard of the zero results.  A chain that multiplies padded zeros where the
+// reference skips a tap can differ from the reference's only while its accumulator
+// is -0.0f (x + (+-0) = x for every other x).  The accumulator starts at +0.0f; an
+// exact cancellation gives +0.0f, and (+0) + (+-0) = +0, so the first -0.0f of a
+// chain can only come from a nonzero sum g*x + acc that rounds to zero.  acc is a
+// multiple of 2^-149, so that needs a product with bits below 2^-149, and a product
+// of two binary32 values has at most 48 significant bits: |g*x| < 2^-101.  If
+//     (smallest nonzero |value| of one operand) * (that of the other) >= 2^-101
+// no such product exists, no chain ever holds -0.0f, and the padded chain equals the
+// literal one on all finite data, zero results included.  guard[0..1] hold the two
+// minima (as bit patterns; GUARD_NONE when an operand has no nonzero value), found
+// in one extra pass over the operands (or in the pass that pads them); the kernels
+// recompute a zero result with the literal chain only when guard_tiny() says a tiny
+// product is possible, and a NaN result always (0 * inf of a padded tap).
+// Without it, data with whole dead channels or zero borders (every ReLU network)
+// sent each of its zero results through a serial literal chain.
+// ---------------------------------------------------------------------------
+constexpr unsigned GUARD_NONE = 0x7f800000u;
+// Workspace of the guard: words 0 and 1 are the two minima, then (from word 64) GUARD_PARTS
+// per-workgroup minima for each operand.  No atomics: thousands of them on one address
+// would cost more than the pass itself.
+constexpr int GUARD_PARTS = 2048;
+constexpr size_t GUARD_BYTES = (64 + 2 * GUARD_PARTS) * sizeof(unsigned);
+static_assert(GUARD_BYTES % 256 == 0, "what follows the guard in a workspace stays aligned");
+
+inline unsigned *guard_parts(unsigned *guard, int operand) { return guard + 64 + operand * GUARD_PARTS; }
+
+__device__ __forceinline__ unsigned guard_bits(float v)
+{
+    const unsigned b = __float_as_uint(v) & 0x7fffffffu;
+    return b == 0u ? GUARD_NONE : b; // NaN patterns are above GUARD_NONE and never the minimum
+}
+
+__device__ __forceinline__ unsigned guard_min(unsigned a, unsigned b) { return b < a ? b : a; }
+
+// Minimum over the 256 threads of a workgroup (all of them call), valid in thread 0.
+__device__ __forceinline__ unsigned guard_block_min(unsigned m)
+{
+    __shared__ unsigned wave_min[4];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        m = guard_min(m, (unsigned)__shfl_xor((int)m, o));
+    __syncthreads(); // a previous use of wave_min has been read
+    if ((threadIdx.x & 63) == 0)
+        wave_min[threadIdx.x >> 6] = m;
+    __syncthreads();
+    return guard_min(guard_min(wave_min[0], wave_min[1]), guard_min(wave_min[2], wave_min[3]));
+}
+
+// A null guard: the geometry skips no tap (no padding, whole rows), nothing to decide.
+__device__ __forceinline__ bool guard_tiny(const unsigned *__restrict__ guard)
+{
+    return guard != nullptr && (double)__uint_as_float(guard[0]) * (double)__uint_as_float(guard[1]) < 0x1p-101;
+}
+
+__device__ __forceinline__ bool guard_suspect(float v, bool tiny)
+{
+    return (v != v) || (tiny && (__float_as_uint(v) << 1) == 0u);
+}
+
+// Blocks [0, nblk_a) take the minimum over a[0..na) into the parts of operand 0, the
+// others over b[0..nb) into those of operand 1; either range of blocks may be empty.
+__global__ __launch_bounds__(256) void conv_guard_kernel(const float *__restrict__ a, int64_t na,
+                                                         const float *__restrict__ b, int64_t nb, int nblk_a,
+                                                         unsigned *__restrict__ parts_a,
+                                                         unsigned *__restrict__ parts_b)
+{
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    const bool second = (int)blockIdx.x >= nblk_a;
+    const float *__restrict__ p = second ? b : a;
+    const int64_t n = second ? nb : na;
+    const int blk = second ? (int)blockIdx.x - nblk_a : (int)blockIdx.x;
+    const int64_t stride = (int64_t)(second ? (int)gridDim.x - nblk_a : nblk_a) * 256;
+    const int64_t first = (int64_t)blk * 256 + threadIdx.x;
+    unsigned m = GUARD_NONE;
+    int64_t done = 0;
+    if ((reinterpret_cast<uintptr_t>(p) & 15) == 0)
+    {
+        const v4f *__restrict__ p4 = reinterpret_cast<const v4f *>(p);
+        const int64_t n4 = n / 4;
+        for (int64_t i = first; i < n4; i += stride)
+        {
+            const v4f v = p4[i];
+            m = guard_min(guard_min(m, guard_bits(v.x)),
+                          guard_min(guard_bits(v.y), guard_min(guard_bits(v.z), guard_bits(v.w))));
+        }
+        done = n4 * 4;
+    }
+    for (int64_t i = done + first; i < n; i += stride)
+        m = guard_min(m, guard_bits(p[i]));
+    m = guard_block_min(m);
+    if (threadIdx.x == 0)
+        (second ? parts_b : parts_a)[blk] = m;
+}
+
+// guard[op] = minimum of the first count[op] parts of operand op (GUARD_NONE for none)
+__global__ __launch_bounds__(256) void conv_guard_final_kernel(unsigned *__restrict__ guard, int count_a, int count_b)
+{
+#pragma unroll
+    for (int op = 0; op < 2; op++)
+    {
+        const unsigned *__restrict__ parts = guard + 64 + op * GUARD_PARTS;
+        const int count = op == 0 ? count_a : count_b;
+        unsigned m = GUARD_NONE;
+        for (int i = threadIdx.x; i < count; i += 256)
+            m = guard_min(m, parts[i]);
+        m = guard_block_min(m);
+        if (threadIdx.x == 0)
+            guard[op] = m;
+    }
+}
+
+inline int guard_blocks(int64_t n)
+{
+    const int64_t b = (n + 4095) / 4096; // 16 values per thread
+    return (int)(b < 1 ? 1 : (b > 1024 ? 1024 : b));
+}
+
+// Scans the operands given (a null one is left to the padding pass of its caller, which
+// then sets its own count of parts); returns the counts of parts written.
+inline void launch_guard_scan(const float *a, int64_t na, const float *b, int64_t nb, unsigned *guard, hipStream_t s,
+                              int &count_a, int &count_b)
+{
+    count_a = a ? guard_blocks(na) : 0;
+    count_b = b ? guard_blocks(nb) : 0;
+    if (count_a + count_b > 0)
+        hipLaunchKernelGGL(conv_guard_kernel, dim3((unsigned)(count_a + count_b)), dim3(256), 0, s, a, a ? na : 0, b,
+                           b ? nb : 0, count_a, guard_parts(guard, 0), guard_parts(guard, 1));
+}
+
+inline void launch_guard_final(unsigned *guard, int count_a, int count_b, hipStream_t s)
+{
+    hipLaunchKernelGGL(conv_guard_final_kernel, dim3(1), dim3(256), 0, s, guard, count_a, count_b);
+}
+
+// ---------------------------------------------------------------------------
 // Implicit GEMM for forward (MODE_FWD) and grad-input (MODE_DGRAD).
 // Tile BM x 128 outputs (BM = 64 or 128 rows = output / input channels, 128
 // columns = pixels of one image), BK = 16, 2*BM threads, 8x8 micro-tile per lane.
@@ -184,7 +320,7 @@ template <int BM, int MODE, bool MFMA>
 __global__ __launch_bounds__(2 * BM) void conv_gemm_kernel(const float *__restrict__ Xg, // gathered operand: input (FWD) / grad_output (DGRAD)
                                                            const float *__restrict__ Wt, // kernel
                                                            float *__restrict__ Out, ConvDims d, int wvec,
-                                                           int ovec)
+                                                           int ovec, const unsigned *__restrict__ guard)
 {
     constexpr int NT = 2 * BM;
     constexpr int LDA = BM + 4;
@@ -449,6 +585,7 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_kernel(const float *__restri
             __syncthreads();
         }
         // register r of a block: row 8*(r/4) + 4*(lane/32) + r%4, pixel lane%32
+        const bool tiny = guard_tiny(guard);
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -465,7 +602,7 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_kernel(const float *__restri
                     if (pix >= P)
                         continue;
                     float v = acc[i][j][r];
-                    if (((__float_as_uint(v) << 1) == 0u) || (v != v))
+                    if (guard_suspect(v, tiny))
                     {
                         const int ph = pix / PW, pw = pix - ph * PW;
                         v = MODE == MODE_FWD ? conv2d_exact(Xg, Wt, d, n, ch, ph, pw)
@@ -535,7 +672,8 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_kernel(const float *__restri
             __syncthreads();
         }
 
-        // ---- epilogue: exact recompute of +-0 / NaN results, then store ----
+        // ---- epilogue: literal recompute of the suspect results (see the guard), then store ----
+        const bool tiny = guard_tiny(guard);
 #pragma unroll
         for (int i = 0; i < 8; i++)
         {
@@ -552,7 +690,7 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_kernel(const float *__restri
                 for (int j = 0; j < 4; j++)
                 {
                     v[j] = acc[i][jh * 4 + j];
-                    const bool suspect = ((__float_as_uint(v[j]) << 1) == 0u) || (v[j] != v[j]);
+                    const bool suspect = guard_suspect(v[j], tiny);
                     if (suspect && pix + j < P)
                     {
                         const int ph = (pix + j) / PW, pw = (pix + j) - ph * PW;
@@ -596,17 +734,31 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_kernel(const float *__restri
 // epilogue.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void conv_pad_kernel(const float *__restrict__ src, float *__restrict__ dst,
-                                                       int64_t total, int H, int W, int Hp, int Wp, int PT, int PL)
+                                                       int64_t total, int H, int W, int Hp, int Wp, int PT, int PL,
+                                                       unsigned *__restrict__ parts)
 {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= total)
-        return;
-    const int wp = (int)(idx % Wp);
-    const int64_t t = idx / Wp;
-    const int hp = (int)(t % Hp);
-    const int64_t pl = t / Hp;
-    const int h = hp - PT, w = wp - PL;
-    dst[idx] = (h >= 0 && h < H && w >= 0 && w < W) ? src[(pl * H + h) * W + w] : 0.0f;
+    // grid-stride: at most GUARD_PARTS workgroups, each leaves the minimum of what it copied
+    unsigned m = GUARD_NONE;
+    for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256)
+    {
+        const int wp = (int)(idx % Wp);
+        const int64_t t = idx / Wp;
+        const int hp = (int)(t % Hp);
+        const int64_t pl = t / Hp;
+        const int h = hp - PT, w = wp - PL;
+        const float v = (h >= 0 && h < H && w >= 0 && w < W) ? src[(pl * H + h) * W + w] : 0.0f;
+        dst[idx] = v;
+        m = guard_min(m, guard_bits(v));
+    }
+    m = guard_block_min(m);
+    if (threadIdx.x == 0)
+        parts[blockIdx.x] = m;
+}
+
+inline unsigned pad_blocks(int64_t total)
+{
+    const int64_t b = (total + 255) / 256;
+    return (unsigned)(b < 1 ? 1 : (b > GUARD_PARTS ? GUARD_PARTS : b)); // 2048 x 256 threads fill the chip
 }
 
 __global__ __launch_bounds__(256) void conv_ktab_kernel(int *__restrict__ tabB, int *__restrict__ tabA, int K, int KH,
@@ -634,7 +786,7 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
                                                                 const float *__restrict__ Wt, float *__restrict__ Out,
                                                                 ConvDims d, const int *__restrict__ tabB,
                                                                 const int *__restrict__ tabA, int plane, int Wp,
-                                                                int64_t img_stride)
+                                                                int64_t img_stride, const unsigned *__restrict__ guard)
 {
     constexpr int NT = 2 * BM;
     constexpr int LDA = BM + 4;
@@ -787,6 +939,7 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
     }
 
     float *Oimg = Out + (int64_t)n * (MODE == MODE_FWD ? d.OC : d.IC) * P;
+    const bool tiny = guard_tiny(guard);
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -801,7 +954,7 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
                 if (pix >= P)
                     continue;
                 float v = acc[i][j][r];
-                if (((__float_as_uint(v) << 1) == 0u) || (v != v))
+                if (guard_suspect(v, tiny))
                 {
                     const int ph = pix / PW, pw = pix - ph * PW;
                     v = MODE == MODE_FWD ? conv2d_exact(Xg, Wt, d, n, ch, ph, pw)
@@ -949,7 +1102,8 @@ template <int PIECE>
 __global__ __launch_bounds__(256) void conv_wgrad_kernel(const float *__restrict__ GO,
                                                          const float *__restrict__ X,
                                                          float *__restrict__ GK, ConvDims d, int R, int NP,
-                                                         int Wp, int CP, int hrows, int bufsz, int xvec)
+                                                         int Wp, int CP, int hrows, int bufsz, int xvec,
+                                                         const unsigned *__restrict__ guard)
 {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -1142,7 +1296,7 @@ __global__ __launch_bounds__(256) void conv_wgrad_kernel(const float *__restrict
     }
     if (ovalid && cvalid)
     {
-        if (((__float_as_uint(acc) << 1) == 0u) || (acc != acc))
+        if (guard_suspect(acc, guard_tiny(guard)))
             acc = conv2d_grad_kernel_exact(GO, X, d, oc, ic, kh, kw);
         GK[(int64_t)oc * NC + col] = acc;
     }
@@ -1172,8 +1326,11 @@ __global__ __launch_bounds__(256) void conv_wgrad_kernel(const float *__restrict
 // instruction, grad_output of oc l%16 and the tap of column l%16, both at step l/16.
 // Operands are read a piece (QP instructions) ahead.  Out-of-image taps read staged
 // zeros, so +-0 / NaN results are recomputed with the literal chain, as everywhere
-// in this file.  Requires OW % (4 QP) == 0, OH % R == 0, W % 4 == 0 and 16-byte aligned
-// grad_output and input; other shapes take conv_wgrad_kernel.
+// in this file.  Widths that are not multiples of 4 are first rounded up in copies whose rows
+// end in zeros (conv_pad_kernel): for grad_output the added steps multiply a zero, for the
+// input the added columns fall into the zero pad of the staged rows.
+// Requires OH % R == 0 and 16-byte aligned grad_output and input; other shapes take
+// conv_wgrad_kernel.
 // ---------------------------------------------------------------------------
 typedef float f4v __attribute__((ext_vector_type(4)));
 constexpr int MW_GS = 16; // float4 staging slots of grad_output per staging thread
@@ -1182,11 +1339,13 @@ constexpr int MW_OC = 32; // oc per workgroup
 constexpr int MW_ST = 128; // staging threads
 
 template <int QP, bool UNIT, int XS> // QP: instructions per piece; XS: input staging slots per thread
-__global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__restrict__ GO,
+__global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__restrict__ GOs, // grad_output, rows of 4*QP*NP floats
+                                                              const float *__restrict__ Xs,  // input, rows of xW floats
+                                                              const float *__restrict__ GO,  // both as given (epilogue)
                                                               const float *__restrict__ X,
                                                               float *__restrict__ GK, ConvDims d, int R, int NP,
                                                               int GP, int Wp, int CP, int hrows, int xoff, int bufsz,
-                                                              int xvec)
+                                                              int xW, const unsigned *__restrict__ guard)
 {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int tid = threadIdx.x;
@@ -1195,7 +1354,7 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
     const int c0 = blockIdx.x * 16;
     const int ic_first = c0 / KHW;
     const int oc0 = blockIdx.y * MW_OC;
-    const int OWp = 4 * QP * NP; // = OW
+    const int OWp = 4 * QP * NP; // steps per output row: OW, or OW rounded up to 4 in a zero-padded copy
     const int nchunks = d.N * (d.OH / R);
 
     for (int i = tid; i < 2 * bufsz; i += 256)
@@ -1211,7 +1370,7 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
         // same values), so that no load or store sits behind a branch or a mask (the compiler waits
         // for every outstanding load where branches that contain loads merge).
         // Input: slot = (staged row, 4 floats of it); W % 4 == 0 and 16-byte alignment are given.
-        const int nw4 = d.W >> 2;
+        const int nw4 = xW >> 2;
         const int nxs = nic * hrows * nw4;
         int x_goff[XS], x_hr[XS], x_loff[XS];
 #pragma unroll
@@ -1221,12 +1380,12 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
             s = s < nxs ? s : nxs - 1;
             const int row = s / nw4, w = (s - row * nw4) << 2;
             const int icl = row / hrows, hr = row - icl * hrows;
-            x_goff[i] = (ic_first + icl) * d.H * d.W + w;
+            x_goff[i] = (ic_first + icl) * d.H * xW + w;
             x_hr[i] = hr;
             x_loff[i] = xoff + icl * CP + hr * Wp + d.pW + w;
         }
         // grad_output: slot = (oc, 4 consecutive steps of the chunk)
-        const int spo = (R * d.OW) >> 2; // float4 per oc and chunk
+        const int spo = (R * OWp) >> 2; // float4 per oc and chunk
         uint32_t g_goff[MW_GS];
         int g_loff[MW_GS];
 #pragma unroll
@@ -1236,12 +1395,12 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
             s = s < MW_OC * spo ? s : MW_OC * spo - 1;
             const int o = s / spo, t = (s - o * spo) << 2;
             const int oc = oc0 + o < d.OC ? oc0 + o : d.OC - 1; // rows of missing oc repeat the last one
-            g_goff[i] = (uint32_t)((oc - oc0) * d.OH * d.OW + t) * 4u;
+            g_goff[i] = (uint32_t)((oc - oc0) * d.OH * OWp + t) * 4u;
             g_loff[i] = 64 + o * GP + t;
         }
         f4v xst[XS], gst[MW_GS]; // plain vectors: they must stay in registers
         auto chunk_load = [&](int n, int oh0) {
-            const float *Xn = X + (int64_t)n * d.IC * d.H * d.W;
+            const float *Xn = Xs + (int64_t)n * d.IC * d.H * xW;
             const int hbase = oh0 * d.sH - d.pH;
 #pragma unroll
             for (int i = 0; i < XS; i++)
@@ -1249,13 +1408,13 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
                     const int h = hbase + x_hr[i];
                     const bool ok = h >= 0 && h < d.H;
                     const int hc = h < 0 ? 0 : (h >= d.H ? d.H - 1 : h);
-                    const f4v v = *reinterpret_cast<const f4v *>(Xn + x_goff[i] + hc * d.W);
+                    const f4v v = *reinterpret_cast<const f4v *>(Xn + x_goff[i] + hc * xW);
                     xst[i][0] = ok ? v[0] : 0.0f;
                     xst[i][1] = ok ? v[1] : 0.0f;
                     xst[i][2] = ok ? v[2] : 0.0f;
                     xst[i][3] = ok ? v[3] : 0.0f;
                 }
-            const char *Gn = reinterpret_cast<const char *>(GO + (((int64_t)n * d.OC + oc0) * d.OH + oh0) * d.OW);
+            const char *Gn = reinterpret_cast<const char *>(GOs + (((int64_t)n * d.OC + oc0) * d.OH + oh0) * OWp);
 #pragma unroll
             for (int i = 0; i < MW_GS; i++)
                 gst[i] = *reinterpret_cast<const f4v *>(Gn + g_goff[i]);
@@ -1384,6 +1543,7 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
         __syncthreads();
     }
     // register r of the block: oc 4*(lane/16) + r of the wave's 16, column lane%16
+    const bool tiny = guard_tiny(guard);
 #pragma unroll
     for (int r = 0; r < 4; r++)
     {
@@ -1391,7 +1551,7 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
         if (oc < d.OC && col < NC)
         {
             float v = acc[r];
-            if (((__float_as_uint(v) << 1) == 0u) || (v != v))
+            if (guard_suspect(v, tiny))
                 v = conv2d_grad_kernel_exact(GO, X, d, oc, ic, kh, kw);
             GK[(int64_t)oc * NC + col] = v;
         }
@@ -1415,6 +1575,13 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
     const int ovec = aligned16(out) && (P % 4 == 0);
     hipStream_t s = repdl_stream(stream);
     const bool mfma = repdl_mfma_exact();
+    const int64_t gathered_count =
+        (int64_t)d.N * (MODE == MODE_FWD ? (int64_t)d.IC * d.H * d.W : (int64_t)d.OC * d.OH * d.OW);
+    const int64_t kernel_count = (int64_t)d.OC * (d.IC / d.groups) * KHW;
+    // does the reference skip any tap?  (forward: only into the padding; grad-input: at the
+    // borders of any kernel wider than one tap, and between strides)
+    const bool skips = MODE == MODE_FWD ? (d.pH > 0 || d.pW > 0)
+                                        : (KHW > 1 || d.sH > 1 || d.sW > 1 || d.pH > 0 || d.pW > 0);
     // Fast path: whole tiles of channels, whole k-tiles, grad-input only at stride 1.
     const int bm = M <= 64 ? 64 : 128;
     if (mfma && K % BK == 0 && M % bm == 0 && (MODE == MODE_FWD || (d.sH == 1 && d.sW == 1)))
@@ -1428,53 +1595,78 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
         if (img * 4 < (1LL << 31) && (int64_t)M * K * 4 < (1LL << 31) && (int64_t)d.N * img / 256 < REPDL_I32_MAX)
         {
             const bool pad = PT > 0 || PL > 0;
+            // workspace: the guard words, the two tables, the padded copy
             const size_t tab_bytes = ((size_t)2 * K * sizeof(int) + 255) / 256 * 256;
-            const size_t ws_bytes = tab_bytes + (pad ? (size_t)d.N * img * sizeof(float) : 0);
+            const size_t ws_bytes = GUARD_BYTES + tab_bytes + (pad ? (size_t)d.N * img * sizeof(float) : 0);
             char *ws = nullptr;
             hipError_t e = hipMallocAsync(reinterpret_cast<void **>(&ws), ws_bytes, s);
             if (e != hipSuccess)
                 return (int)e;
-            int *tabB = reinterpret_cast<int *>(ws), *tabA = tabB + K;
-            float *Gp = reinterpret_cast<float *>(ws + tab_bytes);
+            unsigned *guard = reinterpret_cast<unsigned *>(ws);
+            int *tabB = reinterpret_cast<int *>(ws + GUARD_BYTES), *tabA = tabB + K;
+            float *Gp = reinterpret_cast<float *>(ws + GUARD_BYTES + tab_bytes);
+            // guard[0]: the gathered operand (in the padding pass when there is one), guard[1]: the kernel
+            int ca = 0, cb = 0;
+            if (skips)
+                launch_guard_scan(pad ? nullptr : gathered, gathered_count, kernel, kernel_count, guard, s, ca, cb);
+            else
+                guard = nullptr;
             hipLaunchKernelGGL(conv_ktab_kernel, dim3((unsigned)repdl_cdiv(K, 256)), dim3(256), 0, s, tabB, tabA, (int)K,
                                d.KH, d.KW, (int)plane, (int)Wp, MODE, d.IC, d.pH + PT, d.pW + PL);
             if (pad)
             {
                 const int64_t total = (int64_t)d.N * img;
-                hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)repdl_cdiv(total, 256)), dim3(256), 0, s, gathered, Gp,
-                                   total, GH, GW, (int)Hp, (int)Wp, PT, PL);
+                ca = (int)pad_blocks(total);
+                hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)ca), dim3(256), 0, s, gathered, Gp, total, GH, GW,
+                                   (int)Hp, (int)Wp, PT, PL, guard_parts(guard, 0));
             }
+            if (skips)
+                launch_guard_final(guard, ca, cb, s);
             const float *src = pad ? Gp : gathered;
             dim3 grid((unsigned)gx, (unsigned)(M / bm), (unsigned)gz);
             if (bm == 64)
                 hipLaunchKernelGGL((conv_gemm_fast_kernel<64, MODE>), grid, dim3(128), 0, s, src, gathered, kernel, out, d, tabB,
-                                   tabA, (int)plane, (int)Wp, img);
+                                   tabA, (int)plane, (int)Wp, img, guard);
             else
                 hipLaunchKernelGGL((conv_gemm_fast_kernel<128, MODE>), grid, dim3(256), 0, s, src, gathered, kernel, out, d,
-                                   tabB, tabA, (int)plane, (int)Wp, img);
+                                   tabB, tabA, (int)plane, (int)Wp, img, guard);
             const int rc = repdl_launch_status();
             e = hipFreeAsync(ws, s);
             return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
         }
     }
+    REPDL_REQUIRE(repdl_cdiv(M, 128) <= 65535);
+    unsigned *guard = nullptr;
+    hipError_t ge = hipSuccess;
+    if (skips)
+    {
+        ge = hipMallocAsync(reinterpret_cast<void **>(&guard), GUARD_BYTES, s);
+        if (ge != hipSuccess)
+            return (int)ge;
+        int ca = 0, cb = 0;
+        launch_guard_scan(gathered, gathered_count, kernel, kernel_count, guard, s, ca, cb);
+        launch_guard_final(guard, ca, cb, s);
+    }
     if (M <= 64)
     {
         dim3 grid((unsigned)gx, (unsigned)repdl_cdiv(M, 64), (unsigned)gz);
         if (mfma)
-            hipLaunchKernelGGL((conv_gemm_kernel<64, MODE, true>), grid, dim3(128), 0, s, gathered, kernel, out, d, wvec, ovec);
+            hipLaunchKernelGGL((conv_gemm_kernel<64, MODE, true>), grid, dim3(128), 0, s, gathered, kernel, out, d, wvec, ovec, guard);
         else
-            hipLaunchKernelGGL((conv_gemm_kernel<64, MODE, false>), grid, dim3(128), 0, s, gathered, kernel, out, d, wvec, ovec);
+            hipLaunchKernelGGL((conv_gemm_kernel<64, MODE, false>), grid, dim3(128), 0, s, gathered, kernel, out, d, wvec, ovec, guard);
     }
     else
     {
         dim3 grid((unsigned)gx, (unsigned)repdl_cdiv(M, 128), (unsigned)gz);
-        REPDL_REQUIRE(grid.y <= 65535);
         if (mfma)
-            hipLaunchKernelGGL((conv_gemm_kernel<128, MODE, true>), grid, dim3(256), 0, s, gathered, kernel, out, d, wvec, ovec);
+            hipLaunchKernelGGL((conv_gemm_kernel<128, MODE, true>), grid, dim3(256), 0, s, gathered, kernel, out, d, wvec, ovec, guard);
         else
-            hipLaunchKernelGGL((conv_gemm_kernel<128, MODE, false>), grid, dim3(256), 0, s, gathered, kernel, out, d, wvec, ovec);
+            hipLaunchKernelGGL((conv_gemm_kernel<128, MODE, false>), grid, dim3(256), 0, s, gathered, kernel, out, d, wvec, ovec, guard);
     }
-    return repdl_launch_status();
+    const int rc = repdl_launch_status();
+    if (skips)
+        ge = hipFreeAsync(guard, s);
+    return rc != REPDL_OK ? rc : (ge == hipSuccess ? REPDL_OK : (int)ge);
 }
 } // namespace
 
@@ -1539,13 +1731,16 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
     hipStream_t s = repdl_stream(stream);
 
     // Matrix-instruction kernel: geometry of a chunk (see conv_wgrad_mfma_kernel).
-    if (repdl_mfma_exact() && OW % 4 == 0 && W % 4 == 0 && sW <= 16 && aligned16(grad_output) && aligned16(input))
+    if (repdl_mfma_exact() && sW <= 16 && aligned16(grad_output) && aligned16(input) && OW > 0)
     {
         const int64_t KHW = KH * KW, NC = IC * KHW;
-        // instructions per piece: the largest candidate that divides a row of OW / 4 instructions
-        const int64_t nqr = OW / 4;
+        // instructions per piece: the largest candidate that divides a row of OWr / 4 instructions
+        // (OWr: the output width, rounded up to a multiple of 4 in a zero-padded copy of grad_output)
+        const int64_t OWr = (OW + 3) / 4 * 4;
+        const bool gpad = OWr != OW;
+        const int64_t nqr = OWr / 4;
         int64_t QP = 0, NP = 0;
-        for (int64_t qp : {16, 14, 7, 4})
+        for (int64_t qp : {16, 14, 7, 4, 2, 1})
             if (QP == 0 && nqr % qp == 0)
             {
                 QP = qp;
@@ -1573,7 +1768,7 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
             int64_t cp = hr * Wp;
             while (cp % 32 != KHW % 32)
                 cp++;
-            if (MW_OC * r * OW <= 4 * MW_ST * MW_GS && nic_max * hr * nw4 <= MW_ST * MW_XS &&
+            if (MW_OC * r * OWp <= 4 * MW_ST * MW_GS && nic_max * hr * nw4 <= MW_ST * MW_XS &&
                 2 * (64 + MW_OC * gp + nic_max * cp + sH * Wp + 64 + 3) * 4 <= 150 * 1024)
             {
                 R = r;
@@ -1583,14 +1778,52 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
                 break;
             }
         }
-        if (R > 0 && N * (OH / R) <= REPDL_I32_MAX)
+        const int64_t xW = (W + 3) / 4 * 4; // input row pitch the staging waves read
+        const bool xpad = xW != W;
+        if (R > 0 && N * (OH / R) <= REPDL_I32_MAX && fits_i32(IC * H * xW) && fits_i32(repdl_cdiv(NC, 16)) &&
+            repdl_cdiv(OC, MW_OC) <= 65535)
         {
+            // workspace: the guard words, then the operands with rows rounded up to whole
+            // instructions (grad_output) / whole float4 (input), when they are not
+            const size_t xbytes = xpad ? ((size_t)(N * IC * H * xW) * sizeof(float) + 255) / 256 * 256 : 0;
+            const size_t gbytes = gpad ? (size_t)(N * OC * OH * OWp) * sizeof(float) : 0;
+            char *ws = nullptr;
+            hipError_t e = hipMallocAsync(reinterpret_cast<void **>(&ws), GUARD_BYTES + xbytes + gbytes, s);
+            if (e != hipSuccess)
+                return (int)e;
+            unsigned *guard = reinterpret_cast<unsigned *>(ws);
+            float *xws = reinterpret_cast<float *>(ws + GUARD_BYTES);
+            float *gws = reinterpret_cast<float *>(ws + GUARD_BYTES + xbytes);
+            // the reference skips taps only into the padding; rows rounded up add zero steps
+            const bool skips = pH > 0 || pW > 0 || gpad;
+            int ca = 0, cb = 0;
+            if (skips)
+                launch_guard_scan(gpad ? nullptr : grad_output, N * OC * OH * OW, xpad ? nullptr : input, N * IC * H * W, guard,
+                                  s, ca, cb);
+            if (xpad)
+            {
+                const int64_t total = N * IC * H * xW;
+                cb = (int)pad_blocks(total);
+                hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)cb), dim3(256), 0, s, input, xws, total, (int)H, (int)W,
+                                   (int)H, (int)xW, 0, 0, guard_parts(guard, 1));
+            }
+            const float *xsrc = xpad ? xws : input;
+            if (gpad)
+            {
+                const int64_t total = N * OC * OH * OWp;
+                ca = (int)pad_blocks(total);
+                hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)ca), dim3(256), 0, s, grad_output, gws, total, (int)OH,
+                                   (int)OW, (int)OH, (int)OWp, 0, 0, guard_parts(guard, 0));
+            }
+            if (skips)
+                launch_guard_final(guard, ca, cb, s);
+            else
+                guard = nullptr;
+            const float *gsrc = gpad ? gws : grad_output;
             const int64_t xoff = 64 + MW_OC * GP; // 64 zero words, then the grad_output rows, then the input rows
             // (+ a row of slack: the read behind the last piece of a chunk overshoots by one staged row)
             const int64_t bufsz = (xoff + nic_max * CP + sH * Wp + 64 + 3) / 4 * 4; // multiple of 4: float4 stores
-            const int xvec = aligned16(input) && (W % 4 == 0);
             const int64_t gx = repdl_cdiv(NC, 16), gy = repdl_cdiv(OC, MW_OC);
-            REPDL_REQUIRE(fits_i32(gx) && gy <= 65535);
             size_t shmem = (size_t)(2 * bufsz * 4);
             if (shmem < 84 * 1024)
                 shmem = 84 * 1024; // one workgroup per CU: every wave has a SIMD to itself
@@ -1601,10 +1834,13 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
         hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_wgrad_mfma_kernel<Q, U, X>),       \
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);                \
         if (e_ != hipSuccess)                                                                                       \
+        {                                                                                                           \
+            (void)hipFreeAsync(ws, s);                                                                              \
             return (int)e_;                                                                                         \
+        }                                                                                                           \
         hipLaunchKernelGGL((conv_wgrad_mfma_kernel<Q, U, X>), dim3((unsigned)gx, (unsigned)gy), dim3(256), shmem, s, \
-                           grad_output, input, grad_kernel, d, (int)R, (int)NP, (int)GP, (int)Wp, (int)CP,          \
-                           (int)hrows, (int)xoff, (int)bufsz, xvec);                                                \
+                           gsrc, xsrc, grad_output, input, grad_kernel, d, (int)R, (int)NP, (int)GP, (int)Wp,       \
+                           (int)CP, (int)hrows, (int)xoff, (int)bufsz, (int)xW, guard);                             \
     } while (0)
 #define REPDL_WGRAD_MFMA_Q(Q)                     \
     do                                            \
@@ -1624,11 +1860,17 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
                 REPDL_WGRAD_MFMA_Q(14);
             else if (QP == 7)
                 REPDL_WGRAD_MFMA_Q(7);
-            else
+            else if (QP == 4)
                 REPDL_WGRAD_MFMA_Q(4);
+            else if (QP == 2)
+                REPDL_WGRAD_MFMA_Q(2);
+            else
+                REPDL_WGRAD_MFMA_Q(1);
 #undef REPDL_WGRAD_MFMA_Q
 #undef REPDL_WGRAD_MFMA
-            return repdl_launch_status();
+            const int rc = repdl_launch_status();
+            e = hipFreeAsync(ws, s);
+            return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
         }
     }
 
@@ -1672,6 +1914,13 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
     const int64_t gx = repdl_cdiv(NC, 64), gy = repdl_cdiv(OC, 4);
     REPDL_REQUIRE(fits_i32(gx) && gy <= 65535);
     const dim3 grid((unsigned)gx, (unsigned)gy);
+    unsigned *guard = nullptr;
+    hipError_t ge = hipMallocAsync(reinterpret_cast<void **>(&guard), GUARD_BYTES, s);
+    if (ge != hipSuccess)
+        return (int)ge;
+    int ca = 0, cb = 0;
+    launch_guard_scan(grad_output, N * OC * OH * OW, input, N * IC * H * W, guard, s, ca, cb);
+    launch_guard_final(guard, ca, cb, s);
     // More than half of a CU's 160 KiB of LDS: one workgroup per CU, so that each of its
     // four waves has a SIMD to itself (the chains are latency-bound, not throughput-bound).
     size_t shmem = (size_t)(2 * bufsz * 4);
@@ -1683,9 +1932,12 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
         hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_wgrad_kernel<P>),             \
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);           \
         if (e_ != hipSuccess)                                                                                  \
+        {                                                                                                      \
+            (void)hipFreeAsync(guard, s);                                                                      \
             return (int)e_;                                                                                    \
+        }                                                                                                      \
         hipLaunchKernelGGL((conv_wgrad_kernel<P>), grid, dim3(256), shmem, s, grad_output, input, grad_kernel, \
-                           d, (int)R, (int)NP, (int)Wp, (int)CP, (int)hrows, (int)bufsz, xvec);                \
+                           d, (int)R, (int)NP, (int)Wp, (int)CP, (int)hrows, (int)bufsz, xvec, guard);         \
     } while (0)
     if (piece == 16)
         REPDL_WGRAD(16);
@@ -1694,5 +1946,7 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
     else
         REPDL_WGRAD(64);
 #undef REPDL_WGRAD
-    return repdl_launch_status();
+    const int rc = repdl_launch_status();
+    ge = hipFreeAsync(guard, s);
+    return rc != REPDL_OK ? rc : (ge == hipSuccess ? REPDL_OK : (int)ge);
 }

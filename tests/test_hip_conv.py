@@ -1,9 +1,12 @@
 """GPU parity of the three convolutions against the oracle beyond the golden cases: shapes
 that take the matrix-instruction kernels' fast paths (whole channel tiles, K a multiple of
-16, padded-workspace gather; grad-kernel with OW a multiple of 16 or 28) and shapes that
-fall back, strides, paddings larger and smaller than the kernel reach, groups, pixels that
-do not fill the last tile, and data that forces the exact recomputation of zero / NaN
-results (ReLU zeros, signed zeros, infinities)."""
+16, padded-workspace gather; grad-kernel with every piece length, with widths that are
+not multiples of 4 and with strides) and shapes that fall back, strides, paddings larger
+and smaller than the kernel reach, groups, pixels that do not fill the last tile, and three
+kinds of data: plain (ReLU zeros: zero results that the padded chains already get right),
+"special" (signed zeros and infinities: NaN results are recomputed with the literal chain)
+and "tiny" (products that underflow to -0.0f: the guard of the zero results must send them
+through the literal chain, while whole dead channels stay exact zeros)."""
 import pytest
 import torch
 
@@ -28,7 +31,9 @@ def _data(shape, seed, special):
     N, IC, H, W, OC, KH, KW, sH, sW, pH, pW, g = shape
     x = gen.relu_like(seed, N, IC, H, W)
     w = gen.normal_like(seed + 1, OC, IC // g, KH, KW)
-    if special:
+    if special == "tiny":
+        x, w = _tiny(x, 0), _tiny(w, 0)
+    elif special:
         x.view(-1)[::97] = float("inf")
         x.view(-1)[5::211] = -0.0
         w.view(-1)[::53] = 0.0
@@ -36,12 +41,32 @@ def _data(shape, seed, special):
     return x, w
 
 
+def _tiny(t, dim):
+    """The slices of even index along `dim` scaled to about 1e-25 with mixed signs: where two
+    such slices meet in a chain every product underflows to +-0 and the result is a zero
+    whose sign depends on the taps that were skipped."""
+    t = t.clone()
+    flat = t.view(-1)
+    scale = torch.full_like(flat, 1e-25)
+    scale[::3] = -1e-25
+    keep = torch.zeros(t.shape[dim], dtype=torch.bool)
+    keep[1::2] = True
+    shape = [1] * t.dim()
+    shape[dim] = -1
+    scale = torch.where(keep.view(shape).expand_as(t), torch.ones_like(t), scale.view_as(t))
+    return t * scale
+
+
+KINDS = [False, True, "tiny"]
+KIND_IDS = ["plain", "special", "tiny"]
+
+
 def _same(got, want):
     nan = torch.isnan(want)
     return torch.equal(torch.isnan(got), nan) and torch.equal(got.view(torch.int32)[~nan], want.view(torch.int32)[~nan])
 
 
-@pytest.mark.parametrize("special", [False, True], ids=["plain", "special"])
+@pytest.mark.parametrize("special", KINDS, ids=KIND_IDS)
 @pytest.mark.parametrize("shape", FWD, ids=[str(s) for s in FWD])
 def test_forward(shape, special):
     from repdl_amd import ops
@@ -52,7 +77,7 @@ def test_forward(shape, special):
     assert _same(got, oracle.conv2d(x, w, sH, sW, pH, pW, g))
 
 
-@pytest.mark.parametrize("special", [False, True], ids=["plain", "special"])
+@pytest.mark.parametrize("special", KINDS, ids=KIND_IDS)
 @pytest.mark.parametrize("shape", [s for s in FWD if s[-1] == 1], ids=[str(s) for s in FWD if s[-1] == 1])
 def test_grad_input(shape, special):
     from repdl_amd import ops
@@ -61,7 +86,10 @@ def test_grad_input(shape, special):
     OH, OW = (H + 2 * pH - KH) // sH + 1, (W + 2 * pW - KW) // sW + 1
     go = gen.normal_like(7, N, OC, OH, OW) * gen.relu_like(8, N, OC, OH, OW).sign()
     w = gen.normal_like(9, OC, IC, KH, KW)
-    if special:
+    if special == "tiny":
+        go, w = _tiny(go, 0), _tiny(w, 1)
+        go[:, 0] = 0.0
+    elif special:
         go.view(-1)[::101] = float("-inf")
         w.view(-1)[3::41] = -0.0
     got = ops.conv2d_grad_input((N, IC, H, W), w.cuda(), go.cuda(), (sH, sW), (pH, pW)).cpu()
@@ -72,12 +100,17 @@ WGRAD = [
     (3, 20, 18, 16, 40, 3, 3, 1, 1, 1, 1),   # OW = 16: one piece of 4 instructions
     (2, 8, 30, 28, 70, 3, 3, 1, 1, 1, 1),    # OW = 28: pieces of 7, OH = 30 -> chunks of several rows
     (2, 16, 16, 64, 16, 1, 1, 1, 1, 0, 0),   # OW = 64: pieces of 16, 1x1
-    (2, 6, 33, 65, 33, 3, 3, 2, 2, 1, 1),    # stride 2, OW = 33: v_fma_f32 kernel
+    (2, 6, 33, 65, 33, 3, 3, 2, 2, 1, 1),    # stride 2, OW = 33 and W = 65: both operands through padded copies
     (2, 5, 11, 12, 9, 2, 3, 1, 1, 0, 1),     # ragged
+    (4, 8, 14, 14, 16, 3, 3, 1, 1, 1, 1),    # OW = W = 14: rows rounded up to 16, pieces of 4
+    (2, 3, 9, 7, 5, 3, 3, 1, 1, 1, 1),       # OW = 7: pieces of 2
+    (2, 3, 5, 3, 4, 1, 1, 1, 1, 0, 0),       # OW = 3: pieces of 1
+    (2, 4, 12, 40, 6, 3, 5, 1, 3, 1, 2),     # stride 3 along the row
+    (1, 2, 8, 70, 3, 1, 3, 1, 17, 0, 1),     # stride 17: v_fma_f32 kernel
 ]
 
 
-@pytest.mark.parametrize("special", [False, True], ids=["plain", "special"])
+@pytest.mark.parametrize("special", KINDS, ids=KIND_IDS)
 @pytest.mark.parametrize("shape", WGRAD, ids=[str(s) for s in WGRAD])
 def test_grad_kernel(shape, special):
     from repdl_amd import ops
@@ -86,9 +119,12 @@ def test_grad_kernel(shape, special):
     OH, OW = (H + 2 * pH - KH) // sH + 1, (W + 2 * pW - KW) // sW + 1
     x = gen.relu_like(21, N, IC, H, W)
     go = gen.normal_like(22, N, OC, OH, OW)
-    if special:
+    if special == "tiny":
+        x, go = _tiny(x, 1), _tiny(go, 1)
+    elif special:
         x.view(-1)[::89] = float("inf")
         go.view(-1)[::61] = 0.0
+    if special or N > 2:
         go[:, 0] = 0.0  # a whole output channel of zero gradients: results are exact zeros
     got = ops.conv2d_grad_kernel(x.cuda(), (OC, IC, KH, KW), go.cuda(), (sH, sW), (pH, pW)).cpu()
     assert _same(got, oracle.conv2d_grad_kernel(go, x, KH, KW, sH, sW, pH, pW))
