@@ -21,10 +21,12 @@
 //      prefix at the chunk start; tuple (a0,a1,lo0,hi0,lo1,hi1) of the chunk under that
 //      hypothesis; tuples of groups of 8 chunks and of the block (64 chunks) wherever
 //      the hypotheses agree                                        (parallel, reads x again)
-//   4. one wave walks the blocks in order with the true state: a block whose hypothesis
-//      matches the state and whose tuple is valid for it is applied in O(1); otherwise
-//      its 8 groups are tried, then the 8 chunks of a failing group, and a chunk that
-//      fails is replayed with 64 real binary32 additions.
+//      (3b: tuples of super-blocks of 64 blocks, same rule)
+//   4. one wave walks the super-blocks in order with the true state: a node whose
+//      hypothesis matches the state and whose tuple is valid for it is applied in O(1);
+//      otherwise its children are tried -- the 64 blocks of a super-block, the 8 groups
+//      of a block, the 8 chunks of a group -- and a chunk that fails is replayed with 64
+//      real binary32 additions.
 // The hypotheses come from an approximation, but they only decide how much is replayed:
 // every applied map is checked against the true state, so the result is the sequential
 // sum bit for bit for every input (NaN, infinities, zeros and subnormal states simply
@@ -371,81 +373,161 @@ __device__ __forceinline__ bool lane_tup_apply(uint32_t &s, const LaneTup &l, in
     return ok;
 }
 
+// ---- step 3b: tuples of super-blocks (64 blocks) --------------------------------------------
+constexpr int SUP = 64; // blocks per super-block
+
+__global__ __launch_bounds__(256) void sum1d_super_kernel(const Tup *__restrict__ T2, Tup *__restrict__ T3, int64_t nblk,
+                                                          int64_t nsup)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t sb = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (sb >= nsup)
+        return;
+    const int64_t b = sb * SUP + lane;
+    Tup t = b < nblk ? T2[b] : tup_identity(HYP_ANY);
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1)
+        t = tup_join(t, tup_shfl_down(t, off)); // lane 0: the 64 blocks in order
+    if (lane == 0)
+        T3[sb] = t;
+}
+
+// What the walk needs of a block that does not apply as a whole: its data and its group and
+// chunk tuples, one slice per lane.
+struct BlockRegs
+{
+    float4 f[BLK / 256];
+    Tup tgr, tch;
+};
+
+__device__ __forceinline__ void load_block(BlockRegs &r, const float *__restrict__ x, int64_t n,
+                                           const Tup *__restrict__ T1, const Tup *__restrict__ TG, int64_t blk, int lane,
+                                           int vec)
+{
+    r.tgr = TG[blk * GROUPS + (lane & (GROUPS - 1))];
+    r.tch = T1[blk * (BLK / CH) + lane];
+    const int64_t e0 = blk * BLK;
+    if (vec && e0 + BLK <= n)
+    {
+#pragma unroll
+        for (int q = 0; q < BLK / 256; q++)
+            r.f[q] = reinterpret_cast<const float4 *>(x + e0)[q * 64 + lane];
+    }
+    else
+    {
+#pragma unroll
+        for (int q = 0; q < BLK / 256; q++)
+        {
+            const int64_t idx = e0 + (int64_t)(q * 64 + lane) * 4;
+            r.f[q].x = (idx + 0 < n) ? x[idx + 0] : 0.0f; // elements past n: s + 0 = s
+            r.f[q].y = (idx + 1 < n) ? x[idx + 1] : 0.0f;
+            r.f[q].z = (idx + 2 < n) ? x[idx + 2] : 0.0f;
+            r.f[q].w = (idx + 3 < n) ? x[idx + 3] : 0.0f;
+        }
+    }
+}
+
+typedef float f4v __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void read_chunk(const float *__restrict__ xd, int j, f4v (&v)[CH / 4])
+{
+    const f4v *p = reinterpret_cast<const f4v *>(xd + j * CH);
+#pragma unroll
+    for (int k = 0; k < CH / 4; k++)
+        v[k] = p[k];
+}
+
+// 64 real additions
+__device__ __forceinline__ uint32_t replay_chunk(uint32_t s, const f4v (&v)[CH / 4])
+{
+    float acc = __uint_as_float(s);
+#pragma unroll
+    for (int k = 0; k < CH / 4; k++)
+    {
+        acc = acc + v[k].x;
+        acc = acc + v[k].y;
+        acc = acc + v[k].z;
+        acc = acc + v[k].w;
+    }
+    return __builtin_amdgcn_readfirstlane(__float_as_uint(acc));
+}
+
+// One wave.  Super-blocks are tried first (far from binade boundaries a whole run of blocks
+// is one step), then the blocks of a failing super-block.  Failures cluster (they happen
+// where the sum moves along a binade boundary), so when a block fails the next block's data
+// and tuples are requested at once, and inside a failing group the LDS reads of a chunk are
+// issued one chunk ahead of the additions.
 __global__ __launch_bounds__(64) void sum1d_walk_kernel(const float *__restrict__ x, int64_t n,
                                                         const Tup *__restrict__ T1,
                                                         const Tup *__restrict__ TG,
-                                                        const Tup *__restrict__ T2, int64_t nblk, float factor,
-                                                        float *__restrict__ out, int vec)
+                                                        const Tup *__restrict__ T2,
+                                                        const Tup *__restrict__ T3, int64_t nblk, int64_t nsup,
+                                                        float factor, float *__restrict__ out, int vec)
 {
-    __shared__ __attribute__((aligned(16))) float xd[BLK];
+    __shared__ __attribute__((aligned(16))) float xd[BLK + 2 * CH]; // + what the read-ahead overshoots
     const int lane = threadIdx.x;
     uint32_t s = 0u; // +0.0f; wave-uniform throughout
-    Tup next = (lane < nblk) ? T2[lane] : tup_identity(HYP_ANY);
-    for (int64_t g0 = 0; g0 < nblk; g0 += 64)
+    BlockRegs pf;    // the block requested ahead
+    int64_t pf_blk = -1;
+    load_block(pf, x, n, T1, TG, 0, lane, vec); // (any valid block: the registers are then defined)
+    pf_blk = 0;
+    Tup nsup_t = (lane < nsup) ? T3[lane] : tup_identity(HYP_ANY);
+    // block tuples of the super-block being tried, and of the next one
+    Tup blk_next = (lane < nblk) ? T2[lane] : tup_identity(HYP_ANY);
+    for (int64_t g0 = 0; g0 < nsup; g0 += 64)
     {
-        const LaneTup lb = lane_tup(next);
-        if (g0 + 64 < nblk) // the next 64 block tuples, loaded while these are walked
-            next = (g0 + 64 + lane < nblk) ? T2[g0 + 64 + lane] : tup_identity(HYP_ANY);
-        const int cnt = (nblk - g0 < 64) ? (int)(nblk - g0) : 64;
+        const LaneTup ls = lane_tup(nsup_t);
+        if (g0 + 64 < nsup) // the next 64 super-block tuples, loaded while these are walked
+            nsup_t = (g0 + 64 + lane < nsup) ? T3[g0 + 64 + lane] : tup_identity(HYP_ANY);
+        const int cnt = (nsup - g0 < 64) ? (int)(nsup - g0) : 64;
         for (int i = 0; i < cnt; i++)
         {
-            if (lane_tup_apply(s, lb, i))
+            const int64_t sb = g0 + i;
+            const Tup blk_cur = blk_next;
+            {
+                const int64_t b = (sb + 1) * SUP + lane; // always requested: 32 bytes per block
+                blk_next = b < nblk ? T2[b] : tup_identity(HYP_ANY);
+            }
+            if (lane_tup_apply(s, ls, i))
                 continue;
-            // The block as a whole does not apply: bring in its group and chunk tuples and its
-            // data (all loads issued before any is waited for).
-            const int64_t blk = g0 + i;
-            const Tup tgr = TG[blk * GROUPS + (lane & (GROUPS - 1))];
-            const Tup tch = T1[blk * (BLK / CH) + lane];
-            const int64_t e0 = blk * BLK;
-            float4 f[BLK / 256];
-            if (vec && e0 + BLK <= n)
+            const LaneTup lb = lane_tup(blk_cur);
+            for (int bi = 0; bi < SUP; bi++)
             {
-#pragma unroll
-                for (int q = 0; q < BLK / 256; q++)
-                    f[q] = reinterpret_cast<const float4 *>(x + e0)[q * 64 + lane];
-            }
-            else
-            {
-#pragma unroll
-                for (int q = 0; q < BLK / 256; q++)
-                {
-                    const int64_t idx = e0 + (int64_t)(q * 64 + lane) * 4;
-                    f[q].x = (idx + 0 < n) ? x[idx + 0] : 0.0f;
-                    f[q].y = (idx + 1 < n) ? x[idx + 1] : 0.0f;
-                    f[q].z = (idx + 2 < n) ? x[idx + 2] : 0.0f;
-                    f[q].w = (idx + 3 < n) ? x[idx + 3] : 0.0f;
-                }
-            }
-            __syncthreads();
-#pragma unroll
-            for (int q = 0; q < BLK / 256; q++)
-                *reinterpret_cast<float4 *>(&xd[(q * 64 + lane) * 4]) = f[q];
-            __syncthreads();
-            const LaneTup lg = lane_tup(tgr), lc = lane_tup(tch);
-            for (int gr = 0; gr < GROUPS; gr++)
-            {
-                if (lane_tup_apply(s, lg, gr))
+                if (lane_tup_apply(s, lb, bi)) // blocks past the end are identities
                     continue;
-                for (int j = gr * (BLK / CH / GROUPS); j < (gr + 1) * (BLK / CH / GROUPS); j++)
+                // The block as a whole does not apply.
+                const int64_t blk = sb * SUP + bi;
+                if (pf_blk != blk)
+                    load_block(pf, x, n, T1, TG, blk, lane, vec);
+                __syncthreads();
+#pragma unroll
+                for (int q = 0; q < BLK / 256; q++)
+                    *reinterpret_cast<float4 *>(&xd[(q * 64 + lane) * 4]) = pf.f[q];
+                const LaneTup lg = lane_tup(pf.tgr), lc = lane_tup(pf.tch);
+                __syncthreads();
                 {
-                    if (lane_tup_apply(s, lc, j))
+                    const int64_t nb = blk + 1 < nblk ? blk + 1 : blk;
+                    load_block(pf, x, n, T1, TG, nb, lane, vec);
+                    pf_blk = nb;
+                }
+                for (int gr = 0; gr < GROUPS; gr++)
+                {
+                    if (lane_tup_apply(s, lg, gr))
                         continue;
-                    // replay: 64 real additions (elements past n were loaded as +0.0f: s + 0 = s)
-                    const float4 *p = reinterpret_cast<const float4 *>(&xd[j * CH]);
-                    float4 v[CH / 4];
+                    constexpr int CG = BLK / CH / GROUPS; // 8 chunks, reads one chunk ahead
+                    const int j0 = gr * CG;
+                    f4v va[CH / 4], vb[CH / 4];
+                    read_chunk(xd, j0, va);
 #pragma unroll
-                    for (int k = 0; k < CH / 4; k++)
-                        v[k] = p[k];
-                    float acc = __uint_as_float(s);
-#pragma unroll
-                    for (int k = 0; k < CH / 4; k++)
+                    for (int j = 0; j < CG; j += 2)
                     {
-                        acc = acc + v[k].x;
-                        acc = acc + v[k].y;
-                        acc = acc + v[k].z;
-                        acc = acc + v[k].w;
+                        read_chunk(xd, j0 + j + 1, vb);
+                        if (!lane_tup_apply(s, lc, j0 + j))
+                            s = replay_chunk(s, va);
+                        read_chunk(xd, j0 + j + 2, va);
+                        if (!lane_tup_apply(s, lc, j0 + j + 1))
+                            s = replay_chunk(s, vb);
                     }
-                    s = __builtin_amdgcn_readfirstlane(__float_as_uint(acc));
                 }
             }
         }
@@ -466,8 +548,9 @@ REPDL_API size_t repdl_hip_sum1d_workspace_bytes(int64_t n)
     if (n < REPDL_SUM1D_MIN_PARALLEL)
         return 0;
     const size_t nblk = (size_t)repdl_cdiv(n, BLK);
-    return round256(nblk * sizeof(double)) * 2 + round256(nblk * sizeof(Tup)) + round256(nblk * GROUPS * sizeof(Tup)) +
-           round256(nblk * (BLK / CH) * sizeof(Tup));
+    const size_t nsup = (nblk + SUP - 1) / SUP;
+    return round256(nblk * sizeof(double)) * 2 + round256(nsup * sizeof(Tup)) + round256(nblk * sizeof(Tup)) +
+           round256(nblk * GROUPS * sizeof(Tup)) + round256(nblk * (BLK / CH) * sizeof(Tup));
 }
 
 REPDL_API int repdl_hip_sum1d_ws(const float *in, float *out, int64_t n, int average, void *workspace,
@@ -486,6 +569,9 @@ REPDL_API int repdl_hip_sum1d_ws(const float *in, float *out, int64_t n, int ave
     w += round256(nblk * sizeof(double));
     double *prefix = reinterpret_cast<double *>(w);
     w += round256(nblk * sizeof(double));
+    const int64_t nsup = repdl_cdiv(nblk, SUP);
+    Tup *T3 = reinterpret_cast<Tup *>(w);
+    w += round256(nsup * sizeof(Tup));
     Tup *T2 = reinterpret_cast<Tup *>(w);
     w += round256(nblk * sizeof(Tup));
     Tup *TG = reinterpret_cast<Tup *>(w);
@@ -496,7 +582,8 @@ REPDL_API int repdl_hip_sum1d_ws(const float *in, float *out, int64_t n, int ave
     hipLaunchKernelGGL(sum1d_blocksum_kernel, dim3((unsigned)nblk), dim3(256), 0, s, in, n, bsum, vec);
     hipLaunchKernelGGL(sum1d_prefix_kernel, dim3(1), dim3(256), 0, s, bsum, prefix, nblk);
     hipLaunchKernelGGL(sum1d_tuple_kernel, dim3((unsigned)nblk), dim3(256), 0, s, in, n, prefix, T1, TG, T2, vec);
-    hipLaunchKernelGGL(sum1d_walk_kernel, dim3(1), dim3(64), 0, s, in, n, T1, TG, T2, nblk,
+    hipLaunchKernelGGL(sum1d_super_kernel, dim3((unsigned)repdl_cdiv(nsup, 4)), dim3(256), 0, s, T2, T3, nblk, nsup);
+    hipLaunchKernelGGL(sum1d_walk_kernel, dim3(1), dim3(64), 0, s, in, n, T1, TG, T2, T3, nblk, nsup,
                        repdl_sum_factor(average, n), out, vec);
     return repdl_launch_status();
 }
