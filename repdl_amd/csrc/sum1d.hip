@@ -17,6 +17,8 @@
 // Pipeline (n >= SUM1D_MIN_PARALLEL; shorter inputs take the serial kernel of sum.hip):
 //   1. block sums in binary64 over blocks of 4096 elements        (parallel, reads x once)
 //   2. exclusive prefix of the block sums                          (one workgroup)
+//      (1 and 2 run twice: the second time each element counts for what it is worth on
+//      the grid of the state predicted the first time, see quantum_of)
 //   3. per chunk of 64 elements: the binade/sign HYPOTHESIS is read off the binary64
 //      prefix at the chunk start; tuple (a0,a1,lo0,hi0,lo1,hi1) of the chunk under that
 //      hypothesis; tuples of groups of 8 chunks and of the block (64 chunks) wherever
@@ -190,17 +192,57 @@ __device__ __forceinline__ double wave_sum(double v)
     return v;
 }
 
+// The running sum moves by what an element is worth ON THE GRID of the binade the sum is in:
+// S + x rounds to a multiple of the quantum q of S, so the step is x rounded to a multiple of
+// q (ties aside).  Summing the elements exactly instead predicts the wrong state wherever
+// that differs systematically -- a sum of 2^28 values from [0, 1) stops growing at 2^24, where
+// every element is below q/2, while the exact sum goes on to 2^27 and every hypothesis after
+// that point is wrong.  So the prediction is refined: a second pass rounds each element to
+// the grid of the state the first pass predicted for its block, which models exactly that.
+struct Quantum
+{
+    double q, inv_q; // q == 0: leave the element as it is
+};
+
+__device__ __forceinline__ Quantum quantum_of(double state)
+{
+    const uint32_t u = __float_as_uint((float)state);
+    int e = (int)((u >> 23) & 0xFFu);
+    Quantum r;
+    if (e == 255 || state != state)
+    {
+        r.q = r.inv_q = 0.0;
+        return r;
+    }
+    e = e < 1 ? 1 : e; // subnormal states share the smallest normal binade's grid, 2^-149
+    r.q = __longlong_as_double((long long)(e - 150 + 1023) << 52);
+    r.inv_q = __longlong_as_double((long long)(150 - e + 1023) << 52);
+    return r;
+}
+
+__device__ __forceinline__ double quantise(float x, const Quantum &g)
+{
+    return g.q == 0.0 ? (double)x : rint((double)x * g.inv_q) * g.q;
+}
+
+// prev == nullptr: exact sums; else: sums of the elements rounded to the grid of the state
+// prev[block] predicted by the previous pass.
 __global__ __launch_bounds__(256) void sum1d_blocksum_kernel(const float *__restrict__ x, int64_t n,
+                                                             const double *__restrict__ prev,
                                                              double *__restrict__ bsum, int vec)
 {
     __shared__ double part[4];
     const int tid = threadIdx.x;
     float v[16];
     load16(x, n, (int64_t)blockIdx.x * BLK + tid * 16, vec, v);
+    Quantum g;
+    g.q = g.inv_q = 0.0;
+    if (prev != nullptr)
+        g = quantum_of(prev[blockIdx.x]);
     double d = 0.0;
 #pragma unroll
     for (int q = 0; q < 16; q++)
-        d += (double)v[q];
+        d += quantise(v[q], g);
     d = wave_sum(d);
     if ((tid & 63) == 0)
         part[tid >> 6] = d;
@@ -254,13 +296,15 @@ __global__ __launch_bounds__(256) void sum1d_tuple_kernel(const float *__restric
     float v[16];
     load16(x, n, blk * BLK + tid * 16, vec, v);
 
-    // binary64 exclusive prefix over the threads of the block
+    // binary64 exclusive prefix over the threads of the block (elements on the grid of the
+    // state predicted for the block start, as in the refined block sums)
+    const Quantum g = quantum_of(prefix[blk]);
     double d = 0.0;
     bool finite = true, allzero = true;
 #pragma unroll
     for (int q = 0; q < 16; q++)
     {
-        d += (double)v[q];
+        d += quantise(v[q], g);
         const uint32_t a = __float_as_uint(v[q]) & 0x7FFFFFFFu;
         finite = finite && a < 0x7F800000u;
         allzero = allzero && a == 0u;
@@ -579,7 +623,12 @@ REPDL_API int repdl_hip_sum1d_ws(const float *in, float *out, int64_t n, int ave
     Tup *T1 = reinterpret_cast<Tup *>(w);
     hipStream_t s = repdl_stream(stream);
     const int vec = aligned16(in);
-    hipLaunchKernelGGL(sum1d_blocksum_kernel, dim3((unsigned)nblk), dim3(256), 0, s, in, n, bsum, vec);
+    hipLaunchKernelGGL(sum1d_blocksum_kernel, dim3((unsigned)nblk), dim3(256), 0, s, in, n,
+                       static_cast<const double *>(nullptr), bsum, vec);
+    hipLaunchKernelGGL(sum1d_prefix_kernel, dim3(1), dim3(256), 0, s, bsum, prefix, nblk);
+    // one refinement of the prediction (see quantum_of)
+    hipLaunchKernelGGL(sum1d_blocksum_kernel, dim3((unsigned)nblk), dim3(256), 0, s, in, n,
+                       static_cast<const double *>(prefix), bsum, vec);
     hipLaunchKernelGGL(sum1d_prefix_kernel, dim3(1), dim3(256), 0, s, bsum, prefix, nblk);
     hipLaunchKernelGGL(sum1d_tuple_kernel, dim3((unsigned)nblk), dim3(256), 0, s, in, n, prefix, T1, TG, T2, vec);
     hipLaunchKernelGGL(sum1d_super_kernel, dim3((unsigned)repdl_cdiv(nsup, 4)), dim3(256), 0, s, T2, T3, nblk, nsup);

@@ -31,6 +31,10 @@ def _cases():
     yield "inf_nan", np.concatenate([r.standard_normal(90_000), [np.inf], r.standard_normal(50_000), [-np.inf], r.standard_normal(50_000)]).astype(np.float32)
     yield "subnormal_state", (r.integers(-2**20, 2**20, n).astype(np.float64) * 2.0**-149).astype(np.float32)
     yield "cancel_to_zero", np.tile(np.array([3.25, -3.25, 1e-3, -1e-3], dtype=np.float32), 60_000)
+    # the running sum stops growing at 2^24 (every element below half a quantum) two thirds
+    # of the way through, and at 2^22 for the smaller elements that follow a large start
+    yield "stagnation", (0.25 + 0.75 * r.random(1 << 25)).astype(np.float32)
+    yield "stagnation_small", np.concatenate([[2.0**22], r.random(2_000_000) * 0.25, -r.random(500_000) * 0.3]).astype(np.float32)
     yield "just_long_enough", gen.uniform_pm1(3, 32768).numpy()
     yield "just_too_short", gen.uniform_pm1(4, 32767).numpy()
 
