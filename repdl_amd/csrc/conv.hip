@@ -780,7 +780,9 @@ __global__ __launch_bounds__(256) void conv_ktab_kernel(int *__restrict__ tabB, 
     }
 }
 
-template <int BM, int MODE>
+// PB: 32-pixel blocks per wave (2: tiles of 128 pixels; 1, only with BM = 64: tiles of 64 pixels,
+// twice the workgroups at half the duration, for layers whose 128-pixel tiles fill the chip unevenly)
+template <int BM, int MODE, int PB>
 __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__restrict__ Gp,   // padded gathered operand
                                                                 const float *__restrict__ Xg,   // the original one (epilogue)
                                                                 const float *__restrict__ Wt, float *__restrict__ Out,
@@ -790,11 +792,13 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
 {
     constexpr int NT = 2 * BM;
     constexpr int LDA = BM + 4;
-    constexpr int NKR = BM == 64 ? 16 : 8; // k-rows of the gathered tile per wave
+    static_assert(PB == 2 || (PB == 1 && BM == 64), "tiles of 64 pixels only with two waves");
+    constexpr int TBN = PB == 2 ? BN : BN / 2;          // pixels per tile
+    constexpr int NKR = BM == 64 && PB == 2 ? 16 : 8;   // k-rows of the gathered tile per wave
     typedef float v4f __attribute__((ext_vector_type(4)));
     // One buffer for the kernel tile, two for the gathered tile, no row pad on the latter (its
     // rows are written and read by consecutive lanes): 20.3 KiB at BM = 64, seven workgroups per CU.
-    constexpr int LDBF = BN;
+    constexpr int LDBF = TBN;
     __shared__ __attribute__((aligned(16))) float As[BK * LDA];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDBF];
 
@@ -808,11 +812,11 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
     const int PW = MODE == MODE_FWD ? d.OW : d.W;
     const int n = MODE == MODE_FWD ? blockIdx.z / d.groups : blockIdx.z;
     const int g = MODE == MODE_FWD ? blockIdx.z % d.groups : 0;
-    const int m0 = blockIdx.y * BM, p0 = blockIdx.x * BN;
+    const int m0 = blockIdx.y * BM, p0 = blockIdx.x * TBN;
 
     // gathered operand: this lane's pixel, this wave's k-rows
-    const int b_half = BM == 64 ? wave : (wave & 1);
-    const int b_kr0 = BM == 64 ? 0 : 8 * (wave >> 1);
+    const int b_half = PB == 1 ? 0 : (BM == 64 ? wave : (wave & 1));
+    const int b_kr0 = PB == 1 ? 8 * wave : (BM == 64 ? 0 : 8 * (wave >> 1));
     const int pix_local = 64 * b_half + lane;
     const int pixc = p0 + pix_local < P ? p0 + pix_local : P - 1;
     const int pph = pixc / PW, ppw = pixc - pph * PW;
@@ -892,15 +896,15 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
 
     const int l32 = lane & 31, half = lane >> 5;
     const int wm = BM == 64 ? 0 : (wave & 1), wn = BM == 64 ? wave : (wave >> 1);
-    f16v acc[2][2];
+    f16v acc[2][PB];
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < PB; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++)
                 acc[i][j][r] = 0.0f;
-    const int a_off = half * LDA + wm * 64 + l32, b_off = half * LDBF + wn * 64 + l32;
+    const int a_off = half * LDA + wm * 64 + l32, b_off = half * LDBF + wn * (32 * PB) + l32;
 
     const int nkt = K / BK;
     if (nkt > 0)
@@ -916,21 +920,22 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
         if (more)
             load_tiles(kt + 1);
         const float *as = As + a_off, *bs = Bs[cur] + b_off;
-        float a[BK / 2][2], b[BK / 2][2];
+        float a[BK / 2][2], b[BK / 2][PB];
 #pragma unroll
         for (int kp = 0; kp < BK / 2; kp++)
         {
             a[kp][0] = as[2 * kp * LDA];
             a[kp][1] = as[2 * kp * LDA + 32];
-            b[kp][0] = bs[2 * kp * LDBF];
-            b[kp][1] = bs[2 * kp * LDBF + 32];
+#pragma unroll
+            for (int j = 0; j < PB; j++)
+                b[kp][j] = bs[2 * kp * LDBF + 32 * j];
         }
 #pragma unroll
         for (int kp = 0; kp < BK / 2; kp++)
 #pragma unroll
             for (int i = 0; i < 2; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++)
+                for (int j = 0; j < PB; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kp][i], b[kp][j], acc[i][j], 0, 0, 0);
         __syncthreads(); // every wave has read the kernel tile
         if (more)
@@ -948,9 +953,9 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
             const int m = m0 + wm * 64 + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3);
             const int ch = MODE == MODE_FWD ? g * OCg + m : m;
 #pragma unroll
-            for (int j = 0; j < 2; j++)
+            for (int j = 0; j < PB; j++)
             {
-                const int pix = p0 + wn * 64 + 32 * j + l32;
+                const int pix = p0 + wn * (32 * PB) + 32 * j + l32;
                 if (pix >= P)
                     continue;
                 float v = acc[i][j][r];
@@ -1561,6 +1566,19 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
 inline bool fits_i32(int64_t v) { return v >= 0 && v <= REPDL_I32_MAX; }
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// Which pixel-tile width for the two-wave kernel?  Tiles of 128 pixels keep the matrix pipes
+// busier (73 against 71 TFLOP/s on launches of 6000 workgroups), but with 152 registers per
+// lane only 1536 of their workgroups are resident at a time, and a launch of one or two rounds
+// leaves much of the chip idle at its end.  Tiles of 64 pixels make twice the workgroups of
+// half the duration, 2560 resident.  Measured (batch 64, 64 -> 64 channels, 3x3): 28x28
+// 0.122 -> 0.087 ms, 56x56 0.246 -> 0.229, 80x80 0.437 -> 0.422, 112x112 0.807 -> 0.825;
+// grad-input, whose kernel tile is a strided gather, gains only on the small launches
+// (28x28 0.127 -> 0.090, 56x56 0.248 -> 0.257).
+inline bool conv_small_tiles(int mode, int64_t workgroups128)
+{
+    return workgroups128 < (mode == MODE_FWD ? 4096 : 1024);
+}
+
 template <int MODE>
 int launch_conv_gemm(const float *gathered, const float *kernel, float *out, const ConvDims &d, void *stream)
 {
@@ -1623,12 +1641,17 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
             if (skips)
                 launch_guard_final(guard, ca, cb, s);
             const float *src = pad ? Gp : gathered;
-            dim3 grid((unsigned)gx, (unsigned)(M / bm), (unsigned)gz);
-            if (bm == 64)
-                hipLaunchKernelGGL((conv_gemm_fast_kernel<64, MODE>), grid, dim3(128), 0, s, src, gathered, kernel, out, d, tabB,
-                                   tabA, (int)plane, (int)Wp, img, guard);
+            // Tiles of 64 pixels when that fills the chip more evenly (see conv_small_tiles).
+            const bool small_tiles = bm == 64 && conv_small_tiles(MODE, gx * (M / bm) * gz);
+            dim3 grid((unsigned)(small_tiles ? repdl_cdiv(P, BN / 2) : gx), (unsigned)(M / bm), (unsigned)gz);
+            if (bm == 64 && small_tiles)
+                hipLaunchKernelGGL((conv_gemm_fast_kernel<64, MODE, 1>), grid, dim3(128), 0, s, src, gathered, kernel, out, d,
+                                   tabB, tabA, (int)plane, (int)Wp, img, guard);
+            else if (bm == 64)
+                hipLaunchKernelGGL((conv_gemm_fast_kernel<64, MODE, 2>), grid, dim3(128), 0, s, src, gathered, kernel, out, d,
+                                   tabB, tabA, (int)plane, (int)Wp, img, guard);
             else
-                hipLaunchKernelGGL((conv_gemm_fast_kernel<128, MODE>), grid, dim3(256), 0, s, src, gathered, kernel, out, d,
+                hipLaunchKernelGGL((conv_gemm_fast_kernel<128, MODE, 2>), grid, dim3(256), 0, s, src, gathered, kernel, out, d,
                                    tabB, tabA, (int)plane, (int)Wp, img, guard);
             const int rc = repdl_launch_status();
             e = hipFreeAsync(ws, s);
