@@ -796,10 +796,13 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
     constexpr int TBN = PB == 2 ? BN : BN / 2;          // pixels per tile
     constexpr int NKR = BM == 64 && PB == 2 ? 16 : 8;   // k-rows of the gathered tile per wave
     typedef float v4f __attribute__((ext_vector_type(4)));
-    // One buffer for the kernel tile, two for the gathered tile, no row pad on the latter (its
-    // rows are written and read by consecutive lanes): 20.3 KiB at BM = 64, seven workgroups per CU.
+    // Two buffers for the gathered tile, no row pad (its rows are written and read by
+    // consecutive lanes).  The kernel tile has two buffers with 128-pixel tiles (one barrier
+    // per k-tile: 112x112 forward 0.807 -> 0.780 ms) and one with 64-pixel tiles, where the
+    // LDS it saves is a tenth workgroup per CU and worth more than the barrier.
     constexpr int LDBF = TBN;
-    __shared__ __attribute__((aligned(16))) float As[BK * LDA];
+    constexpr int NA = PB == 2 ? 2 : 1;
+    __shared__ __attribute__((aligned(16))) float As[NA][BK * LDA];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDBF];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -871,7 +874,7 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
         }
     };
     auto store_tiles = [&](int buf) {
-        float *as = As, *bs = Bs[buf];
+        float *as = As[NA == 2 ? buf : 0], *bs = Bs[buf];
 #pragma unroll
         for (int j = 0; j < NKR; j++)
             bs[(b_kr0 + j) * LDBF + pix_local] = fb[j];
@@ -919,7 +922,7 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
         const bool more = kt + 1 < nkt;
         if (more)
             load_tiles(kt + 1);
-        const float *as = As + a_off, *bs = Bs[cur] + b_off;
+        const float *as = As[NA == 2 ? cur : 0] + a_off, *bs = Bs[cur] + b_off;
         float a[BK / 2][2], b[BK / 2][PB];
 #pragma unroll
         for (int kp = 0; kp < BK / 2; kp++)
@@ -937,9 +940,10 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
 #pragma unroll
                 for (int j = 0; j < PB; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kp][i], b[kp][j], acc[i][j], 0, 0, 0);
-        __syncthreads(); // every wave has read the kernel tile
+        if (NA == 1)
+            __syncthreads(); // every wave has read the kernel tile
         if (more)
-            store_tiles(cur ^ 1);
+            store_tiles(cur ^ 1); // (NA == 2: last read before the barrier that ended the previous k-tile)
         __syncthreads();
     }
 
