@@ -726,9 +726,10 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_kernel(const float *__restri
 // per-thread constant).  A load is then: scalar base, constant vector offset.
 //   forward     tab[k] = c*Hp*Wp + kh*Wp + kw,                  pix_off = oh*sH*Wp + ow*sW
 //   grad-input  tab[k] = oc*Hp*Wp + (pH+PT-kh)*Wp + (pW+PL-kw), pix_off = h*Wp + w      (stride 1)
-// The kernel operand of grad-input is a strided gather too: W[(oc*IC + ic)*KHW + kh*KW + kw]
-// = tabA[k] + ic*KHW.  Lanes map to pixels (or input channels), k-rows to instructions,
-// so every table entry is wave-uniform.  Requires K % 16 == 0 and M % BM == 0; pixels
+// The kernel operand is read as [M][K] panels with k contiguous: the kernel itself for forward,
+// for grad-input a copy WT[ic][(oc, kh, kw)] that conv_ktab_kernel writes next to the table.
+// Lanes map to pixels, k-rows to instructions, so every table entry is wave-uniform.
+// Requires K % 16 == 0 and M % BM == 0; pixels
 // past the end of the image repeat the last pixel and are not stored.  The padded
 // zeros play the role of the skipped taps exactly as in conv_gemm_kernel, with the same
 // epilogue.
@@ -761,23 +762,31 @@ inline unsigned pad_blocks(int64_t total)
     return (unsigned)(b < 1 ? 1 : (b > GUARD_PARTS ? GUARD_PARTS : b)); // 2048 x 256 threads fill the chip
 }
 
-__global__ __launch_bounds__(256) void conv_ktab_kernel(int *__restrict__ tabB, int *__restrict__ tabA, int K, int KH,
-                                                        int KW, int plane, int Wp, int mode, int IC, int baseH,
-                                                        int baseW)
+// Blocks [0, ceil(K / 256)) write the table; for grad-input the blocks after them write the
+// kernel operand as the [IC][K] panel the matrix kernel reads, WT[ic][k] = W[oc][ic][kh][kw]
+// for k = (oc, kh, kw).
+__global__ __launch_bounds__(256) void conv_ktab_kernel(int *__restrict__ tabB, int K, int KH, int KW, int plane, int Wp,
+                                                        int mode, int IC, int baseH, int baseW,
+                                                        const float *__restrict__ W, float *__restrict__ WT)
 {
+    const int KHW = KH * KW;
+    const int tab_blocks = (K + 255) / 256;
+    if ((int)blockIdx.x >= tab_blocks)
+    {
+        const int64_t idx = (int64_t)(blockIdx.x - tab_blocks) * 256 + threadIdx.x; // = ic * K + k
+        if (idx >= (int64_t)IC * K)
+            return;
+        const int ic = (int)(idx / K), k = (int)(idx - (int64_t)ic * K);
+        const int oc = k / KHW, rem = k - oc * KHW;
+        WT[idx] = W[((int64_t)oc * IC + ic) * KHW + rem];
+        return;
+    }
     const int k = blockIdx.x * 256 + threadIdx.x;
     if (k >= K)
         return;
-    const int KHW = KH * KW;
     const int c = k / KHW, rem = k - c * KHW;
     const int kh = rem / KW, kw = rem - kh * KW;
-    if (mode == MODE_FWD)
-        tabB[k] = c * plane + kh * Wp + kw;
-    else
-    {
-        tabB[k] = c * plane + (baseH - kh) * Wp + (baseW - kw);
-        tabA[k] = c * IC * KHW + kh * KW + kw;
-    }
+    tabB[k] = mode == MODE_FWD ? c * plane + kh * Wp + kw : c * plane + (baseH - kh) * Wp + (baseW - kw);
 }
 
 // PB: 32-pixel blocks per wave (2: tiles of 128 pixels; 1, only with BM = 64: tiles of 64 pixels,
@@ -785,9 +794,10 @@ __global__ __launch_bounds__(256) void conv_ktab_kernel(int *__restrict__ tabB, 
 template <int BM, int MODE, int PB>
 __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__restrict__ Gp,   // padded gathered operand
                                                                 const float *__restrict__ Xg,   // the original one (epilogue)
-                                                                const float *__restrict__ Wt, float *__restrict__ Out,
-                                                                ConvDims d, const int *__restrict__ tabB,
-                                                                const int *__restrict__ tabA, int plane, int Wp,
+                                                                const float *__restrict__ Wt,   // the kernel (epilogue)
+                                                                const float *__restrict__ Wa,   // kernel operand as [M][K] panels
+                                                                float *__restrict__ Out, ConvDims d,
+                                                                const int *__restrict__ tabB, int plane, int Wp,
                                                                 int64_t img_stride, const unsigned *__restrict__ guard)
 {
     constexpr int NT = 2 * BM;
@@ -826,27 +836,20 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
     const int pix_off = MODE == MODE_FWD ? pph * d.sH * Wp + ppw * d.sW : pph * Wp + ppw;
     const float *Gimg = Gp + (int64_t)n * img_stride + (MODE == MODE_FWD ? (int64_t)g * ICg * plane : 0);
     // kernel operand
-    const float *Wg = MODE == MODE_FWD ? Wt + (int64_t)g * OCg * K : Wt;
-    uint32_t a_voff[2]; // FWD: byte offsets of this thread's two float4 slots in the [BM][K] panel
+    const float *Wg = MODE == MODE_FWD ? Wa + (int64_t)g * OCg * K : Wa;
+    uint32_t a_voff[2]; // byte offsets of this thread's two float4 slots in the [BM][K] panel
     int a_st[2];
-    const int a_half = BM == 64 ? 0 : (wave & 1); // DGRAD: this lane's input channel, this wave's 8 k-rows
-    const int a_kr0 = BM == 64 ? 8 * wave : 8 * (wave >> 1);
-    const int a_m = 64 * a_half + lane;
-    if (MODE == MODE_FWD)
-    {
 #pragma unroll
-        for (int i = 0; i < 2; i++)
-        {
-            const int idx = tid + NT * i;
-            const int r = idx >> 2, k4 = (idx & 3) << 2;
-            a_voff[i] = (uint32_t)(r * K + k4) * 4u;
-            a_st[i] = k4 * LDA + r;
-        }
+    for (int i = 0; i < 2; i++)
+    {
+        const int idx = tid + NT * i;
+        const int r = idx >> 2, k4 = (idx & 3) << 2;
+        a_voff[i] = (uint32_t)(r * K + k4) * 4u;
+        a_st[i] = k4 * LDA + r;
     }
-    const int a_ch_off = (m0 + a_m) * KHW; // DGRAD
 
     v4f fa4[2];
-    float fa1[8], fb[NKR];
+    float fb[NKR];
     auto load_tiles = [&](int kt) {
         const int *tb = tabB + kt * BK + b_kr0;
 #pragma unroll
@@ -855,45 +858,23 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
             const float *rowp = Gimg + tb[j];
             fb[j] = rowp[pix_off];
         }
-        if (MODE == MODE_FWD)
-        {
-            const char *ab = reinterpret_cast<const char *>(Wg + (int64_t)m0 * K + kt * BK);
+        const char *ab = reinterpret_cast<const char *>(Wg + (int64_t)m0 * K + kt * BK);
 #pragma unroll
-            for (int i = 0; i < 2; i++)
-                fa4[i] = *reinterpret_cast<const v4f *>(ab + a_voff[i]);
-        }
-        else
-        {
-            const int *ta = tabA + kt * BK + a_kr0;
-#pragma unroll
-            for (int j = 0; j < 8; j++)
-            {
-                const float *wp = Wg + ta[j];
-                fa1[j] = wp[a_ch_off];
-            }
-        }
+        for (int i = 0; i < 2; i++)
+            fa4[i] = *reinterpret_cast<const v4f *>(ab + a_voff[i]);
     };
     auto store_tiles = [&](int buf) {
         float *as = As[NA == 2 ? buf : 0], *bs = Bs[buf];
 #pragma unroll
         for (int j = 0; j < NKR; j++)
             bs[(b_kr0 + j) * LDBF + pix_local] = fb[j];
-        if (MODE == MODE_FWD)
-        {
 #pragma unroll
-            for (int i = 0; i < 2; i++)
-            {
-                as[a_st[i] + 0 * LDA] = fa4[i][0];
-                as[a_st[i] + 1 * LDA] = fa4[i][1];
-                as[a_st[i] + 2 * LDA] = fa4[i][2];
-                as[a_st[i] + 3 * LDA] = fa4[i][3];
-            }
-        }
-        else
+        for (int i = 0; i < 2; i++)
         {
-#pragma unroll
-            for (int j = 0; j < 8; j++)
-                as[(a_kr0 + j) * LDA + a_m] = fa1[j];
+            as[a_st[i] + 0 * LDA] = fa4[i][0];
+            as[a_st[i] + 1 * LDA] = fa4[i][1];
+            as[a_st[i] + 2 * LDA] = fa4[i][2];
+            as[a_st[i] + 3 * LDA] = fa4[i][3];
         }
     };
 
@@ -1574,14 +1555,10 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 // busier (73 against 71 TFLOP/s on launches of 6000 workgroups), but with 152 registers per
 // lane only 1536 of their workgroups are resident at a time, and a launch of one or two rounds
 // leaves much of the chip idle at its end.  Tiles of 64 pixels make twice the workgroups of
-// half the duration, 2560 resident.  Measured (batch 64, 64 -> 64 channels, 3x3): 28x28
-// 0.122 -> 0.087 ms, 56x56 0.246 -> 0.229, 80x80 0.437 -> 0.422, 112x112 0.807 -> 0.825;
-// grad-input, whose kernel tile is a strided gather, gains only on the small launches
-// (28x28 0.127 -> 0.090, 56x56 0.248 -> 0.257).
-inline bool conv_small_tiles(int mode, int64_t workgroups128)
-{
-    return workgroups128 < (mode == MODE_FWD ? 4096 : 1024);
-}
+// half the duration, 2560 resident.  Measured (batch 64, 64 -> 64 channels, 3x3, forward /
+// grad-input): 28x28 0.127 / 0.121 -> 0.087 / 0.087 ms, 56x56 0.247 / 0.241 -> 0.226 / 0.224,
+// 80x80 0.431 / 0.414 -> 0.423 / 0.412, 112x112 0.818 / 0.751 -> 0.818 / 0.773.
+inline bool conv_small_tiles(int64_t workgroups128) { return workgroups128 < 4096; }
 
 template <int MODE>
 int launch_conv_gemm(const float *gathered, const float *kernel, float *out, const ConvDims &d, void *stream)
@@ -1617,24 +1594,28 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
         if (img * 4 < (1LL << 31) && (int64_t)M * K * 4 < (1LL << 31) && (int64_t)d.N * img / 256 < REPDL_I32_MAX)
         {
             const bool pad = PT > 0 || PL > 0;
-            // workspace: the guard words, the two tables, the padded copy
-            const size_t tab_bytes = ((size_t)2 * K * sizeof(int) + 255) / 256 * 256;
-            const size_t ws_bytes = GUARD_BYTES + tab_bytes + (pad ? (size_t)d.N * img * sizeof(float) : 0);
+            // workspace: the guard words, the table, the kernel as [IC][K] panels (grad-input), the padded copy
+            const size_t tab_bytes = ((size_t)K * sizeof(int) + 255) / 256 * 256;
+            const size_t wt_bytes = MODE == MODE_FWD ? 0 : ((size_t)M * K * sizeof(float) + 255) / 256 * 256;
+            const size_t ws_bytes = GUARD_BYTES + tab_bytes + wt_bytes + (pad ? (size_t)d.N * img * sizeof(float) : 0);
             char *ws = nullptr;
             hipError_t e = hipMallocAsync(reinterpret_cast<void **>(&ws), ws_bytes, s);
             if (e != hipSuccess)
                 return (int)e;
             unsigned *guard = reinterpret_cast<unsigned *>(ws);
-            int *tabB = reinterpret_cast<int *>(ws + GUARD_BYTES), *tabA = tabB + K;
-            float *Gp = reinterpret_cast<float *>(ws + GUARD_BYTES + tab_bytes);
+            int *tabB = reinterpret_cast<int *>(ws + GUARD_BYTES);
+            float *WT = reinterpret_cast<float *>(ws + GUARD_BYTES + tab_bytes);
+            float *Gp = reinterpret_cast<float *>(ws + GUARD_BYTES + tab_bytes + wt_bytes);
+            const float *Wa = MODE == MODE_FWD ? kernel : WT;
             // guard[0]: the gathered operand (in the padding pass when there is one), guard[1]: the kernel
             int ca = 0, cb = 0;
             if (skips)
                 launch_guard_scan(pad ? nullptr : gathered, gathered_count, kernel, kernel_count, guard, s, ca, cb);
             else
                 guard = nullptr;
-            hipLaunchKernelGGL(conv_ktab_kernel, dim3((unsigned)repdl_cdiv(K, 256)), dim3(256), 0, s, tabB, tabA, (int)K,
-                               d.KH, d.KW, (int)plane, (int)Wp, MODE, d.IC, d.pH + PT, d.pW + PL);
+            const int64_t ktab_blocks = repdl_cdiv(K, 256) + (MODE == MODE_FWD ? 0 : repdl_cdiv((int64_t)M * K, 256));
+            hipLaunchKernelGGL(conv_ktab_kernel, dim3((unsigned)ktab_blocks), dim3(256), 0, s, tabB, (int)K, d.KH, d.KW,
+                               (int)plane, (int)Wp, MODE, d.IC, d.pH + PT, d.pW + PL, kernel, WT);
             if (pad)
             {
                 const int64_t total = (int64_t)d.N * img;
@@ -1646,17 +1627,17 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
                 launch_guard_final(guard, ca, cb, s);
             const float *src = pad ? Gp : gathered;
             // Tiles of 64 pixels when that fills the chip more evenly (see conv_small_tiles).
-            const bool small_tiles = bm == 64 && conv_small_tiles(MODE, gx * (M / bm) * gz);
+            const bool small_tiles = bm == 64 && conv_small_tiles(gx * (M / bm) * gz);
             dim3 grid((unsigned)(small_tiles ? repdl_cdiv(P, BN / 2) : gx), (unsigned)(M / bm), (unsigned)gz);
             if (bm == 64 && small_tiles)
-                hipLaunchKernelGGL((conv_gemm_fast_kernel<64, MODE, 1>), grid, dim3(128), 0, s, src, gathered, kernel, out, d,
-                                   tabB, tabA, (int)plane, (int)Wp, img, guard);
+                hipLaunchKernelGGL((conv_gemm_fast_kernel<64, MODE, 1>), grid, dim3(128), 0, s, src, gathered, kernel, Wa, out,
+                                   d, tabB, (int)plane, (int)Wp, img, guard);
             else if (bm == 64)
-                hipLaunchKernelGGL((conv_gemm_fast_kernel<64, MODE, 2>), grid, dim3(128), 0, s, src, gathered, kernel, out, d,
-                                   tabB, tabA, (int)plane, (int)Wp, img, guard);
+                hipLaunchKernelGGL((conv_gemm_fast_kernel<64, MODE, 2>), grid, dim3(128), 0, s, src, gathered, kernel, Wa, out,
+                                   d, tabB, (int)plane, (int)Wp, img, guard);
             else
-                hipLaunchKernelGGL((conv_gemm_fast_kernel<128, MODE, 2>), grid, dim3(256), 0, s, src, gathered, kernel, out, d,
-                                   tabB, tabA, (int)plane, (int)Wp, img, guard);
+                hipLaunchKernelGGL((conv_gemm_fast_kernel<128, MODE, 2>), grid, dim3(256), 0, s, src, gathered, kernel, Wa, out,
+                                   d, tabB, (int)plane, (int)Wp, img, guard);
             const int rc = repdl_launch_status();
             e = hipFreeAsync(ws, s);
             return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);

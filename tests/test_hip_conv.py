@@ -130,16 +130,19 @@ def test_grad_kernel(shape, special):
     assert _same(got, oracle.conv2d_grad_kernel(go, x, KH, KW, sH, sW, pH, pW))
 
 
-def test_forward_large_launch():
-    """A forward launch of 4096 workgroups of 128 pixels: the size from which the two-wave
-    kernel keeps its 128-pixel tiles (smaller launches, all the shapes above, take 64-pixel
-    tiles)."""
+def test_large_launch():
+    """Launches of 4096 workgroups of 128 pixels: the size from which the two-wave kernel
+    keeps its 128-pixel tiles (smaller launches, all the shapes above, take 64-pixel tiles)."""
     from repdl_amd import ops
 
     x = gen.relu_like(31, 64, 16, 64, 128)
     w = gen.normal_like(32, 64, 16, 3, 3)
     got = ops.conv2d(x.cuda(), w.cuda(), (1, 1), (1, 1), 1)
     assert gen.sha256(got) == gen.sha256(oracle.conv2d(x, w, 1, 1, 1, 1, 1))
+    go = gen.normal_like(33, 64, 16, 64, 128)
+    w2 = gen.normal_like(34, 16, 64, 3, 3)
+    got = ops.conv2d_grad_input((64, 64, 64, 128), w2.cuda(), go.cuda(), (1, 1), (1, 1))
+    assert gen.sha256(got) == gen.sha256(oracle.conv2d_grad_input(go, w2, 64, 128, 1, 1, 1, 1))
 
 
 @pytest.mark.parametrize("layer", [(64, 64, 56, 56, 64, 3, 1, 1), (64, 256, 56, 56, 64, 1, 1, 0)], ids=["3x3_64_64", "1x1_256_64"])
