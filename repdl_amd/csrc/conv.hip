@@ -735,31 +735,34 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_kernel(const float *__restri
 // epilogue.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void conv_pad_kernel(const float *__restrict__ src, float *__restrict__ dst,
-                                                       int64_t total, int H, int W, int Hp, int Wp, int PT, int PL,
+                                                       int64_t planes, int H, int W, int Hp, int Wp, int PT, int PL,
                                                        unsigned *__restrict__ parts)
 {
-    // grid-stride: at most GUARD_PARTS workgroups, each leaves the minimum of what it copied
+    // A workgroup takes whole planes (grid-stride: at most GUARD_PARTS workgroups, each leaves
+    // the minimum of what it copied); inside a plane the index arithmetic is 32-bit.
     unsigned m = GUARD_NONE;
-    for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256)
+    const int plane = Hp * Wp;
+    for (int64_t pl = blockIdx.x; pl < planes; pl += gridDim.x)
     {
-        const int wp = (int)(idx % Wp);
-        const int64_t t = idx / Wp;
-        const int hp = (int)(t % Hp);
-        const int64_t pl = t / Hp;
-        const int h = hp - PT, w = wp - PL;
-        const float v = (h >= 0 && h < H && w >= 0 && w < W) ? src[(pl * H + h) * W + w] : 0.0f;
-        dst[idx] = v;
-        m = guard_min(m, guard_bits(v));
+        const float *__restrict__ sp = src + pl * H * W;
+        float *__restrict__ dp = dst + pl * plane;
+        for (int i = threadIdx.x; i < plane; i += 256)
+        {
+            const int hp = i / Wp, wp = i - hp * Wp;
+            const int h = hp - PT, w = wp - PL;
+            const float v = (h >= 0 && h < H && w >= 0 && w < W) ? sp[h * W + w] : 0.0f;
+            dp[i] = v;
+            m = guard_min(m, guard_bits(v));
+        }
     }
     m = guard_block_min(m);
     if (threadIdx.x == 0)
         parts[blockIdx.x] = m;
 }
 
-inline unsigned pad_blocks(int64_t total)
+inline unsigned pad_blocks(int64_t planes)
 {
-    const int64_t b = (total + 255) / 256;
-    return (unsigned)(b < 1 ? 1 : (b > GUARD_PARTS ? GUARD_PARTS : b)); // 2048 x 256 threads fill the chip
+    return (unsigned)(planes < 1 ? 1 : (planes > GUARD_PARTS ? GUARD_PARTS : planes)); // 2048 x 256 threads fill the chip
 }
 
 // Blocks [0, ceil(K / 256)) write the table; for grad-input the blocks after them write the
@@ -1618,9 +1621,9 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
                                (int)plane, (int)Wp, MODE, d.IC, d.pH + PT, d.pW + PL, kernel, WT);
             if (pad)
             {
-                const int64_t total = (int64_t)d.N * img;
-                ca = (int)pad_blocks(total);
-                hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)ca), dim3(256), 0, s, gathered, Gp, total, GH, GW,
+                const int64_t planes = (int64_t)d.N * C;
+                ca = (int)pad_blocks(planes);
+                hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)ca), dim3(256), 0, s, gathered, Gp, planes, GH, GW,
                                    (int)Hp, (int)Wp, PT, PL, guard_parts(guard, 0));
             }
             if (skips)
@@ -1788,7 +1791,8 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
         }
         const int64_t xW = (W + 3) / 4 * 4; // input row pitch the staging waves read
         const bool xpad = xW != W;
-        if (R > 0 && N * (OH / R) <= REPDL_I32_MAX && fits_i32(IC * H * xW) && fits_i32(repdl_cdiv(NC, 16)) &&
+        if (R > 0 && N * (OH / R) <= REPDL_I32_MAX && fits_i32(IC * H * xW) && fits_i32(OC * OH * OWp * 4) &&
+            fits_i32(repdl_cdiv(NC, 16)) &&
             repdl_cdiv(OC, MW_OC) <= 65535)
         {
             // workspace: the guard words, then the operands with rows rounded up to whole
@@ -1810,17 +1814,15 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
                                   s, ca, cb);
             if (xpad)
             {
-                const int64_t total = N * IC * H * xW;
-                cb = (int)pad_blocks(total);
-                hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)cb), dim3(256), 0, s, input, xws, total, (int)H, (int)W,
+                cb = (int)pad_blocks(N * IC);
+                hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)cb), dim3(256), 0, s, input, xws, N * IC, (int)H, (int)W,
                                    (int)H, (int)xW, 0, 0, guard_parts(guard, 1));
             }
             const float *xsrc = xpad ? xws : input;
             if (gpad)
             {
-                const int64_t total = N * OC * OH * OWp;
-                ca = (int)pad_blocks(total);
-                hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)ca), dim3(256), 0, s, grad_output, gws, total, (int)OH,
+                ca = (int)pad_blocks(N * OC);
+                hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)ca), dim3(256), 0, s, grad_output, gws, N * OC, (int)OH,
                                    (int)OW, (int)OH, (int)OWp, 0, 0, guard_parts(guard, 0));
             }
             if (skips)
