@@ -198,19 +198,12 @@ __device__ __forceinline__ bool guard_suspect(float v, bool tiny)
     return (v != v) || (tiny && (__float_as_uint(v) << 1) == 0u);
 }
 
-// Blocks [0, nblk_a) take the minimum over a[0..na) into the parts of operand 0, the
-// others over b[0..nb) into those of operand 1; either range of blocks may be empty.
-__global__ __launch_bounds__(256) void conv_guard_kernel(const float *__restrict__ a, int64_t na,
-                                                         const float *__restrict__ b, int64_t nb, int nblk_a,
-                                                         unsigned *__restrict__ parts_a,
-                                                         unsigned *__restrict__ parts_b)
+// Workgroup blk of nblk: the minimum over its grid-stride share of p[0..n) into parts[blk].
+__device__ __forceinline__ void guard_scan_block(const float *__restrict__ p, int64_t n, int blk, int nblk,
+                                                 unsigned *__restrict__ parts)
 {
     typedef float v4f __attribute__((ext_vector_type(4)));
-    const bool second = (int)blockIdx.x >= nblk_a;
-    const float *__restrict__ p = second ? b : a;
-    const int64_t n = second ? nb : na;
-    const int blk = second ? (int)blockIdx.x - nblk_a : (int)blockIdx.x;
-    const int64_t stride = (int64_t)(second ? (int)gridDim.x - nblk_a : nblk_a) * 256;
+    const int64_t stride = (int64_t)nblk * 256;
     const int64_t first = (int64_t)blk * 256 + threadIdx.x;
     unsigned m = GUARD_NONE;
     int64_t done = 0;
@@ -230,7 +223,20 @@ __global__ __launch_bounds__(256) void conv_guard_kernel(const float *__restrict
         m = guard_min(m, guard_bits(p[i]));
     m = guard_block_min(m);
     if (threadIdx.x == 0)
-        (second ? parts_b : parts_a)[blk] = m;
+        parts[blk] = m;
+}
+
+// Blocks [0, nblk_a) take the minimum over a[0..na) into the parts of operand 0, the
+// others over b[0..nb) into those of operand 1; either range of blocks may be empty.
+__global__ __launch_bounds__(256) void conv_guard_kernel(const float *__restrict__ a, int64_t na,
+                                                         const float *__restrict__ b, int64_t nb, int nblk_a,
+                                                         unsigned *__restrict__ parts_a,
+                                                         unsigned *__restrict__ parts_b)
+{
+    if ((int)blockIdx.x < nblk_a)
+        guard_scan_block(a, na, (int)blockIdx.x, nblk_a, parts_a);
+    else
+        guard_scan_block(b, nb, (int)blockIdx.x - nblk_a, (int)gridDim.x - nblk_a, parts_b);
 }
 
 // guard[op] = minimum of the first count[op] parts of operand op (GUARD_NONE for none)
@@ -765,15 +771,23 @@ inline unsigned pad_blocks(int64_t planes)
     return (unsigned)(planes < 1 ? 1 : (planes > GUARD_PARTS ? GUARD_PARTS : planes)); // 2048 x 256 threads fill the chip
 }
 
-// Blocks [0, ceil(K / 256)) write the table; for grad-input the blocks after them write the
-// kernel operand as the [IC][K] panel the matrix kernel reads, WT[ic][k] = W[oc][ic][kh][kw]
-// for k = (oc, kh, kw).
+// The small jobs of a call in one launch.  Blocks [0, ceil(K / 256)) write the table; for
+// grad-input the wt_blocks after them write the kernel operand as the [IC][K] panel the matrix
+// kernel reads, WT[ic][k] = W[oc][ic][kh][kw] for k = (oc, kh, kw); the scan_blocks after
+// those take the kernel's part of the guard of the zero results.
 __global__ __launch_bounds__(256) void conv_ktab_kernel(int *__restrict__ tabB, int K, int KH, int KW, int plane, int Wp,
                                                         int mode, int IC, int baseH, int baseW,
-                                                        const float *__restrict__ W, float *__restrict__ WT)
+                                                        const float *__restrict__ W, float *__restrict__ WT,
+                                                        int wt_blocks, int64_t kernel_count, int scan_blocks,
+                                                        unsigned *__restrict__ parts)
 {
     const int KHW = KH * KW;
     const int tab_blocks = (K + 255) / 256;
+    if ((int)blockIdx.x >= tab_blocks + wt_blocks)
+    {
+        guard_scan_block(W, kernel_count, (int)blockIdx.x - tab_blocks - wt_blocks, scan_blocks, parts);
+        return;
+    }
     if ((int)blockIdx.x >= tab_blocks)
     {
         const int64_t idx = (int64_t)(blockIdx.x - tab_blocks) * 256 + threadIdx.x; // = ic * K + k
@@ -1611,14 +1625,17 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
             float *Gp = reinterpret_cast<float *>(ws + GUARD_BYTES + tab_bytes + wt_bytes);
             const float *Wa = MODE == MODE_FWD ? kernel : WT;
             // guard[0]: the gathered operand (in the padding pass when there is one), guard[1]: the kernel
-            int ca = 0, cb = 0;
+            // guard: the kernel's part in the table launch, the gathered operand's in the padding pass
+            // when there is one
+            int ca = 0, cb = 0, unused = 0;
+            if (skips && !pad)
+                launch_guard_scan(gathered, gathered_count, nullptr, 0, guard, s, ca, unused);
             if (skips)
-                launch_guard_scan(pad ? nullptr : gathered, gathered_count, kernel, kernel_count, guard, s, ca, cb);
-            else
-                guard = nullptr;
-            const int64_t ktab_blocks = repdl_cdiv(K, 256) + (MODE == MODE_FWD ? 0 : repdl_cdiv((int64_t)M * K, 256));
-            hipLaunchKernelGGL(conv_ktab_kernel, dim3((unsigned)ktab_blocks), dim3(256), 0, s, tabB, (int)K, d.KH, d.KW,
-                               (int)plane, (int)Wp, MODE, d.IC, d.pH + PT, d.pW + PL, kernel, WT);
+                cb = guard_blocks(kernel_count);
+            const int64_t wt_blocks = MODE == MODE_FWD ? 0 : repdl_cdiv((int64_t)M * K, 256);
+            hipLaunchKernelGGL(conv_ktab_kernel, dim3((unsigned)(repdl_cdiv(K, 256) + wt_blocks + cb)), dim3(256), 0, s, tabB,
+                               (int)K, d.KH, d.KW, (int)plane, (int)Wp, MODE, d.IC, d.pH + PT, d.pW + PL, kernel, WT,
+                               (int)wt_blocks, kernel_count, cb, guard_parts(guard, 1));
             if (pad)
             {
                 const int64_t planes = (int64_t)d.N * C;
@@ -1628,6 +1645,8 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
             }
             if (skips)
                 launch_guard_final(guard, ca, cb, s);
+            else
+                guard = nullptr;
             const float *src = pad ? Gp : gathered;
             // Tiles of 64 pixels when that fills the chip more evenly (see conv_small_tiles).
             const bool small_tiles = bm == 64 && conv_small_tiles(gx * (M / bm) * gz);
