@@ -745,20 +745,25 @@ __global__ __launch_bounds__(256) void conv_pad_kernel(const float *__restrict__
                                                        unsigned *__restrict__ parts)
 {
     // A workgroup takes whole planes (grid-stride: at most GUARD_PARTS workgroups, each leaves
-    // the minimum of what it copied); inside a plane the index arithmetic is 32-bit.
+    // the minimum of what it copied); a wave takes rows, a lane columns: no divisions.
     unsigned m = GUARD_NONE;
     const int plane = Hp * Wp;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     for (int64_t pl = blockIdx.x; pl < planes; pl += gridDim.x)
     {
         const float *__restrict__ sp = src + pl * H * W;
         float *__restrict__ dp = dst + pl * plane;
-        for (int i = threadIdx.x; i < plane; i += 256)
+        for (int hp = wave; hp < Hp; hp += 4)
         {
-            const int hp = i / Wp, wp = i - hp * Wp;
-            const int h = hp - PT, w = wp - PL;
-            const float v = (h >= 0 && h < H && w >= 0 && w < W) ? sp[h * W + w] : 0.0f;
-            dp[i] = v;
-            m = guard_min(m, guard_bits(v));
+            const int h = hp - PT;
+            const bool hin = h >= 0 && h < H;
+            for (int wp = lane; wp < Wp; wp += 64)
+            {
+                const int w = wp - PL;
+                const float v = (hin && w >= 0 && w < W) ? sp[h * W + w] : 0.0f;
+                dp[hp * Wp + wp] = v;
+                m = guard_min(m, guard_bits(v));
+            }
         }
     }
     m = guard_block_min(m);
