@@ -742,7 +742,7 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_kernel(const float *__restri
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void conv_pad_kernel(const float *__restrict__ src, float *__restrict__ dst,
                                                        int64_t planes, int H, int W, int Hp, int Wp, int PT, int PL,
-                                                       unsigned *__restrict__ parts)
+                                                       int dH, int dW, unsigned *__restrict__ parts)
 {
     // A workgroup takes whole planes (grid-stride: at most GUARD_PARTS workgroups, each leaves
     // the minimum of what it copied); a wave takes rows, a lane columns: no divisions.
@@ -755,12 +755,15 @@ __global__ __launch_bounds__(256) void conv_pad_kernel(const float *__restrict__
         float *__restrict__ dp = dst + pl * plane;
         for (int hp = wave; hp < Hp; hp += 4)
         {
-            const int h = hp - PT;
-            const bool hin = h >= 0 && h < H;
+            // source element (h, w) lands at (PT + h*dH, PL + w*dW); everything else is zero
+            const int hd = hp - PT;
+            const int h = dH == 1 ? hd : hd / dH;
+            const bool hin = hd >= 0 && h < H && (dH == 1 || h * dH == hd);
             for (int wp = lane; wp < Wp; wp += 64)
             {
-                const int w = wp - PL;
-                const float v = (hin && w >= 0 && w < W) ? sp[h * W + w] : 0.0f;
+                const int wd = wp - PL;
+                const int w = dW == 1 ? wd : wd / dW;
+                const float v = (hin && wd >= 0 && w < W && (dW == 1 || w * dW == wd)) ? sp[h * W + w] : 0.0f;
                 dp[hp * Wp + wp] = v;
                 m = guard_min(m, guard_bits(v));
             }
@@ -1605,17 +1608,29 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
                                         : (KHW > 1 || d.sH > 1 || d.sW > 1 || d.pH > 0 || d.pW > 0);
     // Fast path: whole tiles of channels, whole k-tiles, grad-input only at stride 1.
     const int bm = M <= 64 ? 64 : 128;
-    if (mfma && K % BK == 0 && M % bm == 0 && (MODE == MODE_FWD || (d.sH == 1 && d.sW == 1)))
+    if (mfma && K % BK == 0 && M % bm == 0 && (MODE == MODE_FWD || (d.sH <= 4 && d.sW <= 4)))
     {
+        // Strided grad-input: grad_output goes into the workspace DILATED (stride - 1 zeros between
+        // its elements), after which it is the stride-1 case; the zeros take the place of the taps the
+        // reference skips between the strides.  (The matrix instructions then spend 1 - 1/(sH*sW) of
+        // their time on zeros, still well ahead of the gather with its divisions.)
         const int C = MODE == MODE_FWD ? d.IC : d.OC;                 // channels of the gathered tensor
-        const int GH = MODE == MODE_FWD ? d.H : d.OH, GW = MODE == MODE_FWD ? d.W : d.OW;
+        const int SH = MODE == MODE_FWD ? d.H : d.OH, SW = MODE == MODE_FWD ? d.W : d.OW; // source extents
+        const int DH = MODE == MODE_FWD ? 1 : d.sH, DW = MODE == MODE_FWD ? 1 : d.sW;     // dilation
+        const int GH = (SH - 1) * DH + 1, GW = (SW - 1) * DW + 1;
         const int PT = MODE == MODE_FWD ? d.pH : (d.KH - 1 - d.pH > 0 ? d.KH - 1 - d.pH : 0);
         const int PL = MODE == MODE_FWD ? d.pW : (d.KW - 1 - d.pW > 0 ? d.KW - 1 - d.pW : 0);
-        const int64_t Hp = GH + 2 * (int64_t)PT, Wp = GW + 2 * (int64_t)PL;
+        int64_t Hp = GH + 2 * (int64_t)PT, Wp = GW + 2 * (int64_t)PL;
+        if (MODE == MODE_DGRAD)
+        { // rows / columns of the input that no output reaches still read (zeros) up to h + pH + PT
+            Hp = Hp > d.H + d.pH + PT ? Hp : d.H + d.pH + PT;
+            Wp = Wp > d.W + d.pW + PL ? Wp : d.W + d.pW + PL;
+        }
         const int64_t plane = Hp * Wp, img = (int64_t)C * plane;
-        if (img * 4 < (1LL << 31) && (int64_t)M * K * 4 < (1LL << 31) && (int64_t)d.N * img / 256 < REPDL_I32_MAX)
+        if (SH > 0 && SW > 0 && img * 4 < (1LL << 31) && (int64_t)M * K * 4 < (1LL << 31) &&
+            (int64_t)d.N * img / 256 < REPDL_I32_MAX)
         {
-            const bool pad = PT > 0 || PL > 0;
+            const bool pad = PT > 0 || PL > 0 || DH > 1 || DW > 1 || Hp != GH || Wp != GW;
             // workspace: the guard words, the table, the kernel as [IC][K] panels (grad-input), the padded copy
             const size_t tab_bytes = ((size_t)K * sizeof(int) + 255) / 256 * 256;
             const size_t wt_bytes = MODE == MODE_FWD ? 0 : ((size_t)M * K * sizeof(float) + 255) / 256 * 256;
@@ -1645,8 +1660,8 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
             {
                 const int64_t planes = (int64_t)d.N * C;
                 ca = (int)pad_blocks(planes);
-                hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)ca), dim3(256), 0, s, gathered, Gp, planes, GH, GW,
-                                   (int)Hp, (int)Wp, PT, PL, guard_parts(guard, 0));
+                hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)ca), dim3(256), 0, s, gathered, Gp, planes, SH, SW,
+                                   (int)Hp, (int)Wp, PT, PL, DH, DW, guard_parts(guard, 0));
             }
             if (skips)
                 launch_guard_final(guard, ca, cb, s);
@@ -1840,14 +1855,14 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
             {
                 cb = (int)pad_blocks(N * IC);
                 hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)cb), dim3(256), 0, s, input, xws, N * IC, (int)H, (int)W,
-                                   (int)H, (int)xW, 0, 0, guard_parts(guard, 1));
+                                   (int)H, (int)xW, 0, 0, 1, 1, guard_parts(guard, 1));
             }
             const float *xsrc = xpad ? xws : input;
             if (gpad)
             {
                 ca = (int)pad_blocks(N * OC);
                 hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)ca), dim3(256), 0, s, grad_output, gws, N * OC, (int)OH,
-                                   (int)OW, (int)OH, (int)OWp, 0, 0, guard_parts(guard, 0));
+                                   (int)OW, (int)OH, (int)OWp, 0, 0, 1, 1, guard_parts(guard, 0));
             }
             if (skips)
                 launch_guard_final(guard, ca, cb, s);

@@ -77,8 +77,19 @@ def test_forward(shape, special):
     assert _same(got, oracle.conv2d(x, w, sH, sW, pH, pW, g))
 
 
+# grad-input with strides on the matrix path (IC a multiple of 64, OC*KH*KW of 16): grad_output is
+# dilated into the workspace; input rows and columns that no output reaches (remainders of the stride)
+DGRAD = [s for s in FWD if s[-1] == 1] + [
+    (2, 64, 19, 19, 128, 3, 3, 2, 2, 1, 1, 1),
+    (1, 64, 17, 23, 64, 1, 1, 2, 2, 0, 0, 1),
+    (1, 128, 11, 13, 32, 3, 3, 3, 2, 0, 2, 1),
+    (2, 64, 20, 22, 16, 5, 5, 4, 4, 2, 2, 1),
+    (1, 64, 9, 9, 16, 2, 2, 1, 1, 3, 3, 1),      # padding beyond the kernel reach, stride 1
+]
+
+
 @pytest.mark.parametrize("special", KINDS, ids=KIND_IDS)
-@pytest.mark.parametrize("shape", [s for s in FWD if s[-1] == 1], ids=[str(s) for s in FWD if s[-1] == 1])
+@pytest.mark.parametrize("shape", DGRAD, ids=[str(s) for s in DGRAD])
 def test_grad_input(shape, special):
     from repdl_amd import ops
 
