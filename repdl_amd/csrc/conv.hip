@@ -779,51 +779,73 @@ inline unsigned pad_blocks(int64_t planes)
     return (unsigned)(planes < 1 ? 1 : (planes > GUARD_PARTS ? GUARD_PARTS : planes)); // 2048 x 256 threads fill the chip
 }
 
-// The small jobs of a call in one launch.  Blocks [0, ceil(K / 256)) write the table; for
-// grad-input the wt_blocks after them write the kernel operand as the [IC][K] panel the matrix
-// kernel reads, WT[ic][k] = W[oc][ic][kh][kw] for k = (oc, kh, kw); the scan_blocks after
-// those take the kernel's part of the guard of the zero results.
-__global__ __launch_bounds__(256) void conv_ktab_kernel(int *__restrict__ tabB, int K, int KH, int KW, int plane, int Wp,
-                                                        int mode, int IC, int baseH, int baseW,
-                                                        const float *__restrict__ W, float *__restrict__ WT,
-                                                        int wt_blocks, int64_t kernel_count, int scan_blocks,
+// The small jobs of a call in one launch.  Blocks [0, ceil(Kp / 256)) write the table (entries
+// past K repeat the last one: their kernel values are -0.0f).  The panel_blocks after them write
+// the kernel operand as the panels the matrix kernel reads, [groups][Mp][Kp] with k contiguous,
+// rows past M zero and columns past K -0.0f (a product of -0.0f and finite data is a zero, and
+// adding a zero of either sign changes no accumulator that is not -0.0f: see the guard):
+//   forward     panel[g][m][k] = W[g*M + m][k],                     k = (ic, kh, kw)
+//   grad-input  panel[0][m][k] = W[oc][m][kh][kw],                  k = (oc, kh, kw)
+// (forward with whole tiles reads the kernel itself and has no such blocks).  The scan_blocks
+// after those take the kernel's part of the guard of the zero results.
+__global__ __launch_bounds__(256) void conv_ktab_kernel(int *__restrict__ tabB, int K, int Kp, int M, int Mp, int groups,
+                                                        int KH, int KW, int plane, int Wp, int mode, int IC, int baseH,
+                                                        int baseW, const float *__restrict__ W,
+                                                        float *__restrict__ panel, int panel_blocks,
+                                                        int64_t kernel_count, int scan_blocks,
                                                         unsigned *__restrict__ parts)
 {
     const int KHW = KH * KW;
-    const int tab_blocks = (K + 255) / 256;
-    if ((int)blockIdx.x >= tab_blocks + wt_blocks)
+    const int tab_blocks = (Kp + 255) / 256;
+    if ((int)blockIdx.x >= tab_blocks + panel_blocks)
     {
-        guard_scan_block(W, kernel_count, (int)blockIdx.x - tab_blocks - wt_blocks, scan_blocks, parts);
+        guard_scan_block(W, kernel_count, (int)blockIdx.x - tab_blocks - panel_blocks, scan_blocks, parts);
         return;
     }
     if ((int)blockIdx.x >= tab_blocks)
     {
-        const int64_t idx = (int64_t)(blockIdx.x - tab_blocks) * 256 + threadIdx.x; // = ic * K + k
-        if (idx >= (int64_t)IC * K)
+        const int64_t idx = (int64_t)(blockIdx.x - tab_blocks) * 256 + threadIdx.x; // = (g * Mp + m) * Kp + k
+        if (idx >= (int64_t)groups * Mp * Kp)
             return;
-        const int ic = (int)(idx / K), k = (int)(idx - (int64_t)ic * K);
-        const int oc = k / KHW, rem = k - oc * KHW;
-        WT[idx] = W[((int64_t)oc * IC + ic) * KHW + rem];
+        const int k = (int)(idx % Kp);
+        const int64_t gm = idx / Kp;
+        const int m = (int)(gm % Mp), g = (int)(gm / Mp);
+        float v;
+        if (k >= K)
+            v = -0.0f;
+        else if (m >= M)
+            v = 0.0f;
+        else if (mode == MODE_FWD)
+            v = W[((int64_t)g * M + m) * K + k];
+        else
+        {
+            const int oc = k / KHW, rem = k - oc * KHW;
+            v = W[((int64_t)oc * IC + m) * KHW + rem];
+        }
+        panel[idx] = v;
         return;
     }
     const int k = blockIdx.x * 256 + threadIdx.x;
-    if (k >= K)
+    if (k >= Kp)
         return;
-    const int c = k / KHW, rem = k - c * KHW;
+    const int kk = k < K ? k : K - 1;
+    const int c = kk / KHW, rem = kk - c * KHW;
     const int kh = rem / KW, kw = rem - kh * KW;
     tabB[k] = mode == MODE_FWD ? c * plane + kh * Wp + kw : c * plane + (baseH - kh) * Wp + (baseW - kw);
 }
 
 // PB: 32-pixel blocks per wave (2: tiles of 128 pixels; 1, only with BM = 64: tiles of 64 pixels,
-// twice the workgroups at half the duration, for layers whose 128-pixel tiles fill the chip unevenly)
-template <int BM, int MODE, int PB>
+// twice the workgroups at half the duration, for layers whose 128-pixel tiles fill the chip unevenly);
+// RAGGED: the last row tile has rows past M (not stored)
+template <int BM, int MODE, int PB, bool RAGGED>
 __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__restrict__ Gp,   // padded gathered operand
                                                                 const float *__restrict__ Xg,   // the original one (epilogue)
                                                                 const float *__restrict__ Wt,   // the kernel (epilogue)
                                                                 const float *__restrict__ Wa,   // kernel operand as [M][K] panels
                                                                 float *__restrict__ Out, ConvDims d,
                                                                 const int *__restrict__ tabB, int plane, int Wp,
-                                                                int64_t img_stride, const unsigned *__restrict__ guard)
+                                                                int64_t img_stride, const unsigned *__restrict__ guard,
+                                                                int Mp, int Kp) // panel extents (multiples of BM, BK)
 {
     constexpr int NT = 2 * BM;
     constexpr int LDA = BM + 4;
@@ -844,8 +866,8 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int KHW = d.KH * d.KW;
     const int ICg = d.IC / d.groups, OCg = d.OC / d.groups;
-    const int M = MODE == MODE_FWD ? OCg : d.IC;
-    const int K = (MODE == MODE_FWD ? ICg : d.OC) * KHW;
+    const int M = MODE == MODE_FWD ? OCg : d.IC; // rows that exist; the panels have Mp
+    const int K = Kp;                            // k-steps of the panels and the table
     const int P = MODE == MODE_FWD ? d.OH * d.OW : d.H * d.W;
     const int PW = MODE == MODE_FWD ? d.OW : d.W;
     const int n = MODE == MODE_FWD ? blockIdx.z / d.groups : blockIdx.z;
@@ -861,7 +883,7 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
     const int pix_off = MODE == MODE_FWD ? pph * d.sH * Wp + ppw * d.sW : pph * Wp + ppw;
     const float *Gimg = Gp + (int64_t)n * img_stride + (MODE == MODE_FWD ? (int64_t)g * ICg * plane : 0);
     // kernel operand
-    const float *Wg = MODE == MODE_FWD ? Wa + (int64_t)g * OCg * K : Wa;
+    const float *Wg = Wa + (int64_t)g * Mp * K;
     uint32_t a_voff[2]; // byte offsets of this thread's two float4 slots in the [BM][K] panel
     int a_st[2];
 #pragma unroll
@@ -961,6 +983,8 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
         for (int r = 0; r < 16; r++)
         {
             const int m = m0 + wm * 64 + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3);
+            if (RAGGED && m >= M)
+                continue;
             const int ch = MODE == MODE_FWD ? g * OCg + m : m;
 #pragma unroll
             for (int j = 0; j < PB; j++)
@@ -1604,11 +1628,19 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
     const int64_t kernel_count = (int64_t)d.OC * (d.IC / d.groups) * KHW;
     // does the reference skip any tap?  (forward: only into the padding; grad-input: at the
     // borders of any kernel wider than one tap, and between strides)
-    const bool skips = MODE == MODE_FWD ? (d.pH > 0 || d.pW > 0)
-                                        : (KHW > 1 || d.sH > 1 || d.sW > 1 || d.pH > 0 || d.pW > 0);
-    // Fast path: whole tiles of channels, whole k-tiles, grad-input only at stride 1.
-    const int bm = M <= 64 ? 64 : 128;
-    if (mfma && K % BK == 0 && M % bm == 0 && (MODE == MODE_FWD || (d.sH <= 4 && d.sW <= 4)))
+    const bool skips_geom = MODE == MODE_FWD ? (d.pH > 0 || d.pW > 0)
+                                             : (KHW > 1 || d.sH > 1 || d.sW > 1 || d.pH > 0 || d.pW > 0);
+    // Fast path.  Rows and k-steps are rounded up to whole tiles in a padded copy of the kernel
+    // operand (see conv_ktab_kernel); 128-row tiles when that rounds no further than 64-row ones.
+    const int64_t M64 = repdl_cdiv(M, 64) * 64, M128 = repdl_cdiv(M, 128) * 128;
+    const int bm = (M > 64 && M128 == M64) ? 128 : 64;
+    const int64_t Mp = bm == 128 ? M128 : M64, Kp = repdl_cdiv(K, BK) * BK;
+    const int groups = MODE == MODE_FWD ? d.groups : 1;
+    const bool panel = MODE == MODE_DGRAD || Mp != M || Kp != K;
+    // (forward with few, ragged k-steps -- a 3-channel stem layer -- stays with the gather kernel: copying
+    // its large input into the workspace costs more than the gather, 0.39 against 0.45 ms for 3 -> 64, 3x3)
+    const bool few_k = MODE == MODE_FWD && Kp != K && K < 256;
+    if (mfma && M > 0 && K > 0 && !few_k && (MODE == MODE_FWD || (d.sH <= 4 && d.sW <= 4)))
     {
         // Strided grad-input: grad_output goes into the workspace DILATED (stride - 1 zeros between
         // its elements), after which it is the stride-1 case; the zeros take the place of the taps the
@@ -1627,13 +1659,16 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
             Wp = Wp > d.W + d.pW + PL ? Wp : d.W + d.pW + PL;
         }
         const int64_t plane = Hp * Wp, img = (int64_t)C * plane;
-        if (SH > 0 && SW > 0 && img * 4 < (1LL << 31) && (int64_t)M * K * 4 < (1LL << 31) &&
+        if (SH > 0 && SW > 0 && img * 4 < (1LL << 31) && groups * Mp * Kp * 4 < (1LL << 31) && Mp / bm <= 65535 &&
             (int64_t)d.N * img / 256 < REPDL_I32_MAX)
         {
+            // padded k-steps are zero products too: the guard decides about zero results
+            const bool skips = skips_geom || Kp != K;
             const bool pad = PT > 0 || PL > 0 || DH > 1 || DW > 1 || Hp != GH || Wp != GW;
-            // workspace: the guard words, the table, the kernel as [IC][K] panels (grad-input), the padded copy
-            const size_t tab_bytes = ((size_t)K * sizeof(int) + 255) / 256 * 256;
-            const size_t wt_bytes = MODE == MODE_FWD ? 0 : ((size_t)M * K * sizeof(float) + 255) / 256 * 256;
+            // workspace: the guard words, the table, the kernel operand's panels (when not the kernel itself),
+            // the padded copy of the gathered operand
+            const size_t tab_bytes = ((size_t)Kp * sizeof(int) + 255) / 256 * 256;
+            const size_t wt_bytes = panel ? ((size_t)(groups * Mp * Kp) * sizeof(float) + 255) / 256 * 256 : 0;
             const size_t ws_bytes = GUARD_BYTES + tab_bytes + wt_bytes + (pad ? (size_t)d.N * img * sizeof(float) : 0);
             char *ws = nullptr;
             hipError_t e = hipMallocAsync(reinterpret_cast<void **>(&ws), ws_bytes, s);
@@ -1643,7 +1678,7 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
             int *tabB = reinterpret_cast<int *>(ws + GUARD_BYTES);
             float *WT = reinterpret_cast<float *>(ws + GUARD_BYTES + tab_bytes);
             float *Gp = reinterpret_cast<float *>(ws + GUARD_BYTES + tab_bytes + wt_bytes);
-            const float *Wa = MODE == MODE_FWD ? kernel : WT;
+            const float *Wa = panel ? WT : kernel;
             // guard[0]: the gathered operand (in the padding pass when there is one), guard[1]: the kernel
             // guard: the kernel's part in the table launch, the gathered operand's in the padding pass
             // when there is one
@@ -1652,10 +1687,10 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
                 launch_guard_scan(gathered, gathered_count, nullptr, 0, guard, s, ca, unused);
             if (skips)
                 cb = guard_blocks(kernel_count);
-            const int64_t wt_blocks = MODE == MODE_FWD ? 0 : repdl_cdiv((int64_t)M * K, 256);
-            hipLaunchKernelGGL(conv_ktab_kernel, dim3((unsigned)(repdl_cdiv(K, 256) + wt_blocks + cb)), dim3(256), 0, s, tabB,
-                               (int)K, d.KH, d.KW, (int)plane, (int)Wp, MODE, d.IC, d.pH + PT, d.pW + PL, kernel, WT,
-                               (int)wt_blocks, kernel_count, cb, guard_parts(guard, 1));
+            const int64_t wt_blocks = panel ? repdl_cdiv(groups * Mp * Kp, 256) : 0;
+            hipLaunchKernelGGL(conv_ktab_kernel, dim3((unsigned)(repdl_cdiv(Kp, 256) + wt_blocks + cb)), dim3(256), 0, s, tabB,
+                               (int)K, (int)Kp, M, (int)Mp, groups, d.KH, d.KW, (int)plane, (int)Wp, MODE, d.IC, d.pH + PT,
+                               d.pW + PL, kernel, WT, (int)wt_blocks, kernel_count, cb, guard_parts(guard, 1));
             if (pad)
             {
                 const int64_t planes = (int64_t)d.N * C;
@@ -1669,23 +1704,41 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
                 guard = nullptr;
             const float *src = pad ? Gp : gathered;
             // Tiles of 64 pixels when that fills the chip more evenly (see conv_small_tiles).
-            const bool small_tiles = bm == 64 && conv_small_tiles(gx * (M / bm) * gz);
-            dim3 grid((unsigned)(small_tiles ? repdl_cdiv(P, BN / 2) : gx), (unsigned)(M / bm), (unsigned)gz);
+            const bool small_tiles = bm == 64 && conv_small_tiles(gx * (Mp / bm) * gz);
+            dim3 grid((unsigned)(small_tiles ? repdl_cdiv(P, BN / 2) : gx), (unsigned)(Mp / bm), (unsigned)gz);
+#define REPDL_CONV_FAST(BM_, PB_, RG_)                                                                                  \
+    hipLaunchKernelGGL((conv_gemm_fast_kernel<BM_, MODE, PB_, RG_>), grid, dim3(2 * BM_), 0, s, src, gathered, kernel, \
+                       Wa, out, d, tabB, (int)plane, (int)Wp, img, guard, (int)Mp, (int)Kp)
+            const bool ragged = Mp != M;
             if (bm == 64 && small_tiles)
-                hipLaunchKernelGGL((conv_gemm_fast_kernel<64, MODE, 1>), grid, dim3(128), 0, s, src, gathered, kernel, Wa, out,
-                                   d, tabB, (int)plane, (int)Wp, img, guard);
+            {
+                if (ragged)
+                    REPDL_CONV_FAST(64, 1, true);
+                else
+                    REPDL_CONV_FAST(64, 1, false);
+            }
             else if (bm == 64)
-                hipLaunchKernelGGL((conv_gemm_fast_kernel<64, MODE, 2>), grid, dim3(128), 0, s, src, gathered, kernel, Wa, out,
-                                   d, tabB, (int)plane, (int)Wp, img, guard);
+            {
+                if (ragged)
+                    REPDL_CONV_FAST(64, 2, true);
+                else
+                    REPDL_CONV_FAST(64, 2, false);
+            }
             else
-                hipLaunchKernelGGL((conv_gemm_fast_kernel<128, MODE, 2>), grid, dim3(256), 0, s, src, gathered, kernel, Wa, out,
-                                   d, tabB, (int)plane, (int)Wp, img, guard);
+            {
+                if (ragged)
+                    REPDL_CONV_FAST(128, 2, true);
+                else
+                    REPDL_CONV_FAST(128, 2, false);
+            }
+#undef REPDL_CONV_FAST
             const int rc = repdl_launch_status();
             e = hipFreeAsync(ws, s);
             return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
         }
     }
     REPDL_REQUIRE(repdl_cdiv(M, 128) <= 65535);
+    const bool skips = skips_geom;
     unsigned *guard = nullptr;
     hipError_t ge = hipSuccess;
     if (skips)

@@ -22,8 +22,12 @@ FWD = [
     (2, 64, 19, 19, 128, 3, 3, 2, 2, 1, 1, 2),   # fast path, groups, stride 2
     (1, 16, 12, 40, 128, 5, 5, 1, 2, 1, 3, 1),   # fast path, BM = 128, asymmetric stride / padding
     (2, 16, 9, 9, 64, 1, 1, 1, 1, 1, 1, 1),      # padding beyond the kernel reach
-    (2, 8, 14, 14, 24, 3, 3, 1, 1, 1, 1, 1),     # K = 72: general kernel
+    (2, 8, 14, 14, 24, 3, 3, 1, 1, 1, 1, 1),     # K = 72, few and ragged k-steps: gather kernel
     (1, 12, 10, 11, 70, 3, 2, 2, 1, 0, 1, 1),    # ragged everything
+    (2, 32, 12, 13, 96, 3, 3, 1, 1, 1, 1, 1),    # fast path, 96 rows in a 128-row tile
+    (2, 30, 12, 13, 40, 3, 3, 1, 1, 1, 1, 1),    # fast path, K = 270 rounded up to 272, 40 rows in a 64-row tile
+    (2, 60, 10, 10, 80, 3, 3, 1, 1, 1, 1, 2),    # the same per group
+    (1, 20, 9, 9, 200, 4, 4, 1, 1, 2, 2, 1),     # 200 rows: 64-row tiles (192 + 8)
 ]
 
 
