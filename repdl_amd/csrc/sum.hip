@@ -33,12 +33,16 @@ constexpr int RTILE = 8192;    // floats per tile
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-template <int RR, int RT, bool VEC>
+// MULTI: short segments (sum4d_dim023 on small images) -- a tile row holds `spt` whole
+// segments of its chain back to back instead of a piece of one, so that a tile is still
+// thousands of additions long and its walk covers the latency of the next tile's loads
+// (with one 196-element segment per tile, 64 chains of 12 544 took 158 us; so: 35 us).
+template <int RR, int RT, bool VEC, bool MULTI>
 __global__ __launch_bounds__(RT) void rowchain_kernel(const float *__restrict__ in,
                                                       float *__restrict__ out, int64_t rows,
                                                       int64_t nseg, int64_t seglen,
                                                       int64_t row_stride, int64_t seg_stride,
-                                                      float factor)
+                                                      float factor, int spt)
 {
     constexpr int RC = RTILE / RR; // tile columns
     constexpr int RLD = RC + 4;    // padded LDS row: keeps 16-byte alignment, shifts banks by 4
@@ -50,12 +54,49 @@ __global__ __launch_bounds__(RT) void rowchain_kernel(const float *__restrict__ 
     const int walker = blockIdx.x % (RT / 64);
     const int64_t r0 = (int64_t)blockIdx.x * RR;
     const int64_t tiles_per_seg = (seglen + RC - 1) / RC;
-    const int64_t ntiles = nseg * tiles_per_seg;
+    const int64_t ntiles = MULTI ? (nseg + spt - 1) / spt : nseg * tiles_per_seg;
+    const int slen = (int)seglen; // MULTI: seglen <= RC / 2
 
     float acc = 0.0f;
     v4f stage[RV];
 
+    auto load_multi = [&](int64_t t) {
+        const int64_t s0 = t * spt;
+        const int ns = nseg - s0 < spt ? (int)(nseg - s0) : spt;
+        const int valid = ns * slen;
+#pragma unroll
+        for (int i = 0; i < RV; i++)
+        {
+            const int idx = tid + RT * i;
+            const int64_t r = r0 + idx / C4;
+            const int c = (idx % C4) << 2;
+            v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (r < rows && c < valid)
+            {
+                const float *rowp = in + s0 * seg_stride + r * row_stride;
+                const int sg = c / slen, off = c - sg * slen;
+                if (VEC && (slen & 3) == 0) // the four elements lie in one segment, 16-byte aligned
+                    v = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(rowp + sg * seg_stride + off));
+                else
+                {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                    {
+                        const int ce = c + e, sge = ce / slen;
+                        if (ce < valid)
+                            v[e] = rowp[sge * seg_stride + (ce - sge * slen)];
+                    }
+                }
+            }
+            stage[i] = v;
+        }
+    };
     auto load = [&](int64_t t) {
+        if (MULTI)
+        {
+            load_multi(t);
+            return;
+        }
         const int64_t sgm = t / tiles_per_seg, c0 = (t - sgm * tiles_per_seg) * RC;
         const float *base = in + sgm * seg_stride + c0;
 #pragma unroll
@@ -104,7 +145,7 @@ __global__ __launch_bounds__(RT) void rowchain_kernel(const float *__restrict__ 
         if (wave == walker && lane < RR)
         {
             const int64_t sgm = t / tiles_per_seg, c0 = (t - sgm * tiles_per_seg) * RC;
-            const int64_t rem = seglen - c0;
+            const int64_t rem = MULTI ? (nseg - t * spt < spt ? nseg - t * spt : spt) * seglen : seglen - c0;
             const float *row = &tile[lane * RLD];
             // 8*WB elements per step, the next ones read from LDS before the adds of the current
             // ones: with few chains per workgroup the walk is the critical path, and it should
@@ -288,15 +329,27 @@ static int launch_rowchain(const float *in, float *out, int64_t rows, int64_t ns
     REPDL_REQUIRE(grid <= REPDL_I32_MAX);
     const dim3 g((unsigned)grid);
     hipStream_t st = repdl_stream(stream);
-#define REPDL_ROWCHAIN(RRv, RTv)                                                                                \
-    do                                                                                                         \
-    {                                                                                                          \
-        if (vec)                                                                                               \
-            hipLaunchKernelGGL((rowchain_kernel<RRv, RTv, true>), g, dim3(RTv), 0, st, in, out, rows, nseg,    \
-                               seglen, row_stride, seg_stride, factor);                                        \
-        else                                                                                                   \
-            hipLaunchKernelGGL((rowchain_kernel<RRv, RTv, false>), g, dim3(RTv), 0, st, in, out, rows, nseg,   \
-                               seglen, row_stride, seg_stride, factor);                                        \
+    // short segments: whole segments per tile row (see MULTI)
+    const int64_t rc = RTILE / rr;
+    const bool multi = nseg > 1 && seglen > 0 && 2 * seglen <= rc;
+    const int spt = multi ? (int)(rc / seglen) : 1;
+#define REPDL_ROWCHAIN_V(RRv, RTv, V)                                                                               \
+    do                                                                                                             \
+    {                                                                                                              \
+        if (multi)                                                                                                 \
+            hipLaunchKernelGGL((rowchain_kernel<RRv, RTv, V, true>), g, dim3(RTv), 0, st, in, out, rows, nseg,     \
+                               seglen, row_stride, seg_stride, factor, spt);                                       \
+        else                                                                                                       \
+            hipLaunchKernelGGL((rowchain_kernel<RRv, RTv, V, false>), g, dim3(RTv), 0, st, in, out, rows, nseg,    \
+                               seglen, row_stride, seg_stride, factor, spt);                                       \
+    } while (0)
+#define REPDL_ROWCHAIN(RRv, RTv)              \
+    do                                        \
+    {                                         \
+        if (vec)                              \
+            REPDL_ROWCHAIN_V(RRv, RTv, true); \
+        else                                  \
+            REPDL_ROWCHAIN_V(RRv, RTv, false);\
     } while (0)
     if (rr == 64)
         REPDL_ROWCHAIN(64, 256);
@@ -307,6 +360,7 @@ static int launch_rowchain(const float *in, float *out, int64_t rows, int64_t ns
     else
         REPDL_ROWCHAIN(4, 256);
 #undef REPDL_ROWCHAIN
+#undef REPDL_ROWCHAIN_V
     return repdl_launch_status();
 }
 

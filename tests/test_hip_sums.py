@@ -87,7 +87,11 @@ def test_row_and_column_sums(shape):
     assert torch.equal(ops.sum2d_dim1(xu).cpu(), oracle.sum2d_dim1(xu.cpu()))
 
 
-@pytest.mark.parametrize("shape", [(2, 3, 5, 7), (4, 64, 14, 14), (3, 130, 8, 8), (1, 7000, 3, 3)])
+@pytest.mark.parametrize("shape", [(2, 3, 5, 7), (4, 64, 14, 14), (3, 130, 8, 8), (1, 7000, 3, 3),
+                                   # several whole segments per tile row: full and ragged last tiles, widths that are
+                                   # not multiples of 4, more chains per workgroup
+                                   (64, 16, 14, 14), (5, 8, 28, 28), (7, 4, 33, 31), (3, 6200, 4, 4), (23, 5, 2, 2),
+                                   (4, 2, 32, 32), (3, 2, 33, 32)])
 def test_channel_sums(shape):
     from repdl_amd import ops
 
