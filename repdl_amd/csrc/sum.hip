@@ -333,15 +333,31 @@ static int launch_rowchain(const float *in, float *out, int64_t rows, int64_t ns
     const int64_t rc = RTILE / rr;
     const bool multi = nseg > 1 && seglen > 0 && 2 * seglen <= rc;
     const int spt = multi ? (int)(rc / seglen) : 1;
-#define REPDL_ROWCHAIN_V(RRv, RTv, V)                                                                               \
+    // Few workgroups (each walk is then the critical path): ask for LDS the kernel does not use,
+    // so that a workgroup has its CU to itself.  81 KiB in all: neither a second one of these nor
+    // a grad-kernel workgroup (84 KiB) of a launch running beside this one on another stream fits
+    // next to it -- a walk that shares its SIMD with matrix instructions ran 1.85 times longer.
+    const size_t lds_pad = grid <= 256 ? 48 * 1024 : 0;
+#define REPDL_ROWCHAIN_M(RRv, RTv, V, MU)                                                                           \
     do                                                                                                             \
     {                                                                                                              \
-        if (multi)                                                                                                 \
-            hipLaunchKernelGGL((rowchain_kernel<RRv, RTv, V, true>), g, dim3(RTv), 0, st, in, out, rows, nseg,     \
-                               seglen, row_stride, seg_stride, factor, spt);                                       \
-        else                                                                                                       \
-            hipLaunchKernelGGL((rowchain_kernel<RRv, RTv, V, false>), g, dim3(RTv), 0, st, in, out, rows, nseg,    \
-                               seglen, row_stride, seg_stride, factor, spt);                                       \
+        if (lds_pad != 0)                                                                                          \
+        {                                                                                                          \
+            hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void *>(&rowchain_kernel<RRv, RTv, V, MU>), \
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_pad);         \
+            if (e_ != hipSuccess)                                                                                  \
+                return (int)e_;                                                                                    \
+        }                                                                                                          \
+        hipLaunchKernelGGL((rowchain_kernel<RRv, RTv, V, MU>), g, dim3(RTv), lds_pad, st, in, out, rows, nseg,     \
+                           seglen, row_stride, seg_stride, factor, spt);                                           \
+    } while (0)
+#define REPDL_ROWCHAIN_V(RRv, RTv, V)              \
+    do                                             \
+    {                                              \
+        if (multi)                                 \
+            REPDL_ROWCHAIN_M(RRv, RTv, V, true);   \
+        else                                       \
+            REPDL_ROWCHAIN_M(RRv, RTv, V, false);  \
     } while (0)
 #define REPDL_ROWCHAIN(RRv, RTv)              \
     do                                        \
@@ -361,6 +377,7 @@ static int launch_rowchain(const float *in, float *out, int64_t rows, int64_t ns
         REPDL_ROWCHAIN(4, 256);
 #undef REPDL_ROWCHAIN
 #undef REPDL_ROWCHAIN_V
+#undef REPDL_ROWCHAIN_M
     return repdl_launch_status();
 }
 

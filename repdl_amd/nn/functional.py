@@ -44,6 +44,39 @@ def linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tenso
     return _Linear.apply(input, weight, bias)
 
 
+_SIDE_STREAMS = {}
+
+
+def _side_by_side(device: torch.device, jobs):
+    """Runs independent jobs (callables returning a tensor, or None for "not needed") and
+    returns their results in order.  On the GPU the first needed job runs on the current
+    stream and the others on side streams of their own (default priority, made once per
+    device), so that they overlap: the reductions and the grad-kernel of a backward pass are
+    chains as long as the batch -- bound by the latency of one chain, busy on a fraction of
+    the CUs -- and side by side they take the time of the longest instead of the sum.
+    The results are what the jobs return one after the other: the jobs are independent."""
+    todo = [i for i, j in enumerate(jobs) if j is not None]
+    out = [None] * len(jobs)
+    if device.type != "cuda" or len(todo) < 2:
+        for i in todo:
+            out[i] = jobs[i]()
+        return out
+    key = device.index if device.index is not None else torch.cuda.current_device()
+    streams = _SIDE_STREAMS.setdefault(key, [])
+    while len(streams) < len(todo) - 1:
+        streams.append(torch.cuda.Stream(device=key))
+    cur = torch.cuda.current_stream(key)
+    for st, i in zip(streams, todo[1:]):
+        st.wait_stream(cur)  # the inputs are complete
+        with torch.cuda.stream(st):
+            out[i] = jobs[i]()
+    out[todo[0]] = jobs[todo[0]]()
+    for st, i in zip(streams, todo[1:]):
+        cur.wait_stream(st)  # later work on the current stream sees the result, and the inputs are
+        out[i].record_stream(cur)  # not reused before the side stream is done with them
+    return out
+
+
 class _Conv2d(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, bias, stride, padding, groups):
@@ -61,9 +94,11 @@ class _Conv2d(torch.autograd.Function):
             raise NotImplementedError("conv2d backward: groups != 1")
         x, weight = ctx.saved_tensors
         need_x, need_w, need_b = ctx.needs_input_grad[:3]
-        gx = ops.conv2d_grad_input(x.shape, weight, gy, stride, padding) if need_x else None
-        gw = ops.conv2d_grad_kernel(x, weight.shape, gy, stride, padding) if need_w else None
-        gb = ops.sum4d_dim023(gy) if need_b else None
+        # grad-input fills the chip; grad-kernel and the bias sum are latency-bound chains: side by side
+        gx, gw, gb = _side_by_side(gy.device, [
+            (lambda: ops.conv2d_grad_input(x.shape, weight, gy, stride, padding)) if need_x else None,
+            (lambda: ops.conv2d_grad_kernel(x, weight.shape, gy, stride, padding)) if need_w else None,
+            (lambda: ops.sum4d_dim023(gy)) if need_b else None])
         return gx, gw, gb, None, None, None
 
 
@@ -134,14 +169,16 @@ class _BatchNorm(torch.autograd.Function):
         reduce = ops.sum4d_dim023 if gy.dim() == 4 else ops.sum2d_dim0
         need = ctx.needs_input_grad
         w_over_std = ops.div(weight, std)
-        gx = _per_channel(w_over_std, gy) * gy if need[0] else None
-        gmean = (-w_over_std) * reduce(gy) if need[1] else None
-        gvar = None
-        if need[2]:
-            coef = ops.div(weight, 2 * std * std * std)
-            gvar = reduce(gy * (mean_b - x) * _per_channel(coef, gy))
-        gweight = reduce(ops.div(x - mean_b, std_b.expand_as(x)) * gy) if need[3] else None
-        gbias = reduce(gy) if need[4] else None
+        coef = ops.div(weight, 2 * std * std * std) if need[2] else None
+        # one elementwise product and up to three reductions (grad_mean and grad_bias share theirs:
+        # the same operator on the same tensor), all independent: side by side
+        gx, rgy, gvar, gweight = _side_by_side(gy.device, [
+            (lambda: _per_channel(w_over_std, gy) * gy) if need[0] else None,
+            (lambda: reduce(gy)) if need[1] or need[4] else None,
+            (lambda: reduce(gy * (mean_b - x) * _per_channel(coef, gy))) if need[2] else None,
+            (lambda: reduce(ops.div(x - mean_b, std_b.expand_as(x)) * gy)) if need[3] else None])
+        gmean = (-w_over_std) * rgy if need[1] else None
+        gbias = rgy if need[4] else None
         return gx, gmean, gvar, gweight, gbias, None
 
 

@@ -103,3 +103,40 @@ def test_cnn_training_bits(optim):
     a, b = _both(build, run)
     print(optim, "weights", b[0], "logits", b[1], flush=True)
     assert a == b
+
+
+def test_backward_streams_repeated():
+    """The backward passes of conv2d and batch_norm run their independent gradients on side
+    streams.  Many passes in a row with fresh tensors each time (so that the allocator reuses
+    blocks across the streams) must give, every time, the bits of the operators called one
+    after the other on the current stream."""
+    from repdl_amd import ops
+    from repdl_amd.nn import functional as F
+
+    for it in range(12):
+        N, IC, H, W, OC = 8, 16 + 8 * (it % 3), 20, 20, 32
+        x = gen.relu_like(300 + it, N, IC, H, W).cuda().requires_grad_(True)
+        w = (gen.normal_like(400 + it, OC, IC, 3, 3) * 0.1).cuda().requires_grad_(True)
+        b = gen.normal_like(500 + it, OC).cuda().requires_grad_(True)
+        go = gen.normal_like(600 + it, N, OC, H, W).cuda()
+        F.conv2d(x, w, b, 1, 1).backward(go)
+        torch.cuda.synchronize()
+        assert torch.equal(x.grad, ops.conv2d_grad_input(x.shape, w.detach(), go, (1, 1), (1, 1))), it
+        assert torch.equal(w.grad, ops.conv2d_grad_kernel(x.detach(), w.shape, go, (1, 1), (1, 1))), it
+        assert torch.equal(b.grad, ops.sum4d_dim023(go)), it
+
+        mean = gen.normal_like(700 + it, OC).cuda().requires_grad_(True)
+        var = (gen.relu_like(800 + it, OC) + 0.5).cuda().requires_grad_(True)
+        gamma = gen.normal_like(900 + it, OC).cuda().requires_grad_(True)
+        beta = gen.normal_like(1000 + it, OC).cuda().requires_grad_(True)
+        y = gen.normal_like(1100 + it, N, OC, H, W).cuda().requires_grad_(True)
+        from repdl_amd.nn.functional import _BatchNorm
+        _BatchNorm.apply(y, mean, var, gamma, beta, 1e-5).backward(go)
+        torch.cuda.synchronize()
+        std = ops.sqrt(var.detach() + 1e-5)
+        pc = lambda t: t.view(1, -1, 1, 1)
+        assert torch.equal(beta.grad, ops.sum4d_dim023(go)), it
+        assert torch.equal(mean.grad, (-ops.div(gamma.detach(), std)) * ops.sum4d_dim023(go)), it
+        assert torch.equal(gamma.grad, ops.sum4d_dim023(ops.div(y.detach() - pc(mean.detach()), pc(std).expand_as(y)) * go)), it
+        coef = ops.div(gamma.detach(), 2 * std * std * std)
+        assert torch.equal(var.grad, ops.sum4d_dim023(go * (pc(mean.detach()) - y.detach()) * pc(coef))), it
