@@ -1549,15 +1549,27 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
         // behind every instruction, pinned there (left alone, the scheduler moves the reads
         // behind the last instructions of the piece, too late for the next one)
         auto step_piece = [&](const float (&ca)[QP], const float (&cb)[QP], float (&na)[QP], float (&nb)[QP]) {
+            // (reads in pairs: two words 16 bytes apart come with one ds_read2_b32, and the wave,
+            // alone on its SIMD, issues an instruction only every 8 clocks or so -- three
+            // instructions per 32-clock matrix instruction were one too many)
 #pragma unroll
-            for (int u = 0; u < QP; u++)
+            for (int u = 0; u < QP; u += 2)
             {
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ca[u], cb[u], acc, 0, 0, 0);
                 if (u == 0)
                     advance_piece(); // under the first instruction
                 na[u] = ap[4 * u];
+                if (u + 1 < QP)
+                    na[u + 1] = ap[4 * u + 4];
                 nb[u] = xp[4 * u * sW];
+                if (u + 1 < QP)
+                    nb[u + 1] = xp[(4 * u + 4) * sW];
                 __builtin_amdgcn_sched_barrier(0);
+                if (u + 1 < QP)
+                {
+                    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ca[u + 1], cb[u + 1], acc, 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         };
         float a0[QP], b0[QP], a1[QP], b1[QP];
