@@ -98,3 +98,17 @@ def test_channel_sums(shape):
     x = gen.scaled_normal(sum(shape), *shape)
     assert torch.equal(ops.sum4d_dim023(x.cuda()).cpu(), oracle.sum4d_dim023(x))
     assert torch.equal(ops.sum(x.cuda(), dim=(0, 2, 3), keepdim=True, average=True).cpu(), oracle.sum4d_dim023(x, True, True))
+
+
+@pytest.mark.parametrize("shape", [(9, 5, 14, 14), (3, 7, 28, 28), (6, 3, 5, 7)])
+def test_channel_sums_unaligned_pointer(shape):
+    """An input that starts 4 bytes off a 16-byte boundary: the scalar loads of the loader, with
+    several segments per tile row."""
+    from repdl_amd import ops
+
+    n = shape[0] * shape[1] * shape[2] * shape[3]
+    flat = gen.scaled_normal(77, n + 1)
+    x = flat[1:].view(*shape)
+    xd = flat.cuda()[1:].view(*shape)
+    assert xd.data_ptr() % 16 != 0
+    assert torch.equal(ops.sum4d_dim023(xd).cpu(), oracle.sum4d_dim023(x.contiguous()))
