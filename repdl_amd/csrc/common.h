@@ -19,6 +19,12 @@
 // Inputs at least this long take the parallel evaluation of the sequential sum.
 #define REPDL_SUM1D_MIN_PARALLEL 32768
 
+// Row and channel sums take the parallel evaluation when the chains are at least this long and
+// at most REPDL_SUM_ROWS_MAX_PARALLEL in number (few long chains are bound by the latency of one
+// chain; many chains keep the memory system busy with one lane per chain).
+#define REPDL_SUM_ROWS_MIN_PARALLEL 65536
+#define REPDL_SUM_ROWS_MAX_PARALLEL 512
+
 // Largest extent a kernel indexes with 32-bit arithmetic.
 #define REPDL_I32_MAX 2147483647LL
 
@@ -31,6 +37,13 @@ static inline int repdl_launch_status()
 static inline hipStream_t repdl_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 
 static inline int64_t repdl_cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// sum1d.hip: the exact parallel evaluation of sequential sums, for `rows` chains at once
+// (chain r: nseg segments of seglen contiguous floats, segment s at in + r*row_stride + s*seg_stride;
+// nseg > 1 needs seglen % 16 == 0 and nseg*seglen < 2^31); out[r] = factor * sum.
+size_t repdl_sum_chains_workspace_bytes(int64_t rows, int64_t n);
+int repdl_sum_chains(const float *in, float *out, int64_t rows, int64_t nseg, int64_t seglen, int64_t row_stride,
+                     int64_t seg_stride, float factor, void *workspace, size_t workspace_bytes, void *stream);
 
 // True when the binary32 matrix instructions of the current device were checked (or forced,
 // see repdl_hip_set_matrix_path) to evaluate k-ascending chains of single-rounding FMAs;

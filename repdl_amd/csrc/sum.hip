@@ -321,6 +321,21 @@ static int launch_rowchain(const float *in, float *out, int64_t rows, int64_t ns
 {
     if (rows == 0)
         return REPDL_OK;
+    // Few long chains: one lane per chain would be bound by the latency of a chain (8 to 10 clocks
+    // per element whatever the data).  The parallel evaluation of sum1d.hip, all chains at once.
+    const int64_t len = nseg * seglen;
+    if (rows <= REPDL_SUM_ROWS_MAX_PARALLEL && len >= REPDL_SUM_ROWS_MIN_PARALLEL &&
+        (nseg == 1 || (seglen % 16 == 0 && len <= REPDL_I32_MAX)))
+    {
+        const size_t bytes = repdl_sum_chains_workspace_bytes(rows, len);
+        void *ws = nullptr;
+        hipError_t e = hipMallocAsync(&ws, bytes, repdl_stream(stream));
+        if (e != hipSuccess)
+            return (int)e;
+        const int rc = repdl_sum_chains(in, out, rows, nseg, seglen, row_stride, seg_stride, factor, ws, bytes, stream);
+        e = hipFreeAsync(ws, repdl_stream(stream));
+        return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
+    }
     // Chains per workgroup: enough workgroups to fill 256 CUs two to four times
     // over, all resident at once, and as many walking lanes as that allows.
     const bool vec = (reinterpret_cast<uintptr_t>(in) & 15) == 0 && row_stride % 4 == 0 && seg_stride % 4 == 0;

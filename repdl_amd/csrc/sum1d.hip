@@ -161,11 +161,38 @@ __device__ __forceinline__ Tup tup_join(const Tup &a, const Tup &b)
     return c;
 }
 
-// ---- step 1: binary64 block sums -------------------------------------------------------
-__device__ __forceinline__ void load16(const float *__restrict__ x, int64_t n, int64_t i0, bool vec, float (&v)[16])
+// ---- the chains ------------------------------------------------------------------------------
+// The same pipeline runs on `rows` independent chains at once (row sums of a matrix with few,
+// long rows; the channel sums of an NCHW tensor): row r is blockIdx.y (blockIdx.x in the
+// one-dimensional launches), its element i sits at
+//     x + r*row_stride + (i / seglen)*seg_stride + i % seglen
+// (sum1d and row sums: one segment, seglen = n; channel sums: a segment per image, seglen = H*W,
+// which must then be a multiple of 16 so that the 16 elements of a thread and the float4 of the
+// walk never straddle two segments, and n < 2^31 so that the division is a 32-bit one).  Every
+// per-row array (block sums, prefixes, tuples) holds the rows back to back.
+struct Chains
 {
+    int64_t n, row_stride, seg_stride, nblk, nsup;
+    int seglen;    // (unused unless segmented)
+    int segmented; // more than one segment
+};
+
+__device__ __forceinline__ const float *chain_ptr(const float *__restrict__ xr, const Chains &c, int64_t i)
+{
+    if (!c.segmented)
+        return xr + i;
+    const uint32_t sg = (uint32_t)i / (uint32_t)c.seglen;
+    return xr + (int64_t)sg * c.seg_stride + ((uint32_t)i - sg * (uint32_t)c.seglen);
+}
+
+// ---- step 1: binary64 block sums -------------------------------------------------------
+// 16 consecutive elements from i0 (a multiple of 16) of the chain at xr
+__device__ __forceinline__ void load16(const float *__restrict__ xr, const Chains &c, int64_t i0, bool vec, float (&v)[16])
+{
+    const int64_t n = c.n;
     if (vec && i0 + 15 < n)
     {
+        const float *x = chain_ptr(xr, c, i0) - i0;
 #pragma unroll
         for (int q = 0; q < 4; q++)
         {
@@ -180,7 +207,7 @@ __device__ __forceinline__ void load16(const float *__restrict__ x, int64_t n, i
     {
 #pragma unroll
         for (int q = 0; q < 16; q++)
-            v[q] = (i0 + q < n) ? x[i0 + q] : 0.0f;
+            v[q] = (i0 + q < n) ? *chain_ptr(xr, c, i0 + q) : 0.0f;
     }
 }
 
@@ -227,18 +254,21 @@ __device__ __forceinline__ double quantise(float x, const Quantum &g)
 
 // prev == nullptr: exact sums; else: sums of the elements rounded to the grid of the state
 // prev[block] predicted by the previous pass.
-__global__ __launch_bounds__(256) void sum1d_blocksum_kernel(const float *__restrict__ x, int64_t n,
+__global__ __launch_bounds__(256) void sum1d_blocksum_kernel(const float *__restrict__ x, Chains c,
                                                              const double *__restrict__ prev,
                                                              double *__restrict__ bsum, int vec)
 {
     __shared__ double part[4];
     const int tid = threadIdx.x;
+    const int64_t row = blockIdx.y;
+    x += row * c.row_stride;
+    bsum += row * c.nblk;
     float v[16];
-    load16(x, n, (int64_t)blockIdx.x * BLK + tid * 16, vec, v);
+    load16(x, c, (int64_t)blockIdx.x * BLK + tid * 16, vec, v);
     Quantum g;
     g.q = g.inv_q = 0.0;
     if (prev != nullptr)
-        g = quantum_of(prev[blockIdx.x]);
+        g = quantum_of(prev[row * c.nblk + blockIdx.x]);
     double d = 0.0;
 #pragma unroll
     for (int q = 0; q < 16; q++)
@@ -257,6 +287,8 @@ __global__ __launch_bounds__(256) void sum1d_prefix_kernel(const double *__restr
 {
     __shared__ double seg[256];
     const int tid = threadIdx.x;
+    bsum += (int64_t)blockIdx.x * nblk; // one workgroup per row
+    prefix += (int64_t)blockIdx.x * nblk;
     const int64_t per = (nblk + 255) / 256;
     const int64_t b0 = tid * per, b1 = (b0 + per < nblk) ? b0 + per : nblk;
     double s = 0.0;
@@ -284,7 +316,7 @@ __global__ __launch_bounds__(256) void sum1d_prefix_kernel(const double *__restr
 }
 
 // ---- step 3: chunk and block tuples --------------------------------------------------------
-__global__ __launch_bounds__(256) void sum1d_tuple_kernel(const float *__restrict__ x, int64_t n,
+__global__ __launch_bounds__(256) void sum1d_tuple_kernel(const float *__restrict__ x, Chains c,
                                                           const double *__restrict__ prefix,
                                                           Tup *__restrict__ T1, Tup *__restrict__ TG,
                                                           Tup *__restrict__ T2, int vec)
@@ -292,9 +324,14 @@ __global__ __launch_bounds__(256) void sum1d_tuple_kernel(const float *__restric
     __shared__ double wtot[4];
     __shared__ Tup wt[4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int64_t blk = blockIdx.x;
+    const int64_t blk = blockIdx.x, row = blockIdx.y;
+    x += row * c.row_stride;
+    prefix += row * c.nblk;
+    T1 += row * c.nblk * (BLK / CH);
+    TG += row * c.nblk * GROUPS;
+    T2 += row * c.nblk;
     float v[16];
-    load16(x, n, blk * BLK + tid * 16, vec, v);
+    load16(x, c, blk * BLK + tid * 16, vec, v);
 
     // binary64 exclusive prefix over the threads of the block (elements on the grid of the
     // state predicted for the block start, as in the refined block sums)
@@ -427,6 +464,8 @@ __global__ __launch_bounds__(256) void sum1d_super_kernel(const Tup *__restrict_
     const int64_t sb = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (sb >= nsup)
         return;
+    T2 += (int64_t)blockIdx.y * nblk; // row
+    T3 += (int64_t)blockIdx.y * nsup;
     const int64_t b = sb * SUP + lane;
     Tup t = b < nblk ? T2[b] : tup_identity(HYP_ANY);
 #pragma unroll
@@ -444,18 +483,43 @@ struct BlockRegs
     Tup tgr, tch;
 };
 
-__device__ __forceinline__ void load_block(BlockRegs &r, const float *__restrict__ x, int64_t n,
+// (x: the row's base; T1, TG: the row's tuples)
+__device__ __forceinline__ void load_block(BlockRegs &r, const float *__restrict__ x, const Chains &c,
                                            const Tup *__restrict__ T1, const Tup *__restrict__ TG, int64_t blk, int lane,
                                            int vec)
 {
+    const int64_t n = c.n;
     r.tgr = TG[blk * GROUPS + (lane & (GROUPS - 1))];
     r.tch = T1[blk * (BLK / CH) + lane];
     const int64_t e0 = blk * BLK;
     if (vec && e0 + BLK <= n)
     {
+        if (!c.segmented)
+        {
 #pragma unroll
-        for (int q = 0; q < BLK / 256; q++)
-            r.f[q] = reinterpret_cast<const float4 *>(x + e0)[q * 64 + lane];
+            for (int q = 0; q < BLK / 256; q++)
+                r.f[q] = reinterpret_cast<const float4 *>(x + e0)[q * 64 + lane];
+        }
+        else
+        {
+            // this lane's float4 q starts at element e0 + 4*lane + 256*q: one division for q = 0,
+            // then steps of 256 with the segment wrapped by subtraction (a float4 never straddles
+            // two segments: their length is a multiple of 16)
+            const uint32_t i0 = (uint32_t)(e0 + 4 * lane);
+            uint32_t sg = i0 / (uint32_t)c.seglen;
+            uint32_t off = i0 - sg * (uint32_t)c.seglen;
+#pragma unroll
+            for (int q = 0; q < BLK / 256; q++)
+            {
+                r.f[q] = *reinterpret_cast<const float4 *>(x + (int64_t)sg * c.seg_stride + off);
+                off += 256;
+                while (off >= (uint32_t)c.seglen)
+                {
+                    off -= (uint32_t)c.seglen;
+                    sg++;
+                }
+            }
+        }
     }
     else
     {
@@ -463,10 +527,10 @@ __device__ __forceinline__ void load_block(BlockRegs &r, const float *__restrict
         for (int q = 0; q < BLK / 256; q++)
         {
             const int64_t idx = e0 + (int64_t)(q * 64 + lane) * 4;
-            r.f[q].x = (idx + 0 < n) ? x[idx + 0] : 0.0f; // elements past n: s + 0 = s
-            r.f[q].y = (idx + 1 < n) ? x[idx + 1] : 0.0f;
-            r.f[q].z = (idx + 2 < n) ? x[idx + 2] : 0.0f;
-            r.f[q].w = (idx + 3 < n) ? x[idx + 3] : 0.0f;
+            r.f[q].x = (idx + 0 < n) ? *chain_ptr(x, c, idx + 0) : 0.0f; // elements past n: s + 0 = s
+            r.f[q].y = (idx + 1 < n) ? *chain_ptr(x, c, idx + 1) : 0.0f;
+            r.f[q].z = (idx + 2 < n) ? *chain_ptr(x, c, idx + 2) : 0.0f;
+            r.f[q].w = (idx + 3 < n) ? *chain_ptr(x, c, idx + 3) : 0.0f;
         }
     }
 }
@@ -501,19 +565,26 @@ __device__ __forceinline__ uint32_t replay_chunk(uint32_t s, const f4v (&v)[CH /
 // where the sum moves along a binade boundary), so when a block fails the next block's data
 // and tuples are requested at once, and inside a failing group the LDS reads of a chunk are
 // issued one chunk ahead of the additions.
-__global__ __launch_bounds__(64) void sum1d_walk_kernel(const float *__restrict__ x, int64_t n,
+__global__ __launch_bounds__(64) void sum1d_walk_kernel(const float *__restrict__ x, Chains c,
                                                         const Tup *__restrict__ T1,
                                                         const Tup *__restrict__ TG,
                                                         const Tup *__restrict__ T2,
-                                                        const Tup *__restrict__ T3, int64_t nblk, int64_t nsup,
-                                                        float factor, float *__restrict__ out, int vec)
+                                                        const Tup *__restrict__ T3, float factor,
+                                                        float *__restrict__ out, int vec)
 {
     __shared__ __attribute__((aligned(16))) float xd[BLK + 2 * CH]; // + what the read-ahead overshoots
     const int lane = threadIdx.x;
+    const int64_t row = blockIdx.x, nblk = c.nblk, nsup = c.nsup;
+    x += row * c.row_stride;
+    T1 += row * nblk * (BLK / CH);
+    TG += row * nblk * GROUPS;
+    T2 += row * nblk;
+    T3 += row * nsup;
+    out += row;
     uint32_t s = 0u; // +0.0f; wave-uniform throughout
     BlockRegs pf;    // the block requested ahead
     int64_t pf_blk = -1;
-    load_block(pf, x, n, T1, TG, 0, lane, vec); // (any valid block: the registers are then defined)
+    load_block(pf, x, c, T1, TG, 0, lane, vec); // (any valid block: the registers are then defined)
     pf_blk = 0;
     Tup nsup_t = (lane < nsup) ? T3[lane] : tup_identity(HYP_ANY);
     // block tuples of the super-block being tried, and of the next one
@@ -542,7 +613,7 @@ __global__ __launch_bounds__(64) void sum1d_walk_kernel(const float *__restrict_
                 // The block as a whole does not apply.
                 const int64_t blk = sb * SUP + bi;
                 if (pf_blk != blk)
-                    load_block(pf, x, n, T1, TG, blk, lane, vec);
+                    load_block(pf, x, c, T1, TG, blk, lane, vec);
                 __syncthreads();
 #pragma unroll
                 for (int q = 0; q < BLK / 256; q++)
@@ -551,7 +622,7 @@ __global__ __launch_bounds__(64) void sum1d_walk_kernel(const float *__restrict_
                 __syncthreads();
                 {
                     const int64_t nb = blk + 1 < nblk ? blk + 1 : blk;
-                    load_block(pf, x, n, T1, TG, nb, lane, vec);
+                    load_block(pf, x, c, T1, TG, nb, lane, vec);
                     pf_blk = nb;
                 }
                 for (int gr = 0; gr < GROUPS; gr++)
@@ -587,14 +658,71 @@ inline size_t round256(size_t v) { return (v + 255) & ~(size_t)255; }
 // serial single-chain kernel of sum.hip
 int repdl_sum1d_serial(const float *in, float *out, int64_t n, int average, void *stream);
 
+// Scratch for `rows` chains of n elements.
+size_t repdl_sum_chains_workspace_bytes(int64_t rows, int64_t n)
+{
+    const size_t nblk = (size_t)repdl_cdiv(n, BLK) * (size_t)rows;
+    const size_t nsup = (size_t)repdl_cdiv(repdl_cdiv(n, BLK), SUP) * (size_t)rows;
+    return round256(nblk * sizeof(double)) * 2 + round256(nsup * sizeof(Tup)) + round256(nblk * sizeof(Tup)) +
+           round256(nblk * GROUPS * sizeof(Tup)) + round256(nblk * (BLK / CH) * sizeof(Tup));
+}
+
+// out[r] = factor * (the sequential sum of chain r), r < rows, by the parallel evaluation.
+// Chain r: nseg segments of seglen contiguous floats, segment s at in + r*row_stride +
+// s*seg_stride.  The caller has checked: n = nseg*seglen >= 1, rows in [1, 65535], and for
+// nseg > 1 that seglen is a multiple of 16 and n < 2^31.
+int repdl_sum_chains(const float *in, float *out, int64_t rows, int64_t nseg, int64_t seglen, int64_t row_stride,
+                     int64_t seg_stride, float factor, void *workspace, size_t workspace_bytes, void *stream)
+{
+    const int64_t n = nseg * seglen;
+    REPDL_REQUIRE(rows >= 1 && rows <= 65535 && n >= 1 && in != nullptr && out != nullptr);
+    REPDL_REQUIRE(nseg == 1 || (seglen % 16 == 0 && n <= REPDL_I32_MAX));
+    if (workspace == nullptr || workspace_bytes < repdl_sum_chains_workspace_bytes(rows, n) ||
+        (reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
+        return REPDL_E_WORKSPACE;
+    const int64_t nblk = repdl_cdiv(n, BLK), nsup = repdl_cdiv(nblk, SUP);
+    REPDL_REQUIRE(nblk <= REPDL_I32_MAX);
+    Chains c;
+    c.n = n;
+    c.row_stride = row_stride;
+    c.seg_stride = nseg > 1 ? seg_stride : 0;
+    c.nblk = nblk;
+    c.nsup = nsup;
+    c.seglen = nseg > 1 ? (int)seglen : 0;
+    c.segmented = nseg > 1;
+    char *w = static_cast<char *>(workspace);
+    double *bsum = reinterpret_cast<double *>(w);
+    w += round256(rows * nblk * sizeof(double));
+    double *prefix = reinterpret_cast<double *>(w);
+    w += round256(rows * nblk * sizeof(double));
+    Tup *T3 = reinterpret_cast<Tup *>(w);
+    w += round256(rows * nsup * sizeof(Tup));
+    Tup *T2 = reinterpret_cast<Tup *>(w);
+    w += round256(rows * nblk * sizeof(Tup));
+    Tup *TG = reinterpret_cast<Tup *>(w);
+    w += round256(rows * nblk * GROUPS * sizeof(Tup));
+    Tup *T1 = reinterpret_cast<Tup *>(w);
+    hipStream_t s = repdl_stream(stream);
+    // 16-byte loads: every row and segment starts on a 16-byte boundary
+    const int vec = aligned16(in) && (rows == 1 || row_stride % 4 == 0) && (nseg == 1 || seg_stride % 4 == 0);
+    const dim3 g2((unsigned)nblk, (unsigned)rows);
+    hipLaunchKernelGGL(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(nullptr), bsum, vec);
+    hipLaunchKernelGGL(sum1d_prefix_kernel, dim3((unsigned)rows), dim3(256), 0, s, bsum, prefix, nblk);
+    // one refinement of the prediction (see quantum_of)
+    hipLaunchKernelGGL(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(prefix), bsum, vec);
+    hipLaunchKernelGGL(sum1d_prefix_kernel, dim3((unsigned)rows), dim3(256), 0, s, bsum, prefix, nblk);
+    hipLaunchKernelGGL(sum1d_tuple_kernel, g2, dim3(256), 0, s, in, c, prefix, T1, TG, T2, vec);
+    hipLaunchKernelGGL(sum1d_super_kernel, dim3((unsigned)repdl_cdiv(nsup, 4), (unsigned)rows), dim3(256), 0, s, T2, T3, nblk,
+                       nsup);
+    hipLaunchKernelGGL(sum1d_walk_kernel, dim3((unsigned)rows), dim3(64), 0, s, in, c, T1, TG, T2, T3, factor, out, vec);
+    return repdl_launch_status();
+}
+
 REPDL_API size_t repdl_hip_sum1d_workspace_bytes(int64_t n)
 {
     if (n < REPDL_SUM1D_MIN_PARALLEL)
         return 0;
-    const size_t nblk = (size_t)repdl_cdiv(n, BLK);
-    const size_t nsup = (nblk + SUP - 1) / SUP;
-    return round256(nblk * sizeof(double)) * 2 + round256(nsup * sizeof(Tup)) + round256(nblk * sizeof(Tup)) +
-           round256(nblk * GROUPS * sizeof(Tup)) + round256(nblk * (BLK / CH) * sizeof(Tup));
+    return repdl_sum_chains_workspace_bytes(1, n);
 }
 
 REPDL_API int repdl_hip_sum1d_ws(const float *in, float *out, int64_t n, int average, void *workspace,
@@ -603,38 +731,7 @@ REPDL_API int repdl_hip_sum1d_ws(const float *in, float *out, int64_t n, int ave
     REPDL_REQUIRE(n >= 0 && out != nullptr && (n == 0 || in != nullptr));
     if (n < REPDL_SUM1D_MIN_PARALLEL)
         return repdl_sum1d_serial(in, out, n, average, stream);
-    if (workspace == nullptr || workspace_bytes < repdl_hip_sum1d_workspace_bytes(n) ||
-        (reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
-        return REPDL_E_WORKSPACE;
-    const int64_t nblk = repdl_cdiv(n, BLK);
-    REPDL_REQUIRE(nblk <= REPDL_I32_MAX);
-    char *w = static_cast<char *>(workspace);
-    double *bsum = reinterpret_cast<double *>(w);
-    w += round256(nblk * sizeof(double));
-    double *prefix = reinterpret_cast<double *>(w);
-    w += round256(nblk * sizeof(double));
-    const int64_t nsup = repdl_cdiv(nblk, SUP);
-    Tup *T3 = reinterpret_cast<Tup *>(w);
-    w += round256(nsup * sizeof(Tup));
-    Tup *T2 = reinterpret_cast<Tup *>(w);
-    w += round256(nblk * sizeof(Tup));
-    Tup *TG = reinterpret_cast<Tup *>(w);
-    w += round256(nblk * GROUPS * sizeof(Tup));
-    Tup *T1 = reinterpret_cast<Tup *>(w);
-    hipStream_t s = repdl_stream(stream);
-    const int vec = aligned16(in);
-    hipLaunchKernelGGL(sum1d_blocksum_kernel, dim3((unsigned)nblk), dim3(256), 0, s, in, n,
-                       static_cast<const double *>(nullptr), bsum, vec);
-    hipLaunchKernelGGL(sum1d_prefix_kernel, dim3(1), dim3(256), 0, s, bsum, prefix, nblk);
-    // one refinement of the prediction (see quantum_of)
-    hipLaunchKernelGGL(sum1d_blocksum_kernel, dim3((unsigned)nblk), dim3(256), 0, s, in, n,
-                       static_cast<const double *>(prefix), bsum, vec);
-    hipLaunchKernelGGL(sum1d_prefix_kernel, dim3(1), dim3(256), 0, s, bsum, prefix, nblk);
-    hipLaunchKernelGGL(sum1d_tuple_kernel, dim3((unsigned)nblk), dim3(256), 0, s, in, n, prefix, T1, TG, T2, vec);
-    hipLaunchKernelGGL(sum1d_super_kernel, dim3((unsigned)repdl_cdiv(nsup, 4)), dim3(256), 0, s, T2, T3, nblk, nsup);
-    hipLaunchKernelGGL(sum1d_walk_kernel, dim3(1), dim3(64), 0, s, in, n, T1, TG, T2, T3, nblk, nsup,
-                       repdl_sum_factor(average, n), out, vec);
-    return repdl_launch_status();
+    return repdl_sum_chains(in, out, 1, 1, n, 0, 0, repdl_sum_factor(average, n), workspace, workspace_bytes, stream);
 }
 
 REPDL_API int repdl_hip_sum1d(const float *in, float *out, int64_t n, int average, void *stream)

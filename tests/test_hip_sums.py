@@ -112,3 +112,51 @@ def test_channel_sums_unaligned_pointer(shape):
     xd = flat.cuda()[1:].view(*shape)
     assert xd.data_ptr() % 16 != 0
     assert torch.equal(ops.sum4d_dim023(xd).cpu(), oracle.sum4d_dim023(x.contiguous()))
+
+
+def _long_rows():
+    """Few, long chains: row sums and channel sums that take the parallel evaluation (chains of at
+    least 65536 elements, at most 512 of them), with the data that attacks it."""
+    r = _rng(12)
+    L = 70_000
+    rows = [
+        gen.uniform_pm1(7, L).numpy(),
+        (r.random(L) * 3).astype(np.float32),
+        np.concatenate([[1024.0], np.where(r.random(L - 1) < 0.5, 1.0, -1.0) + r.standard_normal(L - 1) * 1e-3]).astype(np.float32),
+        np.concatenate([[2.0**24], np.ones(L // 2 - 1), [-2.0**23], np.full(L - L // 2 - 1, 0.5)]).astype(np.float32),
+        np.zeros(L, dtype=np.float32),
+        np.concatenate([r.standard_normal(L // 2), [np.inf], r.standard_normal(L - L // 2 - 1)]).astype(np.float32),
+        (r.integers(-2**20, 2**20, L).astype(np.float64) * 2.0**-149).astype(np.float32),
+        np.tile(np.array([3.25, -3.25, 1e-3, -1e-3], dtype=np.float32), L // 4),
+    ]
+    return np.stack(rows)
+
+
+def test_row_sums_few_long_rows():
+    from repdl_amd import ops
+
+    m = torch.from_numpy(_long_rows())  # 8 x 70000 (70000 % 16 == 0)
+    got, want = ops.sum2d_dim1(m.cuda()).cpu(), oracle.sum2d_dim1(m)
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(got), nan) and torch.equal(got[~nan].view(torch.int32), want[~nan].view(torch.int32))
+    m2 = gen.scaled_normal(90, 5, 65537)  # a row length that is no multiple of 4: scalar loads
+    assert torch.equal(ops.sum2d_dim1(m2.cuda()).cpu(), oracle.sum2d_dim1(m2))
+    m3 = gen.uniform_pm1(91, 300, 66000)
+    assert torch.equal(ops.sum2d_dim1(m3.cuda(), average=True).cpu(), oracle.sum2d_dim1(m3, average=True))
+
+
+@pytest.mark.parametrize("shape", [(8, 5, 96, 96), (3, 4, 160, 144), (70, 3, 32, 32), (9, 2, 90, 90), (2, 64, 224, 224)])
+def test_channel_sums_few_long_chains(shape):
+    """Channel sums whose chains (N*H*W elements) are long and few: a segment per image; (9, 2, 90, 90)
+    has segments that are no multiple of 16 and stays with the row-chain kernel."""
+    from repdl_amd import ops
+
+    x = gen.uniform_pm1(sum(shape), *shape) if shape[0] != 3 else gen.scaled_normal(5, *shape)
+    assert torch.equal(ops.sum4d_dim023(x.cuda()).cpu(), oracle.sum4d_dim023(x))
+    xr = x.clamp(min=0)
+    assert torch.equal(ops.sum4d_dim023(xr.cuda(), average=True).cpu(), oracle.sum4d_dim023(xr, average=True))
+    n = x.numel()
+    flat = torch.cat([torch.zeros(1), x.view(-1)]).cuda()
+    xd = flat[1:].view(*shape)  # 4 bytes off a 16-byte boundary
+    assert xd.data_ptr() % 16 != 0
+    assert torch.equal(ops.sum4d_dim023(xd).cpu(), oracle.sum4d_dim023(x))
