@@ -36,8 +36,8 @@ HBM_PEAK_GBS = 8000.0
 # reads 524300 for 1 GiB (factor 1.99995 KiB per count), WRITE_SIZE 1048576 (factor 1.0).  Summary:
 # profiles/hbm_traffic_counters.txt.  Valid for the default workload sizes only.
 MEASURED_TRAFFIC_BYTES = {
-    "mm": 5257433 * 1.99995 * 1024 + 262146 * 1024,       # 1.10e10: operand panels re-read behind L2 (37 % L2 hit rate)
-    "exp": 524343 * 1.99995 * 1024 + 1048580 * 1024,      # 2.147e9 = the algorithmic 8 B/element
+    "mm": 5454440 * 1.99995 * 1024 + 262145 * 1024,       # 1.14e10: operand panels re-read behind L2 (35 % L2 hit rate)
+    "exp": 524338 * 1.99995 * 1024 + 1048579 * 1024,      # 2.147e9 = the algorithmic 8 B/element
     "sum2d_dim1": 524395 * 1.99995 * 1024 + 64 * 1024,    # 1.074e9 = the algorithmic 4 B/element
 }
 
