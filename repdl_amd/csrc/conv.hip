@@ -15,9 +15,8 @@
 // unless acc is -0.0f, and a chain can hold -0.0f only after a product so small
 // that it rounds to zero; with non-finite data the padded product is a NaN that
 // sticks.  So the epilogue recomputes with the literal skip-the-tap chain (the
-// *_exact functions below, which are also the whole of the direct kernels) every NaN
-// result, and the zero results only when the operands can produce such a product
-// (see "the guard of the zero results" below).
+// *_exact functions below) every NaN result, and the zero results only when the
+// operands can produce such a product (see "the guard of the zero results" below).
 //
 // grad-kernel has only OC*IC*KH*KW outputs, each a chain as long as the batch
 // (N*OH*OW): it is limited by chain length and parallelism, not by FMA rate.
@@ -118,23 +117,6 @@ __device__ __forceinline__ float conv2d_grad_kernel_exact(const float *__restric
         }
     }
     return sum;
-}
-
-__global__ __launch_bounds__(64) void conv2d_grad_kernel_direct(const float *__restrict__ GO,
-                                                                const float *__restrict__ I,
-                                                                float *__restrict__ GK, ConvDims d,
-                                                                int64_t total)
-{
-    const int64_t idx = (int64_t)blockIdx.x * 64 + threadIdx.x;
-    if (idx >= total)
-        return;
-    const int kw = (int)(idx % d.KW);
-    int64_t t = idx / d.KW;
-    const int kh = (int)(t % d.KH);
-    t /= d.KH;
-    const int ic = (int)(t % d.IC);
-    const int oc = (int)(t / d.IC);
-    GK[idx] = conv2d_grad_kernel_exact(GO, I, d, oc, ic, kh, kw);
 }
 
 // ---------------------------------------------------------------------------
@@ -1025,12 +1007,6 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
 // NaN results suspect as in the implicit GEMMs; those are recomputed with the
 // literal chain.
 // ---------------------------------------------------------------------------
-// value of v in lane k (a compile-time lane index), broadcast as a wave-uniform scalar
-__device__ __forceinline__ float lane_value(float v, int k)
-{
-    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), k));
-}
-
 // A step of a chain is an instruction pair: the FMA of this step and, next to it, the
 // broadcast for the step eight ahead.  v_readlane_b32 has a long latency before its SGPR
 // result can feed a VALU operand (about 12 clocks measured), short enough to hide behind
