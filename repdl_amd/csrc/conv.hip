@@ -1585,6 +1585,85 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
     }
 }
 
+// ---------------------------------------------------------------------------
+// grad-kernel as one matrix product, for layers with MANY SHORT chains (the late layers of
+// a network: 512 x 512 x 3 x 3 chains of 64 x 7 x 7 steps).  The chain kernel above is built
+// for the opposite case; there it pays its per-workgroup start-up a dozen times over.
+//     GK[oc][(ic,kh,kw)] = sum_k GOt[k][oc] * col[k][(ic,kh,kw)],   k = (n, oh, ow) ascending
+// with GOt the grad_output with k outermost and col the im2col of the input (a zero where the
+// tap falls outside the image), both written into a workspace; the product is repdl_hip_mm
+// (transA), whose chains run over k in exactly this order.  The zeros stand for skipped taps
+// as everywhere: a pass over the result recomputes the NaN results, and the zero results when
+// the guard asks, with the literal chain.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void wgrad_got_kernel(const float *__restrict__ GO, float *__restrict__ GOt, int64_t total,
+                                                        int OC, int OHW)
+{
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; // = k * OC + oc
+    if (idx >= total)
+        return;
+    const int oc = (int)(idx % OC);
+    const int64_t k = idx / OC;
+    const int64_t n = k / OHW;
+    const int p = (int)(k - n * OHW);
+    GOt[idx] = GO[(n * OC + oc) * OHW + p];
+}
+
+__global__ __launch_bounds__(256) void wgrad_col_kernel(const float *__restrict__ X, float *__restrict__ col, int64_t total,
+                                                        ConvDims d, int NC)
+{
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; // = k * NC + (ic, kh, kw)
+    if (idx >= total)
+        return;
+    const int c = (int)(idx % NC);
+    const int64_t k = idx / NC;
+    const int KHW = d.KH * d.KW;
+    const int ic = c / KHW, rem = c - ic * KHW;
+    const int kh = rem / d.KW, kw = rem - kh * d.KW;
+    const int ow = (int)(k % d.OW);
+    const int64_t t = k / d.OW;
+    const int oh = (int)(t % d.OH);
+    const int64_t n = t / d.OH;
+    const int h = oh * d.sH - d.pH + kh, w = ow * d.sW - d.pW + kw;
+    col[idx] = (h >= 0 && h < d.H && w >= 0 && w < d.W) ? X[((n * d.IC + ic) * d.H + h) * d.W + w] : 0.0f;
+}
+
+__global__ __launch_bounds__(256) void wgrad_fixup_kernel(const float *__restrict__ GO, const float *__restrict__ X,
+                                                          float *__restrict__ GK, ConvDims d, int64_t total,
+                                                          const unsigned *__restrict__ guard)
+{
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total)
+        return;
+    const float v = GK[idx];
+    if (!guard_suspect(v, guard_tiny(guard)))
+        return;
+    const int kw = (int)(idx % d.KW);
+    int64_t t = idx / d.KW;
+    const int kh = (int)(t % d.KH);
+    t /= d.KH;
+    const int ic = (int)(t % d.IC);
+    const int oc = (int)(t / d.IC);
+    GK[idx] = conv2d_grad_kernel_exact(GO, X, d, oc, ic, kh, kw);
+}
+
+// Rough times of the two grad-kernel routes (seconds), from measurements on the layers of a
+// ResNet at batch 64: the chain kernel needs 12 clocks per step of a chain and about 34 us per
+// round of 256 workgroups (one per CU) on top; the product runs at about 100 TFLOP/s once it
+// has enough tiles, never faster than its own k-chain (32 clocks per step with 32x32x2
+// instructions), plus the passes that write its operands.
+inline bool wgrad_prefers_gemm(int64_t OC, int64_t NC, int64_t K)
+{
+    const double clk = 1.0 / 2.35e9;
+    const double rounds = (double)repdl_cdiv(repdl_cdiv(NC, 16) * repdl_cdiv(OC, 32), 256);
+    const double step = (double)K * 12.0 * clk;
+    const double t_chain = rounds <= 1.0 ? step : rounds * (step + 34e-6);
+    const double flop = 2.0 * (double)OC * (double)NC * (double)K;
+    const double t_mm = flop / 100e12 > (double)K * 32.0 * clk ? flop / 100e12 : (double)K * 32.0 * clk;
+    const double t_gemm = t_mm + (double)K * (double)(NC + OC) * 8.0 / 3e12 + 40e-6;
+    return t_gemm < 0.8 * t_chain;
+}
+
 inline bool fits_i32(int64_t v) { return v >= 0 && v <= REPDL_I32_MAX; }
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
@@ -1820,6 +1899,46 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
     ConvDims d{(int)N, (int)IC, (int)H, (int)W, (int)OC, (int)KH, (int)KW, (int)OH,
                (int)OW, (int)sH, (int)sW, (int)pH, (int)pW, 1};
     hipStream_t s = repdl_stream(stream);
+
+    // Many short chains: one matrix product (see wgrad_col_kernel).
+    {
+        const int64_t NC = IC * KH * KW, K = N * OH * OW;
+        if (repdl_mfma_exact() && K > 0 && fits_i32(K) && fits_i32(NC) && K * NC < (1LL << 31) && K * OC < (1LL << 31) &&
+            wgrad_prefers_gemm(OC, NC, K))
+        {
+            const bool skips = pH > 0 || pW > 0;
+            const size_t got_bytes = ((size_t)(K * OC) * sizeof(float) + 255) / 256 * 256;
+            const size_t col_bytes = (size_t)(K * NC) * sizeof(float);
+            char *ws = nullptr;
+            hipError_t e = hipMallocAsync(reinterpret_cast<void **>(&ws), GUARD_BYTES + got_bytes + col_bytes, s);
+            if (e != hipSuccess)
+                return (int)e;
+            unsigned *guard = reinterpret_cast<unsigned *>(ws);
+            float *GOt = reinterpret_cast<float *>(ws + GUARD_BYTES);
+            float *col = reinterpret_cast<float *>(ws + GUARD_BYTES + got_bytes);
+            if (skips)
+            {
+                int ca = 0, cb = 0;
+                launch_guard_scan(grad_output, N * OC * OH * OW, input, N * IC * H * W, guard, s, ca, cb);
+                launch_guard_final(guard, ca, cb, s);
+            }
+            hipLaunchKernelGGL(wgrad_got_kernel, dim3((unsigned)repdl_cdiv(K * OC, 256)), dim3(256), 0, s, grad_output, GOt,
+                               K * OC, (int)OC, (int)(OH * OW));
+            hipLaunchKernelGGL(wgrad_col_kernel, dim3((unsigned)repdl_cdiv(K * NC, 256)), dim3(256), 0, s, input, col, K * NC,
+                               d, (int)NC);
+            int rc = repdl_launch_status();
+            if (rc == REPDL_OK)
+                rc = repdl_hip_mm(GOt, col, grad_kernel, OC, NC, K, 1, 0, stream);
+            if (rc == REPDL_OK && skips)
+            {
+                hipLaunchKernelGGL(wgrad_fixup_kernel, dim3((unsigned)repdl_cdiv(total, 256)), dim3(256), 0, s, grad_output,
+                                   input, grad_kernel, d, total, guard);
+                rc = repdl_launch_status();
+            }
+            e = hipFreeAsync(ws, s);
+            return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
+        }
+    }
 
     // Matrix-instruction kernel: geometry of a chunk (see conv_wgrad_mfma_kernel).
     if (repdl_mfma_exact() && sW <= 16 && aligned16(grad_output) && aligned16(input) && OW > 0)

@@ -122,6 +122,9 @@ WGRAD = [
     (2, 3, 5, 3, 4, 1, 1, 1, 1, 0, 0),       # OW = 3: pieces of 1
     (2, 4, 12, 40, 6, 3, 5, 1, 3, 1, 2),     # stride 3 along the row
     (1, 2, 8, 70, 3, 1, 3, 1, 17, 0, 1),     # stride 17: v_fma_f32 kernel
+    (4, 64, 7, 7, 512, 3, 3, 1, 1, 1, 1),    # many short chains: one matrix product over an im2col workspace
+    (2, 128, 7, 7, 2048, 1, 1, 1, 1, 0, 0),  # the same, 1x1 without padding (nothing to fix up)
+    (3, 64, 15, 15, 512, 3, 3, 2, 2, 1, 1),  # the same with strides
 ]
 
 
