@@ -79,7 +79,9 @@ int repdl_hip_mm(const float *A, const float *B, float *C, int64_t M, int64_t N,
  * tap in grad-input); on the matrix path also a zero-padded copy of the gathered operand
  * of conv2d / conv2d_grad_input with two small offset tables, and for conv2d_grad_kernel
  * copies of grad_output / input with rows rounded up to a multiple of 4 floats when
- * their widths are not one.  At most the size of the operands with their borders. */
+ * their widths are not one -- at most the size of the operands with their borders -- or,
+ * for layers with many short chains (OC*IC*KH*KW large, N*OH*OW small), grad_output with
+ * the batch outermost and the im2col of the input (N*OH*OW * IC*KH*KW floats, below 2^31). */
 int repdl_hip_conv2d(const float *input, const float *kernel, float *output, int64_t N, int64_t IC,
                      int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t sH,
                      int64_t sW, int64_t pH, int64_t pW, int64_t groups, void *stream);
