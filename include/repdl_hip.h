@@ -77,7 +77,8 @@ int repdl_hip_mm(const float *A, const float *B, float *C, int64_t M, int64_t N,
  * allocator (hipMallocAsync / hipFreeAsync on `stream`): 17 KiB whenever the geometry
  * makes the reference skip taps (padding, strides of grad-input, kernels wider than one
  * tap in grad-input); on the matrix path also a zero-padded copy of the gathered operand
- * of conv2d / conv2d_grad_input with two small offset tables, and for conv2d_grad_kernel
+ * of conv2d / conv2d_grad_input with two small offset tables (or, for images of at most
+ * 100 pixels with many channels, its im2col: output elements x IC*KH*KW floats), and for conv2d_grad_kernel
  * copies of grad_output / input with rows rounded up to a multiple of 4 floats when
  * their widths are not one -- at most the size of the operands with their borders -- or,
  * for layers with many short chains (OC*IC*KH*KW large, N*OH*OW small), grad_output with

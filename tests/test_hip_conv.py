@@ -28,6 +28,12 @@ FWD = [
     (2, 30, 12, 13, 40, 3, 3, 1, 1, 1, 1, 1),    # fast path, K = 270 rounded up to 272, 40 rows in a 64-row tile
     (2, 60, 10, 10, 80, 3, 3, 1, 1, 1, 1, 2),    # the same per group
     (1, 20, 9, 9, 200, 4, 4, 1, 1, 2, 2, 1),     # 200 rows: 64-row tiles (192 + 8)
+    # small images, many channels: one matrix product over an im2col workspace (forward and grad-input)
+    (32, 64, 8, 8, 128, 3, 3, 1, 1, 1, 1, 1),
+    (24, 128, 9, 10, 64, 3, 3, 1, 1, 1, 1, 1),
+    (40, 128, 15, 15, 128, 3, 3, 2, 2, 1, 1, 1),   # (forward only: its 15x15 input is too large for grad-input to take this route)
+    (32, 128, 9, 9, 128, 5, 3, 2, 1, 2, 1, 1),     # strides in grad-input: input 9x9, output 5x9
+    (32, 512, 8, 8, 128, 1, 1, 1, 1, 0, 0, 1),
 ]
 
 
