@@ -103,7 +103,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--quick", action="store_true", help="headline only, no secondary operators, no full parity")
-    ap.add_argument("--only", default="", help="comma list of secondary ops to run (sum2d,sum1d,exp,log,sqrt,div,conv)")
+    ap.add_argument("--only", default="", help="comma list of secondary ops to run (sum2d,sum1d,exp,log,sqrt,div,conv,adam)")
     ap.add_argument("--size", type=int, default=8192, help="mm size (M=N=K); the metric is quoted at 8192")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 1 GiB elementwise copy kernel (torch.add(x, 0)), the known-size kernel "
@@ -315,6 +315,30 @@ def main() -> int:
                         "cpu_baseline": {"value": round(flop / dt / 1e9, 2), "unit": "GFLOP/s", "cores": oracle.threads(),
                                          "kind": "port", "sample": "the full layer"}})
                 del x_d, w_d, go_d
+
+        if want("adam"):
+            import ctypes
+            import math
+
+            na = 1 << 26
+            g = torch.Generator().manual_seed(7)
+            p_h, g_h = torch.randn(na, generator=g) * 0.05, torch.randn(na, generator=g) * torch.exp2(torch.rand(na, generator=g) * 20 - 20)
+            m_h, v_h = torch.randn(na, generator=g) * 1e-3, torch.rand(na, generator=g) * 1e-5
+            lr, betas, eps, wd, t = 1e-3, (0.9, 0.999), 1e-8, 1e-2, 10
+            dev_t = [x.to(dev) for x in (p_h, g_h, m_h, v_h)]
+            desc = (_lib.AdamTensor * 1)(_lib.AdamTensor(dev_t[0].data_ptr(), dev_t[1].data_ptr(), dev_t[2].data_ptr(),
+                                                         dev_t[3].data_ptr(), None, na, math.sqrt(1 - betas[1] ** t),
+                                                         -(lr / (1 - betas[0] ** t))))
+            stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+            def f(): _lib.call("repdl_hip_adam_step", desc, 1, betas[0], 1 - betas[0], betas[1], 1 - betas[1], eps, wd, stream)
+            f()  # one step on both sides, compared before the timed steps run on
+            dt, _ = cpu_time(lambda: oracle.adam_step(p_h, g_h, m_h, v_h, None, t, lr, betas, eps, wd))
+            par = {"equal": all(sha(a) == sha(b) for a, b in zip(dev_t, (p_h, g_h, m_h, v_h))), "sha256_gpu": sha(dev_t[0])}
+            cpu = {"value": round(28.0 * na / dt / 1e9, 3), "unit": "GB/s", "cores": oracle.threads(), "kind": "port",
+                   "sample": "the full 2^26 elements, one step"}
+            result["also"].append(hbm_entry("adam_step", "one fused Adam step (weight decay on) over 2^26 parameters",
+                                            28.0 * na, f, args.steps, args.warmup, par, cpu))
+            del dev_t
 
     if args.copy_probe:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()

@@ -11,7 +11,8 @@
  * Conventions
  *   - All pointers are DEVICE pointers to contiguous row-major float32 data
  *     (int64 for class labels) on the device that is current when the call is
- *     made.  Outputs are caller-allocated.  Inputs are never written.
+ *     made.  Outputs are caller-allocated.  Inputs are never written
+ *     (the optimizer steps update their state tensors in place and say so).
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
  *     Calls enqueue work and return without synchronising.
  *   - Return value: 0 on success; a positive value is a hipError_t from the
@@ -158,6 +159,56 @@ int repdl_hip_softmax(const float *in, float *out, int64_t M, int64_t N, void *s
  * indices in [0,N), out is one float.  workspace: M floats of device memory. */
 int repdl_hip_cross_entropy(const float *in, const int64_t *target, float *out, int64_t M,
                             int64_t N, float *workspace, void *stream);
+
+/* Optimizer steps -- the reference has no backend function for these: repdl/optim.py:56-83
+ * writes Adam as a sequence of PyTorch tensor operations around ops.sqrt and a true
+ * division (a dozen launches and temporaries per parameter).  These entry points evaluate
+ * that same sequence per element, every rounding in the same place, in one pass over all
+ * the tensors of a parameter group.  param, exp_avg, exp_avg_sq and max_exp_avg_sq are
+ * updated in place; grad is read only; tensors must not overlap.  The scalars are the
+ * binary32 roundings of the values the Python code computes in binary64 (PyTorch rounds a
+ * Python number that meets a float32 tensor once, to binary32).  A NaN operand gives a NaN
+ * result whose sign and payload are unspecified.
+ *
+ * Adam, per element (optim.py:64-83), with b1 = beta1, c1 = one_minus_beta1 = float(1 - beta1),
+ * likewise b2 and c2:
+ *   g' = weight_decay != 0 ? fma(weight_decay, p, g) : g
+ *   m  = fma(c1, g', RN(m * b1))
+ *   v  = RN(RN(v * b2) + RN(RN(g' * g') * c2))
+ *   s  = max_exp_avg_sq ? (vmax = max(vmax, v), NaN if either is) : v
+ *   d  = RN(RN(RN(sqrt(s)) / sqrt_bias_correction2) + eps), a true division
+ *   p  = RN(p + RN(RN(m / d) * step_scale))
+ * where sqrt_bias_correction2 = float(sqrt(1 - beta2^t)) and step_scale =
+ * float(-(lr / (1 - beta1^t))) for the tensor's step count t (optim.py:60-61, 82).
+ * max_exp_avg_sq == NULL means amsgrad is off for that tensor. */
+typedef struct
+{
+    float *param;
+    const float *grad;
+    float *exp_avg;
+    float *exp_avg_sq;
+    float *max_exp_avg_sq;
+    int64_t n;
+    float sqrt_bias_correction2;
+    float step_scale;
+} repdl_adam_tensor;
+
+/* tensors: HOST array of `count` descriptors (device pointers inside); read before the
+ * call returns.  Empty tensors (n == 0) are skipped. */
+int repdl_hip_adam_step(const repdl_adam_tensor *tensors, int count, float beta1, float one_minus_beta1,
+                        float beta2, float one_minus_beta2, float eps, float weight_decay, void *stream);
+
+/* Plain gradient descent with both roundings kept: p = RN(p - RN(g * lr)).  (PyTorch's own
+ * update, param.add_(grad, alpha=-lr), rounds once on devices that fuse it and twice on
+ * those that do not.) */
+typedef struct
+{
+    float *param;
+    const float *grad;
+    int64_t n;
+} repdl_sgd_tensor;
+
+int repdl_hip_sgd_step(const repdl_sgd_tensor *tensors, int count, float lr, void *stream);
 
 #ifdef __cplusplus
 }

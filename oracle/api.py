@@ -33,6 +33,8 @@ def lib() -> ctypes.CDLL:
         _lib.repdl_oracle_cross_entropy.restype = ctypes.c_float
         _lib.repdl_oracle_threads.restype = ctypes.c_int
         _lib.repdl_oracle_div_scalar.argtypes = [_P, ctypes.c_float, _P, _I64]
+        _lib.repdl_oracle_adam_step.argtypes = [_P, _P, _P, _P, _P, _I64] + [ctypes.c_float] * 8
+        _lib.repdl_oracle_sgd_step.argtypes = [_P, _P, _I64, ctypes.c_float]
     return _lib
 
 
@@ -168,3 +170,26 @@ def cross_entropy(input, target) -> torch.Tensor:
     scratch = torch.empty(x.shape[0], dtype=torch.float32)
     v = lib().repdl_oracle_cross_entropy(_p(x), _p(t), _I64(x.shape[0]), _I64(x.shape[1]), _p(scratch))
     return torch.tensor(v, dtype=torch.float32)
+
+
+def adam_step(param, grad, exp_avg, exp_avg_sq, max_exp_avg_sq, step, lr, betas, eps, weight_decay) -> None:
+    """One Adam update of one tensor, in place (repdl/optim.py:56-83); ``step`` is the
+    count after the increment; ``max_exp_avg_sq`` None = amsgrad off.  The scalars are
+    computed in binary64 as the Python code does and rounded to binary32 once."""
+    import math
+
+    beta1, beta2 = betas
+    for t in (param, exp_avg, exp_avg_sq, max_exp_avg_sq):
+        if t is not None and (t.device.type != "cpu" or t.dtype != torch.float32 or not t.is_contiguous()):
+            raise TypeError("oracle updates contiguous float32 CPU tensors in place")
+    g = _f32(grad)
+    bc1, bc2 = 1 - beta1 ** step, 1 - beta2 ** step
+    lib().repdl_oracle_adam_step(
+        _p(param), _p(g), _p(exp_avg), _p(exp_avg_sq), _p(max_exp_avg_sq) if max_exp_avg_sq is not None else None,
+        _I64(param.numel()), beta1, 1 - beta1, beta2, 1 - beta2, eps, weight_decay, math.sqrt(bc2), -(lr / bc1))
+
+
+def sgd_step(param, grad, lr) -> None:
+    if param.device.type != "cpu" or param.dtype != torch.float32 or not param.is_contiguous():
+        raise TypeError("oracle updates contiguous float32 CPU tensors in place")
+    lib().repdl_oracle_sgd_step(_p(param), _p(_f32(grad)), _I64(param.numel()), lr)

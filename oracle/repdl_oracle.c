@@ -342,20 +342,21 @@ ORACLE_API void repdl_oracle_log(const float *I, float *O, int64_t n)
  *   0xFFC00000 that a bare sqrtsd gives); NaN inputs keep sign and payload and
  *   are quieted; sqrt(-0) = -0.
  * ---------------------------------------------------------------------- */
+static inline float ieee_sqrt(float x)
+{
+    uint32_t u = f2u(x);
+    if ((u & 0x7fffffffu) > 0x7f800000u)
+        return u2f(u | 0x00400000u);
+    if ((u >> 31) && (u & 0x7fffffffu))
+        return u2f(0x7fc00000u);
+    return (float)sqrt((double)x);
+}
+
 ORACLE_API void repdl_oracle_sqrt(const float *I, float *O, int64_t n)
 {
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < n; i++)
-    {
-        float x = I[i];
-        uint32_t u = f2u(x);
-        if ((u & 0x7fffffffu) > 0x7f800000u)
-            O[i] = u2f(u | 0x00400000u);
-        else if ((u >> 31) && (u & 0x7fffffffu))
-            O[i] = u2f(0x7fc00000u);
-        else
-            O[i] = (float)sqrt((double)x);
-    }
+        O[i] = ieee_sqrt(I[i]);
 }
 
 /* ------------------------------------------------------------------------
@@ -457,4 +458,74 @@ ORACLE_API float repdl_oracle_cross_entropy(const float *I, const int64_t *targe
         scratch[i] = l;
     }
     return repdl_oracle_sum1d(scratch, M, 1);
+}
+
+/* ------------------------------------------------------------------------
+ * Optimizer steps.  repdl/optim.py:56-83 writes Adam as PyTorch tensor
+ *   operations, each rounding once; this is that sequence per element, with
+ *   the scalars already rounded to binary32 as PyTorch rounds a Python number
+ *   that meets a float32 tensor:
+ *     :64-66  grad.add(param, alpha=wd)       -> fmaf(wd, p, g)   [only if wd != 0]
+ *     :68     exp_avg.mul_(b1).add_(g, alpha) -> fmaf(c1, g, m * b1)
+ *             (Tensor.add with alpha is one fused multiply-add in PyTorch's CPU
+ *             kernels, vector body and scalar tail alike; checked against torch
+ *             in tests/test_oracle_pin.py)
+ *     :69     exp_avg_sq.mul_(b2).add_(mul(g, g).mul(c2)): four roundings
+ *     :71-74  torch.maximum: NaN if either operand is
+ *     :75-81  ops.div(ops.sqrt(s), sqrt(bc2)).add_(eps)
+ *     :82-83  param.add_(div(exp_avg, denom).mul(-step_size))
+ *   vmax == NULL: amsgrad off.  Pinning: against the same sequence of torch
+ *   CPU operators over several steps (tests/test_oracle_pin.py).
+ * ---------------------------------------------------------------------- */
+static inline float max_nan(float a, float b)
+{
+    if (a != a)
+        return a;
+    if (b != b)
+        return b;
+    return a > b ? a : b;
+}
+
+ORACLE_API void repdl_oracle_adam_step(float *P, const float *G, float *M, float *V, float *VMAX, int64_t n,
+                                       float b1, float c1, float b2, float c2, float eps, float wd,
+                                       float sqrt_bc2, float step_scale)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++)
+    {
+        float g = G[i];
+        if (wd != 0.0f)
+            g = fmaf(wd, P[i], g);
+        const float mb = M[i] * b1;
+        const float m = fmaf(c1, g, mb);
+        const float vb = V[i] * b2;
+        const float gg = g * g;
+        const float ggc = gg * c2;
+        const float v = vb + ggc;
+        float s = v;
+        if (VMAX)
+        {
+            s = max_nan(VMAX[i], v);
+            VMAX[i] = s;
+        }
+        const float root = ieee_sqrt(s);
+        const float scaled = ieee_div(root, sqrt_bc2);
+        const float denom = scaled + eps;
+        const float q = ieee_div(m, denom);
+        const float upd = q * step_scale;
+        P[i] = P[i] + upd;
+        M[i] = m;
+        V[i] = v;
+    }
+}
+
+/* p <- p - RN(g * lr): two roundings (the product, then the difference). */
+ORACLE_API void repdl_oracle_sgd_step(float *P, const float *G, int64_t n, float lr)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++)
+    {
+        const float step = G[i] * lr;
+        P[i] = P[i] - step;
+    }
 }

@@ -17,6 +17,21 @@ _I64 = ctypes.c_int64
 _INT = ctypes.c_int
 _F32 = ctypes.c_float
 
+
+
+class AdamTensor(ctypes.Structure):
+    """repdl_adam_tensor of repdl_hip.h"""
+
+    _fields_ = [("param", _P), ("grad", _P), ("exp_avg", _P), ("exp_avg_sq", _P), ("max_exp_avg_sq", _P),
+                ("n", _I64), ("sqrt_bias_correction2", _F32), ("step_scale", _F32)]
+
+
+class SgdTensor(ctypes.Structure):
+    """repdl_sgd_tensor of repdl_hip.h"""
+
+    _fields_ = [("param", _P), ("grad", _P), ("n", _I64)]
+
+
 # name -> argument types (all return int), exactly the declarations of repdl_hip.h
 SIGNATURES = {
     "repdl_hip_mm": [_P, _P, _P, _I64, _I64, _I64, _INT, _INT, _P],
@@ -35,6 +50,8 @@ SIGNATURES = {
     "repdl_hip_div_scalar": [_P, _F32, _P, _I64, _P],
     "repdl_hip_softmax": [_P, _P, _I64, _I64, _P],
     "repdl_hip_cross_entropy": [_P, _P, _P, _I64, _I64, _P, _P],
+    "repdl_hip_adam_step": [ctypes.POINTER(AdamTensor), _INT] + [_F32] * 6 + [_P],
+    "repdl_hip_sgd_step": [ctypes.POINTER(SgdTensor), _INT, _F32, _P],
     "repdl_hip_mfma_selftest": [_I64, _I64, ctypes.c_uint64, ctypes.POINTER(ctypes.c_uint64)],
     "repdl_hip_set_matrix_path": [_INT],
 }
