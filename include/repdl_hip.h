@@ -71,6 +71,14 @@ int repdl_hip_matrix_path(void);
 int repdl_hip_mm(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K,
                  int transA, int transB, void *stream);
 
+/* mm with the bias of a linear layer -- repdl/nn/linear.py:21-22, 37: `mm(x, W, transB)`
+ * followed by `+= bias`.  The reference makes the addition a second pass over the
+ * output; here it is the last operation on each output's register: C(i,j) =
+ * RN(chain(i,j) + bias[j]), one IEEE addition after the complete chain, the same bits.
+ * bias is [N] (NULL: no bias, exactly repdl_hip_mm). */
+int repdl_hip_mm_bias(const float *A, const float *B, const float *bias, float *C, int64_t M, int64_t N,
+                      int64_t K, int transA, int transB, void *stream);
+
 /* conv2d -- backend/cuda/convolution.cu:153-183 (bound at :385); semantics
  * backend/cpu/convolution.cpp:12-52.  NCHW; kernel is [OC, IC/groups, KH, KW];
  * output is [N, OC, OH, OW] with OH = (H + 2 pH - KH) / sH + 1.
@@ -87,6 +95,14 @@ int repdl_hip_mm(const float *A, const float *B, float *C, int64_t M, int64_t N,
 int repdl_hip_conv2d(const float *input, const float *kernel, float *output, int64_t N, int64_t IC,
                      int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t sH,
                      int64_t sW, int64_t pH, int64_t pW, int64_t groups, void *stream);
+
+/* conv2d with the layer's bias -- repdl/nn/conv.py:27-28: conv2d followed by
+ * `+= bias` broadcast over [N, OC, OH, OW].  output(n,oc,oh,ow) = RN(chain + bias[oc]):
+ * one IEEE addition after the complete chain, made in the kernel's epilogue instead of
+ * a second pass over the output.  bias is [OC] (NULL: none, exactly repdl_hip_conv2d). */
+int repdl_hip_conv2d_bias(const float *input, const float *kernel, const float *bias, float *output, int64_t N,
+                          int64_t IC, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t sH,
+                          int64_t sW, int64_t pH, int64_t pW, int64_t groups, void *stream);
 
 /* conv2d_grad_input -- backend/cuda/convolution.cu:259-287 (bound at :386);
  * semantics backend/cpu/convolution.cpp:54-90.  groups == 1.

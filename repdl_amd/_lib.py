@@ -35,7 +35,9 @@ class SgdTensor(ctypes.Structure):
 # name -> argument types (all return int), exactly the declarations of repdl_hip.h
 SIGNATURES = {
     "repdl_hip_mm": [_P, _P, _P, _I64, _I64, _I64, _INT, _INT, _P],
+    "repdl_hip_mm_bias": [_P, _P, _P, _P, _I64, _I64, _I64, _INT, _INT, _P],
     "repdl_hip_conv2d": [_P, _P, _P] + [_I64] * 12 + [_P],
+    "repdl_hip_conv2d_bias": [_P, _P, _P, _P] + [_I64] * 12 + [_P],
     "repdl_hip_conv2d_grad_input": [_P, _P, _P] + [_I64] * 13 + [_P],
     "repdl_hip_conv2d_grad_kernel": [_P, _P, _P] + [_I64] * 13 + [_P],
     "repdl_hip_sum1d": [_P, _P, _I64, _INT, _P],

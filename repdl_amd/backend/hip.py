@@ -1,7 +1,8 @@
 """``repdl_amd.backend.hip`` -- the module that takes the place of RepDL's compiled
 ``repdl.backend.cuda`` (backend/cuda/bind.cpp:12-19): the same ten functions with the
 same positional signatures, tensors in and a new tensor out, plus the elementwise
-operators (``exp``, ``log``, ``sqrt``, ``div``, ``div_scalar``).
+operators (``exp``, ``log``, ``sqrt``, ``div``, ``div_scalar``) and ``mm_bias`` /
+``conv2d_bias`` (a layer's bias added in the kernel's epilogue).
 
 Two bindings of the one C-ABI library (include/repdl_hip.h) can serve it:
 
@@ -22,7 +23,13 @@ except ImportError:  # not built
     _ext_binding = None
 
 FUNCTIONS = ("mm", "conv2d", "conv2d_grad_input", "conv2d_grad_kernel", "sum1d", "sum2d_dim0", "sum2d_dim1",
-             "sum4d_dim023", "softmax", "cross_entropy", "exp", "log", "sqrt", "div", "div_scalar")
+             "sum4d_dim023", "softmax", "cross_entropy", "exp", "log", "sqrt", "div", "div_scalar", "mm_bias", "conv2d_bias")
+if _ext_binding is not None and not all(hasattr(_ext_binding, fn) for fn in FUNCTIONS):
+    import warnings
+
+    warnings.warn("repdl_amd.backend._hip_ext was built from an older csrc/bind.cpp and is ignored; "
+                  "rebuild it with `python -m repdl_amd.build`")
+    _ext_binding = None
 BINDING = None
 
 

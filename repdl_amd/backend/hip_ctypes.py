@@ -2,7 +2,8 @@
 ``repdl.backend.cuda`` (backend/cuda/bind.cpp:12-19) bound to the C ABI with ctypes:
 the same ten functions with the same positional signatures, tensors in and a new
 tensor out, plus the elementwise operators (``exp``, ``log``, ``sqrt``, ``div``,
-``div_scalar``).  ``repdl_amd.backend.hip`` serves these when the compiled binding
+``div_scalar``) and ``mm_bias`` / ``conv2d_bias`` (the layer's bias added in the
+kernel's epilogue).  ``repdl_amd.backend.hip`` serves these when the compiled binding
 (csrc/bind.cpp) has not been built; both call the same library.
 
 Each function validates its tensors (float32, on the GPU, made contiguous),
@@ -48,21 +49,43 @@ def _same_device(a: torch.Tensor, b: torch.Tensor) -> None:
         raise RuntimeError("tensors are on different devices: %s and %s" % (a.device, b.device))
 
 
+def _bias(bias, like: torch.Tensor, channels: int):
+    """The bias of a layer as a pointer: [channels] on the same device, or None."""
+    if bias is None:
+        return None, None
+    b = _check(bias, "bias", 1)
+    _same_device(b, like)
+    if b.shape[0] != channels:
+        raise RuntimeError("bias has %d elements for %d output channels" % (b.shape[0], channels))
+    return b, _ptr(b)
+
+
 def mm(input: torch.Tensor, mat2: torch.Tensor, transA: bool, transB: bool) -> torch.Tensor:
+    return mm_bias(input, mat2, None, transA, transB)
+
+
+def mm_bias(input: torch.Tensor, mat2: torch.Tensor, bias, transA: bool, transB: bool) -> torch.Tensor:
+    """mm followed by ``+= bias`` (repdl/nn/linear.py:21-22), the addition made in the kernel's epilogue."""
     a, b = _check(input, "input", 2), _check(mat2, "mat2", 2)
     _same_device(a, b)
     M, K = (a.shape[0], a.shape[1]) if not transA else (a.shape[1], a.shape[0])
     N, Kb = (b.shape[1], b.shape[0]) if not transB else (b.shape[0], b.shape[1])
     if K != Kb:
         raise RuntimeError("mm: inner dimensions differ (%d vs %d)" % (K, Kb))
+    hold, bp = _bias(bias, a, N)
     out = torch.empty((M, N), dtype=torch.float32, device=a.device)
     with torch.cuda.device(a.device):
-        _lib.call("repdl_hip_mm", _ptr(a), _ptr(b), _ptr(out), M, N, K, int(bool(transA)), int(bool(transB)),
+        _lib.call("repdl_hip_mm_bias", _ptr(a), _ptr(b), bp, _ptr(out), M, N, K, int(bool(transA)), int(bool(transB)),
                   _stream(a))
     return out
 
 
 def conv2d(input, kernel, strideH, strideW, paddingH, paddingW, groups) -> torch.Tensor:
+    return conv2d_bias(input, kernel, None, strideH, strideW, paddingH, paddingW, groups)
+
+
+def conv2d_bias(input, kernel, bias, strideH, strideW, paddingH, paddingW, groups) -> torch.Tensor:
+    """conv2d followed by ``+= bias`` per output channel (repdl/nn/conv.py:27-28), in the epilogue."""
     x, k = _check(input, "input", 4), _check(kernel, "kernel", 4)
     _same_device(x, k)
     N, IC, H, W = x.shape
@@ -72,9 +95,10 @@ def conv2d(input, kernel, strideH, strideW, paddingH, paddingW, groups) -> torch
     if H + 2 * paddingH < KH or W + 2 * paddingW < KW:
         raise RuntimeError("conv2d: kernel larger than padded input")
     OH, OW = (H + 2 * paddingH - KH) // strideH + 1, (W + 2 * paddingW - KW) // strideW + 1
+    hold, bp = _bias(bias, x, OC)
     out = torch.empty((N, OC, OH, OW), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
-        _lib.call("repdl_hip_conv2d", _ptr(x), _ptr(k), _ptr(out), N, IC, H, W, OC, KH, KW, strideH, strideW,
+        _lib.call("repdl_hip_conv2d_bias", _ptr(x), _ptr(k), bp, _ptr(out), N, IC, H, W, OC, KH, KW, strideH, strideW,
                   paddingH, paddingW, groups, _stream(x))
     return out
 

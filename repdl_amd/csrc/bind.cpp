@@ -2,7 +2,8 @@
 // (backend/cuda/bind.cpp:6-19): a PyTorch C++ extension module that exports the same ten
 // functions with the same positional signatures (matrix_multiplication.cu:234-235, 267;
 // convolution.cu:153-155, 259-262, 359-362, 385-387; summation.cu:149-155;
-// softmax.cpp:15, 28; cross_entropy.cpp:15, 31), plus exp / log / sqrt / div / div_scalar.
+// softmax.cpp:15, 28; cross_entropy.cpp:15, 31), plus exp / log / sqrt / div / div_scalar and
+// mm_bias / conv2d_bias (the layer's bias added in the kernel's epilogue).
 // It is the only file of this library that knows about PyTorch: every function checks its
 // tensors, allocates the output on the input's device, and hands raw pointers and the current
 // stream to the C ABI of include/repdl_hip.h.  Host C++ only; built with the host compiler
@@ -41,7 +42,24 @@ void same_device(const torch::Tensor &a, const torch::Tensor &b)
 void ok(int rc, const char *what) { TORCH_CHECK(rc == 0, what, " failed with code ", rc, ": ", repdl_hip_error_string(rc)); }
 } // namespace
 
-torch::Tensor mm(const torch::Tensor &input, const torch::Tensor &mat2, bool transA, bool transB)
+namespace
+{
+// the bias of a layer: [channels] on the same device, or none
+const float *bias_pointer(const c10::optional<torch::Tensor> &bias, torch::Tensor &hold, const torch::Tensor &like,
+                          int64_t channels)
+{
+    if (!bias.has_value())
+        return nullptr;
+    hold = checked(*bias, "bias", 1);
+    same_device(hold, like);
+    TORCH_CHECK(hold.size(0) == channels, "bias has ", hold.size(0), " elements for ", channels, " output channels");
+    return hold.data_ptr<float>();
+}
+} // namespace
+
+// mm followed by `+= bias` (repdl/nn/linear.py:21-22) with the addition in the kernel's epilogue
+torch::Tensor mm_bias(const torch::Tensor &input, const torch::Tensor &mat2, const c10::optional<torch::Tensor> &bias,
+                      bool transA, bool transB)
 {
     const auto a = checked(input, "input", 2), b = checked(mat2, "mat2", 2);
     same_device(a, b);
@@ -49,15 +67,23 @@ torch::Tensor mm(const torch::Tensor &input, const torch::Tensor &mat2, bool tra
     const int64_t N = !transB ? b.size(1) : b.size(0), Kb = !transB ? b.size(0) : b.size(1);
     TORCH_CHECK(K == Kb, "mm: inner dimensions differ (", K, " vs ", Kb, ")");
     const DeviceGuard guard(a.device());
+    torch::Tensor hold;
+    const float *bp = bias_pointer(bias, hold, a, N);
     auto out = torch::empty({M, N}, a.options());
-    ok(repdl_hip_mm(a.data_ptr<float>(), b.data_ptr<float>(), out.data_ptr<float>(), M, N, K, transA, transB,
-                    current_stream()),
+    ok(repdl_hip_mm_bias(a.data_ptr<float>(), b.data_ptr<float>(), bp, out.data_ptr<float>(), M, N, K, transA, transB,
+                         current_stream()),
        "repdl_hip_mm");
     return out;
 }
 
-torch::Tensor conv2d(const torch::Tensor &input, const torch::Tensor &kernel, int64_t sH, int64_t sW, int64_t pH,
-                     int64_t pW, int64_t groups)
+torch::Tensor mm(const torch::Tensor &input, const torch::Tensor &mat2, bool transA, bool transB)
+{
+    return mm_bias(input, mat2, c10::nullopt, transA, transB);
+}
+
+// conv2d followed by `+= bias` per output channel (repdl/nn/conv.py:27-28), the addition in the epilogue
+torch::Tensor conv2d_bias(const torch::Tensor &input, const torch::Tensor &kernel, const c10::optional<torch::Tensor> &bias,
+                          int64_t sH, int64_t sW, int64_t pH, int64_t pW, int64_t groups)
 {
     const auto x = checked(input, "input", 4), k = checked(kernel, "kernel", 4);
     same_device(x, k);
@@ -69,11 +95,19 @@ torch::Tensor conv2d(const torch::Tensor &input, const torch::Tensor &kernel, in
     TORCH_CHECK(H + 2 * pH >= KH && W + 2 * pW >= KW, "conv2d: kernel larger than padded input");
     const int64_t OH = (H + 2 * pH - KH) / sH + 1, OW = (W + 2 * pW - KW) / sW + 1;
     const DeviceGuard guard(x.device());
+    torch::Tensor hold;
+    const float *bp = bias_pointer(bias, hold, x, OC);
     auto out = torch::empty({N, OC, OH, OW}, x.options());
-    ok(repdl_hip_conv2d(x.data_ptr<float>(), k.data_ptr<float>(), out.data_ptr<float>(), N, IC, H, W, OC, KH, KW, sH,
-                        sW, pH, pW, groups, current_stream()),
+    ok(repdl_hip_conv2d_bias(x.data_ptr<float>(), k.data_ptr<float>(), bp, out.data_ptr<float>(), N, IC, H, W, OC, KH, KW,
+                             sH, sW, pH, pW, groups, current_stream()),
        "repdl_hip_conv2d");
     return out;
+}
+
+torch::Tensor conv2d(const torch::Tensor &input, const torch::Tensor &kernel, int64_t sH, int64_t sW, int64_t pH,
+                     int64_t pW, int64_t groups)
+{
+    return conv2d_bias(input, kernel, c10::nullopt, sH, sW, pH, pW, groups);
 }
 
 torch::Tensor conv2d_grad_input(const torch::Tensor &grad_output, const torch::Tensor &kernel, int64_t H, int64_t W,
@@ -243,4 +277,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("sqrt", &h::sqrt);
     m.def("div", &h::div);
     m.def("div_scalar", &h::div_scalar);
+    m.def("mm_bias", &h::mm_bias);
+    m.def("conv2d_bias", &h::conv2d_bias);
 }

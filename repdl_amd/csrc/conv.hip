@@ -27,7 +27,11 @@ namespace
 struct ConvDims
 {
     int N, IC, H, W, OC, KH, KW, OH, OW, sH, sW, pH, pW, groups;
+    const float *bias; // forward only: [OC], added once to each output after its chain; null = none
 };
+
+// repdl/nn/conv.py:27-28: the bias is one rounded addition to the finished chain
+__device__ __forceinline__ float with_bias(float v, const ConvDims &d, int oc) { return d.bias != nullptr ? v + d.bias[oc] : v; }
 
 // ---------------------------------------------------------------------------
 // The literal chains (exact by construction).
@@ -331,6 +335,15 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_kernel(const float *__restri
     const int g = MODE == MODE_FWD ? blockIdx.z % d.groups : 0;
     const int m0 = blockIdx.y * BM, p0 = blockIdx.x * BN;
 
+    // forward with a bias: the values of this tile's rows, read from LDS in the epilogue
+    __shared__ float bias_s[BM];
+    if (MODE == MODE_FWD && d.bias != nullptr)
+    {
+        if (tid < BM)
+            bias_s[tid] = m0 + tid < M ? d.bias[g * OCg + m0 + tid] : 0.0f;
+        __syncthreads();
+    }
+
     KStep kstep;
     kstep.dc = BK / KHW;
     kstep.dkh = (BK % KHW) / d.KW;
@@ -596,6 +609,8 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_kernel(const float *__restri
                         v = MODE == MODE_FWD ? conv2d_exact(Xg, Wt, d, n, ch, ph, pw)
                                              : conv2d_grad_input_exact(Xg, Wt, d, n, ch, ph, pw);
                     }
+                    if (MODE == MODE_FWD && d.bias != nullptr)
+                        v = v + bias_s[m - m0];
                     Oimg[(int64_t)ch * P + pix] = v;
                 }
             }
@@ -685,6 +700,8 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_kernel(const float *__restri
                         v[j] = MODE == MODE_FWD ? conv2d_exact(Xg, Wt, d, n, ch, ph, pw)
                                                 : conv2d_grad_input_exact(Xg, Wt, d, n, ch, ph, pw);
                     }
+                    if (MODE == MODE_FWD && d.bias != nullptr)
+                        v[j] = v[j] + bias_s[m - m0];
                 }
                 float *p = Oimg + (int64_t)ch * P + pix;
                 if (ovec && pix + 3 < P)
@@ -919,12 +936,20 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
                 acc[i][j][r] = 0.0f;
     const int a_off = half * LDA + wm * 64 + l32, b_off = half * LDBF + wn * (32 * PB) + l32;
 
+    // forward with a bias: the values of this tile's rows go to LDS behind the first tiles (the
+    // barrier that publishes those publishes them) and are read back in the epilogue
+    __shared__ float bias_s[BM];
+    const bool has_bias = MODE == MODE_FWD && d.bias != nullptr;
+    float bias_r = 0.0f;
     const int nkt = K / BK;
     if (nkt > 0)
-    {
         load_tiles(0);
+    if (has_bias && tid < BM && m0 + tid < M)
+        bias_r = d.bias[g * OCg + m0 + tid];
+    if (nkt > 0)
         store_tiles(0);
-    }
+    if (has_bias && tid < BM)
+        bias_s[tid] = bias_r;
     __syncthreads();
     for (int kt = 0; kt < nkt; kt++)
     {
@@ -981,6 +1006,8 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
                     v = MODE == MODE_FWD ? conv2d_exact(Xg, Wt, d, n, ch, ph, pw)
                                          : conv2d_grad_input_exact(Xg, Wt, d, n, ch, ph, pw);
                 }
+                if (has_bias)
+                    v = v + bias_s[m - m0];
                 Oimg[(int64_t)ch * P + pix] = v;
             }
         }
@@ -1919,7 +1946,7 @@ __global__ __launch_bounds__(256) void conv_mm_out_kernel(const float *__restric
         const int ph = p / PW, pw = p - ph * PW;
         v = MODE == MODE_FWD ? conv2d_exact(Xg, Wt, d, (int)n, ch, ph, pw) : conv2d_grad_input_exact(Xg, Wt, d, (int)n, ch, ph, pw);
     }
-    Out[idx] = v;
+    Out[idx] = MODE == MODE_FWD ? with_bias(v, d, ch) : v;
 }
 
 // Small images, many channels, one group, the matrix path on: see above.  (Measured at batch 64:
@@ -1984,6 +2011,14 @@ REPDL_API int repdl_hip_conv2d(const float *input, const float *kernel, float *o
                                int64_t sH, int64_t sW, int64_t pH, int64_t pW, int64_t groups,
                                void *stream)
 {
+    return repdl_hip_conv2d_bias(input, kernel, nullptr, output, N, IC, H, W, OC, KH, KW, sH, sW, pH, pW, groups, stream);
+}
+
+REPDL_API int repdl_hip_conv2d_bias(const float *input, const float *kernel, const float *bias, float *output,
+                                    int64_t N, int64_t IC, int64_t H, int64_t W, int64_t OC, int64_t KH,
+                                    int64_t KW, int64_t sH, int64_t sW, int64_t pH, int64_t pW, int64_t groups,
+                                    void *stream)
+{
     REPDL_REQUIRE(N >= 0 && IC >= 0 && H >= 0 && W >= 0 && OC >= 0 && KH > 0 && KW > 0);
     REPDL_REQUIRE(sH > 0 && sW > 0 && pH >= 0 && pW >= 0 && groups > 0);
     REPDL_REQUIRE(IC % groups == 0 && OC % groups == 0);
@@ -1996,7 +2031,7 @@ REPDL_API int repdl_hip_conv2d(const float *input, const float *kernel, float *o
     REPDL_REQUIRE(fits_i32(H * W) && fits_i32(OH * OW) && fits_i32(IC * KH * KW) && fits_i32(N) && fits_i32(OC));
     REPDL_REQUIRE(fits_i32(OH * sH + KH + pH) && fits_i32(OW * sW + KW + pW));
     ConvDims d{(int)N, (int)IC, (int)H, (int)W, (int)OC, (int)KH, (int)KW, (int)OH,
-               (int)OW, (int)sH, (int)sW, (int)pH, (int)pW, (int)groups};
+               (int)OW, (int)sH, (int)sW, (int)pH, (int)pW, (int)groups, bias};
     if (conv_prefers_mm(d, OC, IC * KH * KW, OH * OW))
         return launch_conv_mm<MODE_FWD>(input, kernel, output, d, stream);
     return launch_conv_gemm<MODE_FWD>(input, kernel, output, d, stream);

@@ -135,8 +135,9 @@ __device__ __forceinline__ void fma_step(const float *__restrict__ As, const flo
 template <bool TA, bool TB>
 __global__ __launch_bounds__(NT) void mm_kernel(const float *__restrict__ A,
                                                 const float *__restrict__ B, float *__restrict__ C,
-                                                int64_t M, int64_t N, int64_t K, int avec, int bvec,
-                                                int cvec, int64_t gx, int64_t gy, int64_t ntiles8)
+                                                const float *__restrict__ bias, int64_t M, int64_t N,
+                                                int64_t K, int avec, int bvec, int cvec, int64_t gx, int64_t gy,
+                                                int64_t ntiles8)
 {
     constexpr bool A_KC = !TA; // A[m*K + k]
     constexpr bool B_KC = TB;  // B[n*K + k]
@@ -219,15 +220,22 @@ __global__ __launch_bounds__(NT) void mm_kernel(const float *__restrict__ A,
         {
             int64_t n = n0 + tx * 4 + jh * 64;
             float *p = C + m * N + n;
+            float v[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+            {
+                v[j] = acc[i][jh * 4 + j];
+                if (bias != nullptr && n + j < N)
+                    v[j] = v[j] + bias[n + j]; // one rounded add after the chain
+            }
             if (cvec && n + 3 < N)
-                *reinterpret_cast<float4 *>(p) =
-                    make_float4(acc[i][jh * 4 + 0], acc[i][jh * 4 + 1], acc[i][jh * 4 + 2], acc[i][jh * 4 + 3]);
+                *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
             else
             {
 #pragma unroll
                 for (int j = 0; j < 4; j++)
                     if (n + j < N)
-                        p[j] = acc[i][jh * 4 + j];
+                        p[j] = v[j];
             }
         }
     }
@@ -332,9 +340,9 @@ __device__ __forceinline__ void store_tile_pad(float *__restrict__ S, int tid, c
 
 template <bool TA, bool TB, int FM, int FN, int WGM, int WGN>
 __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_kernel(const float *__restrict__ A, const float *__restrict__ B,
-                                                                float *__restrict__ C, int64_t M, int64_t N, int64_t K,
-                                                                int avec, int bvec, int64_t gx, int64_t gy,
-                                                                int64_t ntiles8)
+                                                                float *__restrict__ C, const float *__restrict__ bias,
+                                                                int64_t M, int64_t N, int64_t K, int avec, int bvec,
+                                                                int64_t gx, int64_t gy, int64_t ntiles8)
 {
     constexpr int NTH = 64 * WGM * WGN;
     constexpr int TM = 32 * FM * WGM, TN = 32 * FN * WGN;
@@ -438,7 +446,7 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_kernel(const float *__r
             {
                 const int64_t n = n0 + wn * 32 * FN + 32 * j + l32;
                 if (n < N)
-                    C[m * N + n] = acc[i][j][r];
+                    C[m * N + n] = bias != nullptr ? acc[i][j][r] + bias[n] : acc[i][j][r];
             }
         }
 }
@@ -452,8 +460,10 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_kernel(const float *__r
 template <bool TA, bool TB, int FM, int FN, int WGM, int WGN, bool EDGE>
 __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_fast_kernel(const float *__restrict__ A,
                                                                      const float *__restrict__ B,
-                                                                     float *__restrict__ C, int64_t M, int64_t N,
-                                                                     int64_t K, int64_t gx, int64_t gy, int64_t ntiles8)
+                                                                     float *__restrict__ C,
+                                                                     const float *__restrict__ bias, int64_t M,
+                                                                     int64_t N, int64_t K, int64_t gx, int64_t gy,
+                                                                     int64_t ntiles8)
 {
     constexpr int NTH = 64 * WGM * WGN;
     constexpr int TM = 32 * FM * WGM, TN = 32 * FN * WGN;
@@ -713,6 +723,14 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_fast_kernel(const float
         __syncthreads();
     }
 
+    // bias: one rounded add per output after its chain; a lane owns FN columns
+    float bv[FN];
+#pragma unroll
+    for (int j = 0; j < FN; j++)
+    {
+        const int64_t nn = n0 + wn * 32 * FN + 32 * j + l32;
+        bv[j] = bias != nullptr && (!EDGE || nn < N) ? bias[nn] : 0.0f;
+    }
 #pragma unroll
     for (int i = 0; i < FM; i++)
 #pragma unroll
@@ -726,14 +744,14 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_fast_kernel(const float
             {
                 const int64_t nn = n0 + wn * 32 * FN + 32 * j + l32;
                 if (!EDGE || nn < N)
-                    __builtin_nontemporal_store(acc[i][j][r], &C[m * N + nn]);
+                    __builtin_nontemporal_store(bias != nullptr ? acc[i][j][r] + bv[j] : acc[i][j][r], &C[m * N + nn]);
             }
         }
 }
 
 template <bool TA, bool TB, int FM, int FN, int WGM, int WGN>
-int launch_mfma_t(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int avec, int bvec,
-                  hipStream_t s)
+int launch_mfma_t(const float *A, const float *B, float *C, const float *bias, int64_t M, int64_t N, int64_t K, int avec,
+                  int bvec, hipStream_t s)
 {
     constexpr int TM = 32 * FM * WGM, TN = 32 * FN * WGN;
     constexpr size_t shmem = (size_t)2 * BK * (TM + 4 + TN + 4) * sizeof(float);
@@ -759,7 +777,7 @@ int launch_mfma_t(const float *A, const float *B, float *C, int64_t M, int64_t N
             if (e != hipSuccess)
                 return (int)e;
         }
-        hipLaunchKernelGGL(kern, dim3((unsigned)(gx * gy)), dim3(64 * WGM * WGN), shmem, s, A, B, C, M, N, K, gx, gy,
+        hipLaunchKernelGGL(kern, dim3((unsigned)(gx * gy)), dim3(64 * WGM * WGN), shmem, s, A, B, C, bias, M, N, K, gx, gy,
                            ntiles8);
         return repdl_launch_status();
     }
@@ -771,22 +789,22 @@ int launch_mfma_t(const float *A, const float *B, float *C, int64_t M, int64_t N
         if (e != hipSuccess)
             return (int)e;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)(gx * gy)), dim3(64 * WGM * WGN), shmem, s, A, B, C, M, N, K, avec, bvec, gx, gy,
-                       ntiles8);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(gx * gy)), dim3(64 * WGM * WGN), shmem, s, A, B, C, bias, M, N, K, avec, bvec,
+                       gx, gy, ntiles8);
     return repdl_launch_status();
 }
 
 template <int FM, int FN, int WGM, int WGN>
-int launch_mfma(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K, int transA, int transB,
-                int avec, int bvec, hipStream_t s)
+int launch_mfma(const float *A, const float *B, float *C, const float *bias, int64_t M, int64_t N, int64_t K, int transA,
+                int transB, int avec, int bvec, hipStream_t s)
 {
     if (!transA && !transB)
-        return launch_mfma_t<false, false, FM, FN, WGM, WGN>(A, B, C, M, N, K, avec, bvec, s);
+        return launch_mfma_t<false, false, FM, FN, WGM, WGN>(A, B, C, bias, M, N, K, avec, bvec, s);
     if (transA && !transB)
-        return launch_mfma_t<true, false, FM, FN, WGM, WGN>(A, B, C, M, N, K, avec, bvec, s);
+        return launch_mfma_t<true, false, FM, FN, WGM, WGN>(A, B, C, bias, M, N, K, avec, bvec, s);
     if (!transA && transB)
-        return launch_mfma_t<false, true, FM, FN, WGM, WGN>(A, B, C, M, N, K, avec, bvec, s);
-    return launch_mfma_t<true, true, FM, FN, WGM, WGN>(A, B, C, M, N, K, avec, bvec, s);
+        return launch_mfma_t<false, true, FM, FN, WGM, WGN>(A, B, C, bias, M, N, K, avec, bvec, s);
+    return launch_mfma_t<true, true, FM, FN, WGM, WGN>(A, B, C, bias, M, N, K, avec, bvec, s);
 }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -794,6 +812,12 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 REPDL_API int repdl_hip_mm(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K,
                            int transA, int transB, void *stream)
+{
+    return repdl_hip_mm_bias(A, B, nullptr, C, M, N, K, transA, transB, stream);
+}
+
+REPDL_API int repdl_hip_mm_bias(const float *A, const float *B, const float *bias, float *C, int64_t M, int64_t N,
+                                int64_t K, int transA, int transB, void *stream)
 {
     REPDL_REQUIRE(M >= 0 && N >= 0 && K >= 0);
     if (M == 0 || N == 0)
@@ -816,11 +840,11 @@ REPDL_API int repdl_hip_mm(const float *A, const float *B, float *C, int64_t M, 
         switch (cfg)
         {
         case 0:
-            return launch_mfma<1, 1, 2, 2>(A, B, C, M, N, K, transA, transB, avec, bvec, s);
+            return launch_mfma<1, 1, 2, 2>(A, B, C, bias, M, N, K, transA, transB, avec, bvec, s);
         case 1:
-            return launch_mfma<2, 2, 2, 2>(A, B, C, M, N, K, transA, transB, avec, bvec, s);
+            return launch_mfma<2, 2, 2, 2>(A, B, C, bias, M, N, K, transA, transB, avec, bvec, s);
         default:
-            return launch_mfma<4, 2, 2, 4>(A, B, C, M, N, K, transA, transB, avec, bvec, s);
+            return launch_mfma<4, 2, 2, 4>(A, B, C, bias, M, N, K, transA, transB, avec, bvec, s);
         }
     }
     const int64_t gx = repdl_cdiv(N, BN), gy = repdl_cdiv(M, BM);
@@ -829,12 +853,16 @@ REPDL_API int repdl_hip_mm(const float *A, const float *B, float *C, int64_t M, 
     const int cvec = aligned16(C) && (N % 4 == 0);
     dim3 grid((unsigned)(gx * gy)), block(NT);
     if (!transA && !transB)
-        hipLaunchKernelGGL((mm_kernel<false, false>), grid, block, 0, s, A, B, C, M, N, K, avec, bvec, cvec, gx, gy, ntiles8);
+        hipLaunchKernelGGL((mm_kernel<false, false>), grid, block, 0, s, A, B, C, bias, M, N, K, avec, bvec, cvec, gx, gy,
+                           ntiles8);
     else if (transA && !transB)
-        hipLaunchKernelGGL((mm_kernel<true, false>), grid, block, 0, s, A, B, C, M, N, K, avec, bvec, cvec, gx, gy, ntiles8);
+        hipLaunchKernelGGL((mm_kernel<true, false>), grid, block, 0, s, A, B, C, bias, M, N, K, avec, bvec, cvec, gx, gy,
+                           ntiles8);
     else if (!transA && transB)
-        hipLaunchKernelGGL((mm_kernel<false, true>), grid, block, 0, s, A, B, C, M, N, K, avec, bvec, cvec, gx, gy, ntiles8);
+        hipLaunchKernelGGL((mm_kernel<false, true>), grid, block, 0, s, A, B, C, bias, M, N, K, avec, bvec, cvec, gx, gy,
+                           ntiles8);
     else
-        hipLaunchKernelGGL((mm_kernel<true, true>), grid, block, 0, s, A, B, C, M, N, K, avec, bvec, cvec, gx, gy, ntiles8);
+        hipLaunchKernelGGL((mm_kernel<true, true>), grid, block, 0, s, A, B, C, bias, M, N, K, avec, bvec, cvec, gx, gy,
+                           ntiles8);
     return repdl_launch_status();
 }

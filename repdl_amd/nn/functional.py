@@ -21,10 +21,7 @@ class _Linear(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, bias):
         ctx.save_for_backward(x, weight)
-        y = ops.mm(x, weight, transB=True)  # x [B,in] . W[out,in]^T
-        if bias is not None:
-            y += bias
-        return y
+        return ops.mm_bias(x, weight, bias, transB=True)  # x [B,in] . W[out,in]^T, then + bias
 
     @staticmethod
     def backward(ctx, gy):
@@ -82,10 +79,7 @@ class _Conv2d(torch.autograd.Function):
     def forward(ctx, x, weight, bias, stride, padding, groups):
         ctx.save_for_backward(x, weight)
         ctx.conf = (stride, padding, groups)
-        y = ops.conv2d(x, weight, stride=stride, padding=padding, groups=groups)
-        if bias is not None:
-            y += bias.unsqueeze(-1).unsqueeze(-1)
-        return y
+        return ops.conv2d_bias(x, weight, bias, stride=stride, padding=padding, groups=groups)
 
     @staticmethod
     def backward(ctx, gy):

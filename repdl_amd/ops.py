@@ -12,7 +12,7 @@ added as public operators.
 """
 from __future__ import annotations
 
-from typing import Sequence, Union
+from typing import Optional, Sequence, Union
 
 import torch
 
@@ -32,11 +32,28 @@ def mm(input: torch.Tensor, mat2: torch.Tensor, transA: bool = False, transB: bo
     return _backend(input).mm(input, mat2, transA, transB)
 
 
+def mm_bias(input: torch.Tensor, mat2: torch.Tensor, bias: Optional[torch.Tensor], transA: bool = False,
+            transB: bool = False) -> torch.Tensor:
+    """``mm(...)`` followed by ``+= bias`` over the rows (the reference's linear layer,
+    nn/linear.py:21-22), the one rounded addition made where the chain ends instead of in a
+    second pass.  Not in the reference's ``ops``."""
+    return _backend(input).mm_bias(input, mat2, bias, transA, transB)
+
+
 def conv2d(input: torch.Tensor, weight: torch.Tensor, stride: Sequence[int], padding: Sequence[int],
            groups: int) -> torch.Tensor:
     sh, sw = stride
     ph, pw = padding
     return _backend(input).conv2d(input, weight, sh, sw, ph, pw, groups)
+
+
+def conv2d_bias(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], stride: Sequence[int],
+                padding: Sequence[int], groups: int) -> torch.Tensor:
+    """``conv2d(...)`` followed by ``+= bias`` per output channel (nn/conv.py:27-28), the
+    addition made in the kernel's epilogue.  Not in the reference's ``ops``."""
+    sh, sw = stride
+    ph, pw = padding
+    return _backend(input).conv2d_bias(input, weight, bias, sh, sw, ph, pw, groups)
 
 
 def conv2d_grad_input(input_shape: Sequence[int], weight: torch.Tensor, grad_output: torch.Tensor,

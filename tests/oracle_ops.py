@@ -31,6 +31,20 @@ class _OracleBackend:
     sqrt = staticmethod(oracle.sqrt)
 
     @staticmethod
+    def mm_bias(input, mat2, bias, transA, transB):
+        y = oracle.mm(input, mat2, transA, transB)  # repdl/nn/linear.py:21-22
+        if bias is not None:
+            y += bias
+        return y
+
+    @staticmethod
+    def conv2d_bias(input, kernel, bias, sH, sW, pH, pW, groups):
+        y = oracle.conv2d(input, kernel, sH, sW, pH, pW, groups)  # repdl/nn/conv.py:27-28
+        if bias is not None:
+            y += bias.unsqueeze(-1).unsqueeze(-1)
+        return y
+
+    @staticmethod
     def div(a, b):
         shape = torch.broadcast_shapes(a.shape, b.shape)
         return oracle.div(a.expand(shape).contiguous(), b.expand(shape).contiguous())

@@ -87,6 +87,25 @@ def test_forward(shape, special):
     assert _same(got, oracle.conv2d(x, w, sH, sW, pH, pW, g))
 
 
+@pytest.mark.parametrize("special", KINDS, ids=KIND_IDS)
+@pytest.mark.parametrize("shape", FWD, ids=[str(s) for s in FWD])
+def test_forward_with_bias(shape, special):
+    """conv2d_bias = conv2d followed by one rounded `+= bias` per channel (repdl/nn/conv.py:27-28)
+    on every forward kernel; zero results that are recomputed with the literal chain get their
+    bias after the recomputation (the sign of a zero sum decides -0 + -0 against +0 + -0)."""
+    from repdl_amd import ops
+
+    N, IC, H, W, OC, KH, KW, sH, sW, pH, pW, g = shape
+    x, w = _data(shape, 150, special)
+    bias = gen.scaled_normal(151, OC, lo=-20, hi=10)
+    bias[::4] = -0.0
+    bias[1::9] = 0.0
+    want = oracle.conv2d(x, w, sH, sW, pH, pW, g)
+    want += bias.unsqueeze(-1).unsqueeze(-1)
+    got = ops.conv2d_bias(x.cuda(), w.cuda(), bias.cuda(), (sH, sW), (pH, pW), g).cpu()
+    assert _same(got, want)
+
+
 # grad-input with strides on the matrix path (IC a multiple of 64, OC*KH*KW of 16): grad_output is
 # dilated into the workspace; input rows and columns that no output reaches (remainders of the stride)
 DGRAD = [s for s in FWD if s[-1] == 1] + [

@@ -23,6 +23,29 @@ def test_layouts_and_edges(shape, tA, tB):
     assert torch.equal(got, oracle.mm(a, b, bool(tA), bool(tB)))
 
 
+@pytest.mark.parametrize("tA,tB", [(0, 1), (0, 0), (1, 0), (1, 1)])
+@pytest.mark.parametrize("shape", SHAPES + [(512, 768, 256), (300, 1000, 64)], ids=str)
+def test_bias_in_the_epilogue(shape, tA, tB):
+    """mm_bias = mm followed by one rounded `+= bias` (repdl/nn/linear.py:21-22), on every kernel
+    variant: whole tiles, edge tiles, the general kernel; bias values that cancel, dwarf and vanish
+    against the products, and signed zeros (-0 + +0 = +0, -0 + -0 = -0)."""
+    from repdl_amd import ops
+
+    M, N, K = shape
+    a = gen.scaled_normal(M * 5 + K, *((K, M) if tA else (M, K)), lo=-6, hi=6)
+    b = gen.normal_like(N * 11 + K, *((N, K) if tB else (K, N)))
+    bias = gen.scaled_normal(N + 1, N, lo=-30, hi=30)
+    bias[::5] = 0.0
+    bias[1::7] = -0.0
+    a[0] = 0.0  # a row of zero chains: the result is the bias with the zero's sign rules
+    want = oracle.mm(a, b, bool(tA), bool(tB))
+    want += bias
+    got = ops.mm_bias(a.cuda(), b.cuda(), bias.cuda(), bool(tA), bool(tB)).cpu()
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+    none = ops.mm_bias(a.cuda(), b.cuda(), None, bool(tA), bool(tB)).cpu()
+    assert torch.equal(none.view(torch.int32), oracle.mm(a, b, bool(tA), bool(tB)).view(torch.int32))
+
+
 def test_unaligned_operands():
     from repdl_amd import ops
 
