@@ -41,7 +41,11 @@ def test_shapes_and_elementwise():
                        ("sum1d", (x[:777], True)), ("sum2d_dim0", (m, False, True)), ("sum2d_dim0", (m, True, False)),
                        ("sum2d_dim1", (m, False, False)), ("sum2d_dim1", (m[:1], False, False)),
                        ("sum4d_dim023", (t4, True, True)), ("sum4d_dim023", (t4, False, False)), ("softmax", (m,)),
-                       ("cross_entropy", (m, gen.labels(7, 33, 47).cuda()))]:
+                       ("cross_entropy", (m, gen.labels(7, 33, 47).cuda())),
+                       ("mm_bias", (m, gen.normal_like(8, 21, 47).cuda(), gen.normal_like(9, 21).cuda(), False, True)),
+                       ("mm_bias", (m, gen.normal_like(8, 21, 47).cuda(), None, False, True)),
+                       ("conv2d_bias", (t4, gen.normal_like(10, 4, 5, 3, 3).cuda(), gen.normal_like(11, 4).cuda(), 1, 2, 1, 0, 1)),
+                       ("conv2d_bias", (t4, gen.normal_like(10, 4, 5, 3, 3).cuda(), None, 1, 2, 1, 0, 1))]:
         a, b = getattr(ext, name)(*args), getattr(ct, name)(*args)
         assert a.shape == b.shape, name
         assert torch.equal(a.view(torch.int32), b.view(torch.int32)), name
@@ -59,3 +63,10 @@ def test_errors():
         ext.mm(x.cuda(), torch.ones(5, 4).cuda(), False, False)  # inner dimensions differ
     with pytest.raises(RuntimeError):
         ext.conv2d(torch.ones(1, 3, 8, 8).cuda(), torch.ones(4, 2, 3, 3).cuda(), 1, 1, 1, 1, 2)
+    from repdl_amd.backend import hip_ctypes as ct
+
+    for mod in (ext, ct):
+        with pytest.raises(RuntimeError):
+            mod.mm_bias(x.cuda(), x.cuda(), torch.ones(5).cuda(), False, False)  # bias length
+        with pytest.raises(RuntimeError):
+            mod.conv2d_bias(torch.ones(1, 3, 8, 8).cuda(), torch.ones(4, 3, 3, 3).cuda(), torch.ones(4), 1, 1, 1, 1, 1)  # bias on the CPU
