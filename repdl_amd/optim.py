@@ -82,7 +82,9 @@ class Adam(torch.optim.Adam):
                     if amsgrad:
                         state["max_exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
                 state["step"] += 1
-                t = state["step"]
+                # an integer whatever holds the count: after load_state_dict PyTorch keeps it as a float32
+                # tensor, and beta ** tensor would compute the bias corrections in binary32
+                t = int(state["step"])
                 g = p.grad
                 m, v = state["exp_avg"], state["exp_avg_sq"]
                 vmax = state["max_exp_avg_sq"] if amsgrad else None

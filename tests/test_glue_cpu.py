@@ -161,3 +161,22 @@ def test_adam_matches_formula():
         pt.grad = g.clone()
         torch.optim.Adam([pt], lr=0.01).step()
         assert torch.allclose(p.detach(), pt.detach(), atol=1e-6)
+
+
+@pytest.mark.parametrize("amsgrad", [False, True])
+def test_adam_resumes_from_a_state_dict_with_the_same_bits(amsgrad):
+    """Four steps in a row == two steps, state_dict() -> load_state_dict() into a fresh optimizer,
+    two more.  (load_state_dict turns the step count into a float32 tensor; the bias corrections
+    must still be the binary64 values of an integer count.)"""
+    x, y = models.images(71, 16), gen.labels(72, 16, 10)
+    make = lambda m: repdl_amd.optim.Adam(m.parameters(), 0.01, weight_decay=0.01, amsgrad=amsgrad)
+    with oracle_for_cpu_tensors():
+        m1 = repdl_amd.from_torch_module(models.cnn(3))
+        models.train_steps(m1, repdl_amd.nn.CrossEntropyLoss(), make(m1), x, y, 4)
+        m2 = repdl_amd.from_torch_module(models.cnn(3))
+        o2 = make(m2)
+        models.train_steps(m2, repdl_amd.nn.CrossEntropyLoss(), o2, x, y, 2)
+        o3 = make(m2)
+        o3.load_state_dict(o2.state_dict())
+        models.train_steps(m2, repdl_amd.nn.CrossEntropyLoss(), o3, x, y, 2)
+    assert repdl_amd.utils.get_hash(m1) == repdl_amd.utils.get_hash(m2)

@@ -148,3 +148,19 @@ def test_optimizer_classes_fused_equals_sequence(optim):
             repdl_amd.optim.FUSED = True
 
     assert run(True) == run(False)
+
+
+def test_adam_resumes_from_a_state_dict_with_the_same_bits():
+    """Four steps in a row == two steps, state_dict() -> load_state_dict() into a fresh optimizer, two
+    more, with the fused kernels (load_state_dict leaves the step count as a float32 tensor)."""
+    x, y = models.images(41, 16).cuda(), gen.labels(42, 16, 10).cuda()
+    make = lambda m: repdl_amd.optim.Adam(m.parameters(), 0.01, weight_decay=0.01, amsgrad=True)
+    m1 = repdl_amd.from_torch_module(models.cnn(3)).cuda()
+    models.train_steps(m1, repdl_amd.nn.CrossEntropyLoss(), make(m1), x, y, 4)
+    m2 = repdl_amd.from_torch_module(models.cnn(3)).cuda()
+    o2 = make(m2)
+    models.train_steps(m2, repdl_amd.nn.CrossEntropyLoss(), o2, x, y, 2)
+    o3 = make(m2)
+    o3.load_state_dict(o2.state_dict())
+    models.train_steps(m2, repdl_amd.nn.CrossEntropyLoss(), o3, x, y, 2)
+    assert repdl_amd.utils.get_hash(m1) == repdl_amd.utils.get_hash(m2)
