@@ -22,7 +22,7 @@
 // Row and channel sums take the parallel evaluation when the chains are at least this long and
 // at most REPDL_SUM_ROWS_MAX_PARALLEL in number (few long chains are bound by the latency of one
 // chain; many chains keep the memory system busy with one lane per chain).
-#define REPDL_SUM_ROWS_MIN_PARALLEL 65536
+#define REPDL_SUM_ROWS_MIN_PARALLEL 49152
 #define REPDL_SUM_ROWS_MAX_PARALLEL 512
 
 // Largest extent a kernel indexes with 32-bit arithmetic.

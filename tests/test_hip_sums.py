@@ -116,7 +116,7 @@ def test_channel_sums_unaligned_pointer(shape):
 
 def _long_rows():
     """Few, long chains: row sums and channel sums that take the parallel evaluation (chains of at
-    least 65536 elements, at most 512 of them), with the data that attacks it."""
+    least 49152 elements, at most 512 of them), with the data that attacks it."""
     r = _rng(12)
     L = 70_000
     rows = [
@@ -141,11 +141,15 @@ def test_row_sums_few_long_rows():
     assert torch.equal(torch.isnan(got), nan) and torch.equal(got[~nan].view(torch.int32), want[~nan].view(torch.int32))
     m2 = gen.scaled_normal(90, 5, 65537)  # a row length that is no multiple of 4: scalar loads
     assert torch.equal(ops.sum2d_dim1(m2.cuda()).cpu(), oracle.sum2d_dim1(m2))
+    for n in (49151, 49152, 49168):  # either side of the length at which rows change kernels
+        m4 = gen.uniform_pm1(92 + n, 3, n)
+        assert torch.equal(ops.sum2d_dim1(m4.cuda()).cpu(), oracle.sum2d_dim1(m4)), n
     m3 = gen.uniform_pm1(91, 300, 66000)
     assert torch.equal(ops.sum2d_dim1(m3.cuda(), average=True).cpu(), oracle.sum2d_dim1(m3, average=True))
 
 
-@pytest.mark.parametrize("shape", [(8, 5, 96, 96), (3, 4, 160, 144), (70, 3, 32, 32), (9, 2, 90, 90), (2, 64, 224, 224)])
+@pytest.mark.parametrize("shape", [(8, 5, 96, 96), (3, 4, 160, 144), (70, 3, 32, 32), (9, 2, 90, 90), (2, 64, 224, 224),
+                                   (64, 8, 28, 28), (48, 3, 32, 32), (47, 3, 32, 32)])
 def test_channel_sums_few_long_chains(shape):
     """Channel sums whose chains (N*H*W elements) are long and few: a segment per image; (9, 2, 90, 90)
     has segments that are no multiple of 16 and stays with the row-chain kernel."""
