@@ -103,7 +103,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--quick", action="store_true", help="headline only, no secondary operators, no full parity")
-    ap.add_argument("--only", default="", help="comma list of secondary ops to run (sum2d,sum1d,exp,log,sqrt,div,conv,adam)")
+    ap.add_argument("--only", default="", help="comma list of secondary ops to run (sum2d,sum1d,exp,log,sqrt,div,conv,linear,adam)")
     ap.add_argument("--size", type=int, default=8192, help="mm size (M=N=K); the metric is quoted at 8192")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 1 GiB elementwise copy kernel (torch.add(x, 0)), the known-size kernel "
@@ -315,6 +315,33 @@ def main() -> int:
                         "cpu_baseline": {"value": round(flop / dt / 1e9, 2), "unit": "GFLOP/s", "cores": oracle.threads(),
                                          "kind": "port", "sample": "the full layer"}})
                 del x_d, w_d, go_d
+
+        if want("linear"):
+            # the other Linear shapes of the metric's GEMM configuration: grad-input (NN, tall K) and
+            # grad-weight (TN, the batch dimension as K); parity on a slab of output rows
+            for (M, N, K, tA, what) in ((4096, 4096, 32768, 0, "NN, Linear grad-input shape"),
+                                         (4096, 4096, 65536, 1, "TN, Linear grad-weight shape (batch as K)")):
+                g = torch.Generator().manual_seed(11 + tA)
+                a_h = torch.randn((K, M) if tA else (M, K), generator=g)
+                b_h = (torch.rand(K, N, generator=g) * 2 - 1) * (1.0 / (K ** 0.5)) if not tA else torch.randn(K, N, generator=g)
+                a_d, b_d = a_h.to(dev), b_h.to(dev)
+                hold = {}
+                def f(): hold["y"] = ops.mm(a_d, b_d, bool(tA), False)
+                wall, ev_mean, ev_min = time_gpu(f, max(2, args.steps // 2), 1)
+                rows = 64
+                slab = a_h[:, :rows].contiguous() if tA else a_h[:rows]
+                dt, y_slab = cpu_time(lambda: (refmods[0].mm(slab, b_h, bool(tA), False) if refmods else oracle.mm(slab, b_h, bool(tA), False)))
+                flop = 2.0 * M * N * K
+                tf = flop / (ev_mean * 1e-3) / 1e12
+                result["also"].append({
+                    "op": "mm", "workload": "%dx%dx%d %s" % (M, N, K, what), "value": round(tf * 1e3, 1), "unit": "GFLOP/s",
+                    "ms_per_step": round(ev_mean, 4),
+                    "roofline": {"bound": "mfma", "achieved": round(tf, 3), "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                 "frac": round(tf / FP32_PEAK_TFLOPS, 4), "traffic": None},
+                    "parity": {"equal": torch.equal(y_slab, hold["y"][:rows].cpu()), "rows_checked": rows, "sha256_gpu": sha(hold["y"])},
+                    "cpu_baseline": {"value": round(2.0 * rows * N * K / dt / 1e9, 2), "unit": "GFLOP/s", "cores": oracle.threads(),
+                                     "kind": kind, "sample": "first %d of %d output rows" % (rows, M)}})
+                del a_d, b_d, a_h, b_h, hold
 
         if want("adam"):
             import ctypes
