@@ -830,22 +830,23 @@ REPDL_API int repdl_hip_mm_bias(const float *A, const float *B, const float *bia
     hipStream_t s = repdl_stream(stream);
     if (repdl_mfma_exact())
     {
-        // the largest tile that still gives every CU several workgroups
-        int cfg = 0;
-        const int64_t target = 2 * 256;
-        if (repdl_cdiv(M, 256) * repdl_cdiv(N, 256) >= target)
-            cfg = 3;
-        else if (repdl_cdiv(M, 128) * repdl_cdiv(N, 128) >= target)
-            cfg = 1;
-        switch (cfg)
-        {
-        case 0:
-            return launch_mfma<1, 1, 2, 2>(A, B, C, bias, M, N, K, transA, transB, avec, bvec, s);
-        case 1:
-            return launch_mfma<2, 2, 2, 2>(A, B, C, bias, M, N, K, transA, transB, avec, bvec, s);
-        default:
+        // Tile choice: tiles run in rounds over the 256 CUs (workgroups that share a CU share its
+        // matrix pipes), so a configuration costs rounds x tile area / efficiency.  Measured rates per CU
+        // relative to the 256x256 tile (135 TFLOP/s when every CU has one or more): 128x128 tiles 0.77
+        // with one per CU, 0.86 with two or three, 0.92 from four on; 64x64 tiles 0.8 up to three per
+        // CU, 0.52 in large launches (twice the operand traffic per flop).  A 4096x4096 output is 256
+        // tiles of 256x256, one per CU, at the full rate (4096x4096x32768: 8.77 -> 8.11 ms against
+        // 128x128 tiles).
+        auto rounds = [&](int64_t tm, int64_t tn) { return repdl_cdiv(repdl_cdiv(M, tm) * repdl_cdiv(N, tn), 256); };
+        const int64_t r256 = rounds(256, 256), r128 = rounds(128, 128), r64 = rounds(64, 64);
+        const double c256 = (double)r256 * 65536.0;
+        const double c128 = (double)r128 * 16384.0 / (r128 >= 4 ? 0.92 : r128 >= 2 ? 0.86 : 0.77);
+        const double c64 = (double)r64 * 4096.0 / (r64 <= 3 ? 0.8 : 0.52);
+        if (c256 <= c128 && c256 <= c64)
             return launch_mfma<4, 2, 2, 4>(A, B, C, bias, M, N, K, transA, transB, avec, bvec, s);
-        }
+        if (c128 <= c64)
+            return launch_mfma<2, 2, 2, 2>(A, B, C, bias, M, N, K, transA, transB, avec, bvec, s);
+        return launch_mfma<1, 1, 2, 2>(A, B, C, bias, M, N, K, transA, transB, avec, bvec, s);
     }
     const int64_t gx = repdl_cdiv(N, BN), gy = repdl_cdiv(M, BM);
     REPDL_REQUIRE(gx * gy <= REPDL_I32_MAX);
