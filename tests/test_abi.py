@@ -117,3 +117,28 @@ def test_compiled_binding_loads_when_built():
             assert callable(getattr(hip, fn))
     else:
         assert hip.BINDING == "ctypes"
+
+
+def test_header_is_plain_c_and_struct_layouts_match(tmp_path):
+    """include/repdl_hip.h compiles as C99 on its own, and the ctypes mirrors of its descriptor
+    structs have the C compiler's sizes and field offsets."""
+    import ctypes
+    import subprocess
+
+    src = tmp_path / "layout.c"
+    src.write_text(
+        '#include <stddef.h>\n#include <stdio.h>\n#include "repdl_hip.h"\n'
+        "int main(void) {\n"
+        '  printf("%zu %zu %zu %zu %zu\\n", sizeof(repdl_adam_tensor), offsetof(repdl_adam_tensor, max_exp_avg_sq),\n'
+        "         offsetof(repdl_adam_tensor, n), offsetof(repdl_adam_tensor, sqrt_bias_correction2),\n"
+        "         offsetof(repdl_adam_tensor, step_scale));\n"
+        '  printf("%zu %zu %zu\\n", sizeof(repdl_sgd_tensor), offsetof(repdl_sgd_tensor, grad), offsetof(repdl_sgd_tensor, n));\n'
+        "  return 0;\n}\n")
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
+                    str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, stdout=subprocess.PIPE, text=True).stdout.split("\n")
+    a, s = _lib.AdamTensor, _lib.SgdTensor
+    assert [int(v) for v in out[0].split()] == [ctypes.sizeof(a), a.max_exp_avg_sq.offset, a.n.offset,
+                                                 a.sqrt_bias_correction2.offset, a.step_scale.offset]
+    assert [int(v) for v in out[1].split()] == [ctypes.sizeof(s), s.grad.offset, s.n.offset]
