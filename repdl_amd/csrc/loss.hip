@@ -6,6 +6,8 @@
 // wave reduction (max is exact, so its order is free), exp / division are done
 // lane-parallel, and the row sum is a strict j = 0..N-1 chain that every lane
 // evaluates redundantly from LDS broadcasts, so all lanes hold the same sum.
+// With many rows a wave per row is the wrong shape (every chain step is an LDS broadcast and
+// an addition issued for one row, and the SIMDs saturate on those): see "rows held on chip".
 // NaN logits are outside the contract (NaN-ness propagates, payload unspecified).
 #include "common.h"
 #include "crmath.h"
@@ -130,6 +132,223 @@ __global__ __launch_bounds__(64) void cross_entropy_rows_kernel(const float *__r
         loss[row] = l - shifted;
     }
 }
+// ---- rows held on chip ------------------------------------------------------------------
+// A workgroup of 256 threads owns R rows of at most 64 * (256 / R) columns.  TPR = 256 / R
+// threads share a row; thread j of them holds the 16-byte granules j, j + TPR, j + 2 TPR, ...
+// of the row in registers (VPT values), so the row is read from memory once, coalesced.
+// The maximum is a reduction over registers and the TPR lanes; the exponentials stay in
+// the registers and are also laid into LDS, row stride N + 1 floats; after a barrier lane
+// l of wave 0 walks row l of that image in order, one addition per column for all R rows
+// at once (the odd stride keeps the lanes on different banks).  The quotients are then
+// taken of the register copy and written once: 8 bytes per element in all (4 for the
+// loss).  Used from ROWS_ONCHIP_MIN rows on, where a wave per row saturates the SIMDs
+// with the per-row chain steps, and up to 4096 columns.
+constexpr int64_t ROWS_ONCHIP_MIN = 4096;
+constexpr int64_t ROWS_ONCHIP_MAX_N = 4096;
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float nan_max(float m, float v) { return (v != v) ? v : ((m != m) ? m : (v > m ? v : m)); }
+
+// SOFTMAX: out = softmax rows.  Otherwise: loss[row] = log(sum_j exp(x_j - m)) - (x_target - m).
+template <int R, int VPT, bool SOFTMAX>
+__global__ __launch_bounds__(256) void rows_onchip_kernel(const float *__restrict__ in, float *__restrict__ out,
+                                                          const int64_t *__restrict__ target, float *__restrict__ loss,
+                                                          int64_t M, int N, int vec_ok)
+{
+    constexpr int TPR = 256 / R; // threads per row
+    constexpr int G = VPT / 4;   // granules per thread
+    __shared__ uint64_t exp_tab[256];
+    __shared__ double log_hi[SOFTMAX ? 1 : 128];
+    __shared__ float log_invc[SOFTMAX ? 1 : 128], log_lo[SOFTMAX ? 1 : 128];
+    __shared__ float rmax[R], rsum[R];
+    extern __shared__ float image[]; // R rows of N + 1 floats
+    const int tid = threadIdx.x;
+    exp_tab[tid] = g_exp_tab2[tid];
+    if (!SOFTMAX && tid < 128)
+    {
+        log_hi[tid] = g_log_hi2[tid];
+        log_invc[tid] = g_log_invc2[tid];
+        log_lo[tid] = g_log_lo2[tid];
+    }
+    const int r = tid / TPR, j = tid % TPR;
+    const int64_t row0 = (int64_t)blockIdx.x * R;
+    const bool live = row0 + r < M;
+    const int64_t row = live ? row0 + r : M - 1; // rows past the end repeat the last one and store nothing
+    const float *x = in + row * N;
+    const int stride = N + 1;
+
+    // the row, once
+    float v[VPT];
+#pragma unroll
+    for (int i = 0; i < G; i++)
+    {
+        const int c = (i * TPR + j) * 4;
+        if (vec_ok && c + 4 <= N)
+        {
+            const v4f t = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(x + c));
+            v[4 * i + 0] = t.x;
+            v[4 * i + 1] = t.y;
+            v[4 * i + 2] = t.z;
+            v[4 * i + 3] = t.w;
+        }
+        else
+        {
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                v[4 * i + k] = c + k < N ? x[c + k] : -__builtin_inff(); // exp(-inf - m) = +0: neutral
+        }
+    }
+    float m = -__builtin_inff();
+#pragma unroll
+    for (int k = 0; k < VPT; k++)
+        m = nan_max(m, v[k]);
+#pragma unroll
+    for (int off = 1; off < TPR; off <<= 1)
+        m = nan_max(m, __shfl_xor(m, off, 64));
+    if (j == 0)
+        rmax[r] = m;
+    __syncthreads(); // tables
+
+    // exponentials: whole granule rounds are skipped with a uniform branch, everything inside is
+    // computed without branches so that the independent evaluations interleave (columns past N hold
+    // -inf and give values that are never stored)
+    float *img = image + r * stride;
+#pragma unroll
+    for (int i = 0; i < G; i++)
+    {
+        if (i * TPR * 4 < N)
+        {
+            const int c = (i * TPR + j) * 4;
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                v[4 * i + k] = crm_exp(v[4 * i + k] - m, exp_tab);
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                if (c + k < N)
+                    img[c + k] = v[4 * i + k];
+        }
+    }
+    __syncthreads();
+    if (tid < R)
+    {
+        // the chain of row `tid`: sixteen values ahead in registers while sixteen are added
+        const float *wr = image + tid * stride;
+        float acc = 0.0f;
+        float cur[16], nxt[16];
+        const int whole = N & ~15;
+        if (whole > 0)
+        {
+#pragma unroll
+            for (int u = 0; u < 16; u++)
+                cur[u] = wr[u];
+        }
+        for (int k = 0; k < whole; k += 16)
+        {
+            if (k + 16 < whole)
+            {
+#pragma unroll
+                for (int u = 0; u < 16; u++)
+                    nxt[u] = wr[k + 16 + u];
+            }
+#pragma unroll
+            for (int u = 0; u < 16; u++)
+                acc = acc + cur[u];
+#pragma unroll
+            for (int u = 0; u < 16; u++)
+                cur[u] = nxt[u];
+        }
+        for (int k = whole; k < N; k++)
+            acc = acc + wr[k];
+        rsum[tid] = acc;
+    }
+    __syncthreads();
+
+    if (SOFTMAX)
+    {
+        if (!live)
+            return;
+        const crm_divisor d = crm_divisor_make(rsum[r]);
+        float *o = out + row * N;
+#pragma unroll
+        for (int i = 0; i < G; i++)
+        {
+            if (i * TPR * 4 < N)
+            {
+                const int c = (i * TPR + j) * 4;
+                v4f t;
+                t.x = crm_div_by(v[4 * i + 0], d);
+                t.y = crm_div_by(v[4 * i + 1], d);
+                t.z = crm_div_by(v[4 * i + 2], d);
+                t.w = crm_div_by(v[4 * i + 3], d);
+                if (vec_ok && c + 4 <= N)
+                    __builtin_nontemporal_store(t, reinterpret_cast<v4f *>(o + c));
+                else
+                {
+#pragma unroll
+                    for (int k = 0; k < 4; k++)
+                        if (c + k < N)
+                            o[c + k] = t[k];
+                }
+            }
+        }
+    }
+    else if (tid < R && row0 + tid < M)
+    {
+        crm_log_tables lt;
+        lt.invc = log_invc;
+        lt.logc_hi = log_hi;
+        lt.logc_lo = log_lo;
+        const float l = crm_log(rsum[tid], lt);
+        const int64_t tg = target[row0 + tid];
+        const float shifted = (tg >= 0 && tg < N) ? in[(row0 + tid) * N + tg] - rmax[tid] : __builtin_nanf("");
+        loss[row0 + tid] = l - shifted;
+    }
+}
+
+template <int R, int VPT, bool SOFTMAX>
+int launch_rows_onchip(const float *in, float *out, const int64_t *target, float *loss, int64_t M, int64_t N, int vec_ok,
+                       hipStream_t s)
+{
+    auto kern = &rows_onchip_kernel<R, VPT, SOFTMAX>;
+    const size_t shmem = (size_t)R * (N + 1) * sizeof(float);
+    if (shmem > 40 * 1024)
+    {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)shmem);
+        if (e != hipSuccess)
+            return (int)e;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)repdl_cdiv(M, R)), dim3(256), shmem, s, in, out, target, loss, M, (int)N, vec_ok);
+    return repdl_launch_status();
+}
+
+// rows per workgroup by row length: the registers of the row's threads must hold it
+template <bool SOFTMAX>
+int rows_onchip(const float *in, float *out, const int64_t *target, float *loss, int64_t M, int64_t N, hipStream_t s)
+{
+    const bool aligned = (reinterpret_cast<uintptr_t>(in) & 15) == 0 && (!SOFTMAX || (reinterpret_cast<uintptr_t>(out) & 15) == 0);
+    const int vec_ok = N % 4 == 0 && aligned;
+    // at most 8192 elements (32 KiB of LDS image, 32 values per thread) per workgroup up to 2048
+    // columns, so that four workgroups share a CU and one's loads overlap another's chain
+    if (N <= 16)
+        return launch_rows_onchip<64, 4, SOFTMAX>(in, out, target, loss, M, N, vec_ok, s);
+    if (N <= 32)
+        return launch_rows_onchip<64, 8, SOFTMAX>(in, out, target, loss, M, N, vec_ok, s);
+    if (N <= 64)
+        return launch_rows_onchip<64, 16, SOFTMAX>(in, out, target, loss, M, N, vec_ok, s);
+    if (N <= 128)
+        return launch_rows_onchip<64, 32, SOFTMAX>(in, out, target, loss, M, N, vec_ok, s);
+    if (N <= 256)
+        return launch_rows_onchip<32, 32, SOFTMAX>(in, out, target, loss, M, N, vec_ok, s);
+    if (N <= 512)
+        return launch_rows_onchip<16, 32, SOFTMAX>(in, out, target, loss, M, N, vec_ok, s);
+    if (N <= 1024)
+        return launch_rows_onchip<8, 32, SOFTMAX>(in, out, target, loss, M, N, vec_ok, s);
+    if (N <= 2048)
+        return launch_rows_onchip<4, 32, SOFTMAX>(in, out, target, loss, M, N, vec_ok, s);
+    return launch_rows_onchip<4, 64, SOFTMAX>(in, out, target, loss, M, N, vec_ok, s);
+}
 } // namespace
 
 REPDL_API int repdl_hip_softmax(const float *in, float *out, int64_t M, int64_t N, void *stream)
@@ -138,6 +357,8 @@ REPDL_API int repdl_hip_softmax(const float *in, float *out, int64_t M, int64_t 
     if (M == 0 || N == 0)
         return REPDL_OK;
     REPDL_REQUIRE(in != nullptr && out != nullptr && M <= REPDL_I32_MAX);
+    if (M >= ROWS_ONCHIP_MIN && N <= ROWS_ONCHIP_MAX_N)
+        return rows_onchip<true>(in, out, nullptr, nullptr, M, N, repdl_stream(stream));
     hipLaunchKernelGGL(softmax_kernel, dim3((unsigned)M), dim3(64), 0, repdl_stream(stream), in, out, M, N);
     return repdl_launch_status();
 }
@@ -151,9 +372,15 @@ REPDL_API int repdl_hip_cross_entropy(const float *in, const int64_t *target, fl
         REPDL_REQUIRE(in != nullptr && target != nullptr && M <= REPDL_I32_MAX);
         if (workspace == nullptr)
             return REPDL_E_WORKSPACE;
-        hipLaunchKernelGGL(cross_entropy_rows_kernel, dim3((unsigned)M), dim3(64), 0, repdl_stream(stream),
-                           in, target, workspace, M, N);
-        int rc = repdl_launch_status();
+        int rc;
+        if (M >= ROWS_ONCHIP_MIN && N <= ROWS_ONCHIP_MAX_N)
+            rc = rows_onchip<false>(in, nullptr, target, workspace, M, N, repdl_stream(stream));
+        else
+        {
+            hipLaunchKernelGGL(cross_entropy_rows_kernel, dim3((unsigned)M), dim3(64), 0, repdl_stream(stream),
+                               in, target, workspace, M, N);
+            rc = repdl_launch_status();
+        }
         if (rc != REPDL_OK)
             return rc;
     }
