@@ -70,7 +70,18 @@ __device__ __forceinline__ float row_exp_sum(const float *x, float *e_out, int64
         }
         __syncthreads();
         const int cnt = (N - c0 < CH) ? (int)(N - c0) : CH;
-        for (int c = 0; c < cnt; c++)
+        int c = 0;
+        for (; c + 16 <= cnt; c += 16)
+        {
+            float b[16]; // sixteen broadcast reads in flight, then their additions in order
+#pragma unroll
+            for (int u = 0; u < 16; u++)
+                b[u] = stage[c + u];
+#pragma unroll
+            for (int u = 0; u < 16; u++)
+                acc = acc + b[u];
+        }
+        for (; c < cnt; c++)
             acc = acc + stage[c];
         __syncthreads();
     }
