@@ -15,7 +15,8 @@ pytestmark = pytest.mark.gpu
 
 SHAPES = [(4095, 10), (4096, 10), (4097, 1), (4100, 63), (4160, 64), (4099, 65), (5000, 130), (4096, 1000), (8192, 257),
           (70000, 12), (4200, 4), (4101, 128), (4098, 256), (4097, 258), (4100, 512), (4099, 515), (4096, 1024), (4097, 1028),
-          (4098, 2048), (4097, 2050), (4099, 4096), (4097, 4097), (4096, 3001)]
+          (4098, 2048), (4097, 2050), (4099, 4096), (4097, 4097), (4096, 3001),
+          (1024, 2048), (1023, 2050), (1500, 1399), (2047, 1024), (2049, 1023)]
 
 
 def _logits(seed, M, N):
