@@ -178,6 +178,22 @@ int repdl_hip_softmax(const float *in, float *out, int64_t M, int64_t N, void *s
 int repdl_hip_cross_entropy(const float *in, const int64_t *target, float *out, int64_t M,
                             int64_t N, float *workspace, void *stream);
 
+/* Batch normalisation, the elementwise passes -- the reference has no backend function for
+ * these: repdl/nn/batchnorm.py:12-66 composes them from PyTorch tensor operations, one
+ * rounding each.  Each entry point evaluates one of those compositions per element with the
+ * same roundings in the same order, in one pass over memory.  Tensors are
+ * [outer][channels][inner] (NCHW: outer = N, inner = H*W; [B,F]: outer = B, inner = 1); mean,
+ * std, weight, bias and coef are [channels]; `/` is the IEEE quotient.
+ *   bn_apply         y   = RN(RN(RN(RN(x - mean[c]) / std[c]) * weight[c]) + bias[c])   (batchnorm.py:25-32)
+ *   bn_gvar_term     out = RN(RN(grad_y * RN(mean[c] - x)) * coef[c])                   (:56-58, before the sum)
+ *   bn_gweight_term  out = RN(RN(RN(x - mean[c]) / std[c]) * grad_y)                    (:60-61, before the sum) */
+int repdl_hip_bn_apply(const float *x, const float *mean, const float *std, const float *weight, const float *bias,
+                       float *y, int64_t outer, int64_t channels, int64_t inner, void *stream);
+int repdl_hip_bn_gvar_term(const float *grad_y, const float *x, const float *mean, const float *coef, float *out,
+                           int64_t outer, int64_t channels, int64_t inner, void *stream);
+int repdl_hip_bn_gweight_term(const float *x, const float *mean, const float *std, const float *grad_y, float *out,
+                              int64_t outer, int64_t channels, int64_t inner, void *stream);
+
 /* Optimizer steps -- the reference has no backend function for these: repdl/optim.py:56-83
  * writes Adam as a sequence of PyTorch tensor operations around ops.sqrt and a true
  * division (a dozen launches and temporaries per parameter).  These entry points evaluate

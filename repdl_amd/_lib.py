@@ -52,6 +52,9 @@ SIGNATURES = {
     "repdl_hip_div_scalar": [_P, _F32, _P, _I64, _P],
     "repdl_hip_softmax": [_P, _P, _I64, _I64, _P],
     "repdl_hip_cross_entropy": [_P, _P, _P, _I64, _I64, _P, _P],
+    "repdl_hip_bn_apply": [_P] * 6 + [_I64] * 3 + [_P],
+    "repdl_hip_bn_gvar_term": [_P] * 5 + [_I64] * 3 + [_P],
+    "repdl_hip_bn_gweight_term": [_P] * 5 + [_I64] * 3 + [_P],
     "repdl_hip_adam_step": [ctypes.POINTER(AdamTensor), _INT] + [_F32] * 6 + [_P],
     "repdl_hip_sgd_step": [ctypes.POINTER(SgdTensor), _INT, _F32, _P],
     "repdl_hip_mfma_selftest": [_I64, _I64, ctypes.c_uint64, ctypes.POINTER(ctypes.c_uint64)],

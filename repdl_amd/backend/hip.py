@@ -2,7 +2,8 @@
 ``repdl.backend.cuda`` (backend/cuda/bind.cpp:12-19): the same ten functions with the
 same positional signatures, tensors in and a new tensor out, plus the elementwise
 operators (``exp``, ``log``, ``sqrt``, ``div``, ``div_scalar``) and ``mm_bias`` /
-``conv2d_bias`` (a layer's bias added in the kernel's epilogue).
+``conv2d_bias`` (a layer's bias added in the kernel's epilogue) and the fused elementwise
+passes of batch normalisation (``bn_apply``, ``bn_gvar_term``, ``bn_gweight_term``).
 
 Two bindings of the one C-ABI library (include/repdl_hip.h) can serve it:
 
@@ -23,7 +24,8 @@ except ImportError:  # not built
     _ext_binding = None
 
 FUNCTIONS = ("mm", "conv2d", "conv2d_grad_input", "conv2d_grad_kernel", "sum1d", "sum2d_dim0", "sum2d_dim1",
-             "sum4d_dim023", "softmax", "cross_entropy", "exp", "log", "sqrt", "div", "div_scalar", "mm_bias", "conv2d_bias")
+             "sum4d_dim023", "softmax", "cross_entropy", "exp", "log", "sqrt", "div", "div_scalar", "mm_bias", "conv2d_bias",
+             "bn_apply", "bn_gvar_term", "bn_gweight_term")
 if _ext_binding is not None and not all(hasattr(_ext_binding, fn) for fn in FUNCTIONS):
     import warnings
 

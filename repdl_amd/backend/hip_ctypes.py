@@ -2,8 +2,8 @@
 ``repdl.backend.cuda`` (backend/cuda/bind.cpp:12-19) bound to the C ABI with ctypes:
 the same ten functions with the same positional signatures, tensors in and a new
 tensor out, plus the elementwise operators (``exp``, ``log``, ``sqrt``, ``div``,
-``div_scalar``) and ``mm_bias`` / ``conv2d_bias`` (the layer's bias added in the
-kernel's epilogue).  ``repdl_amd.backend.hip`` serves these when the compiled binding
+``div_scalar``), ``mm_bias`` / ``conv2d_bias`` (the layer's bias added in the
+kernel's epilogue) and the fused elementwise passes of batch normalisation.  ``repdl_amd.backend.hip`` serves these when the compiled binding
 (csrc/bind.cpp) has not been built; both call the same library.
 
 Each function validates its tensors (float32, on the GPU, made contiguous),
@@ -239,5 +239,61 @@ def cross_entropy(input: torch.Tensor, target: torch.Tensor) -> torch.Tensor:
     work = torch.empty((max(x.shape[0], 1),), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
         _lib.call("repdl_hip_cross_entropy", _ptr(x), _ptr(t), _ptr(out), x.shape[0], x.shape[1], _ptr(work),
+                  _stream(x))
+    return out
+
+
+def _bn_geometry(x: torch.Tensor, *vectors: torch.Tensor):
+    """[N,C,H,W] or [B,F] with per-channel vectors of C (F) elements -> (outer, channels, inner)."""
+    if x.dim() == 4:
+        outer, channels, inner = x.shape[0], x.shape[1], x.shape[2] * x.shape[3]
+    elif x.dim() == 2:
+        outer, channels, inner = x.shape[0], x.shape[1], 1
+    else:
+        raise RuntimeError("batch norm takes 2-D or 4-D tensors, got %d dimensions" % x.dim())
+    for v in vectors:
+        if v.numel() != channels:
+            raise RuntimeError("a per-channel vector has %d elements for %d channels" % (v.numel(), channels))
+        _same_device(v, x)
+    return outer, channels, inner
+
+
+def bn_apply(input, mean, std, weight, bias) -> torch.Tensor:
+    """((input - mean) / std) * weight + bias per channel, every operation rounded (repdl/nn/batchnorm.py:25-32)."""
+    x = _check(input, "input")
+    m, s, w, b = (_check(t, n, 1) for t, n in ((mean, "mean"), (std, "std"), (weight, "weight"), (bias, "bias")))
+    outer, channels, inner = _bn_geometry(x, m, s, w, b)
+    out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        _lib.call("repdl_hip_bn_apply", _ptr(x), _ptr(m), _ptr(s), _ptr(w), _ptr(b), _ptr(out), outer, channels, inner,
+                  _stream(x))
+    return out
+
+
+def bn_gvar_term(grad_output, input, mean, coef) -> torch.Tensor:
+    """(grad_output * (mean - input)) * coef per channel: what grad_var sums (repdl/nn/batchnorm.py:56-58)."""
+    g, x = _check(grad_output, "grad_output"), _check(input, "input")
+    m, c = _check(mean, "mean", 1), _check(coef, "coef", 1)
+    if g.shape != x.shape:
+        raise RuntimeError("grad_output and input differ in shape")
+    _same_device(g, x)
+    outer, channels, inner = _bn_geometry(x, m, c)
+    out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        _lib.call("repdl_hip_bn_gvar_term", _ptr(g), _ptr(x), _ptr(m), _ptr(c), _ptr(out), outer, channels, inner, _stream(x))
+    return out
+
+
+def bn_gweight_term(input, mean, std, grad_output) -> torch.Tensor:
+    """((input - mean) / std) * grad_output per channel: what grad_weight sums (repdl/nn/batchnorm.py:60-61)."""
+    x, g = _check(input, "input"), _check(grad_output, "grad_output")
+    m, s = _check(mean, "mean", 1), _check(std, "std", 1)
+    if g.shape != x.shape:
+        raise RuntimeError("grad_output and input differ in shape")
+    _same_device(g, x)
+    outer, channels, inner = _bn_geometry(x, m, s)
+    out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        _lib.call("repdl_hip_bn_gweight_term", _ptr(x), _ptr(m), _ptr(s), _ptr(g), _ptr(out), outer, channels, inner,
                   _stream(x))
     return out

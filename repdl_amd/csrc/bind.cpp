@@ -3,7 +3,8 @@
 // functions with the same positional signatures (matrix_multiplication.cu:234-235, 267;
 // convolution.cu:153-155, 259-262, 359-362, 385-387; summation.cu:149-155;
 // softmax.cpp:15, 28; cross_entropy.cpp:15, 31), plus exp / log / sqrt / div / div_scalar and
-// mm_bias / conv2d_bias (the layer's bias added in the kernel's epilogue).
+// mm_bias / conv2d_bias (the layer's bias added in the kernel's epilogue) and the fused elementwise
+// passes of batch normalisation (bn_apply, bn_gvar_term, bn_gweight_term).
 // It is the only file of this library that knows about PyTorch: every function checks its
 // tensors, allocates the output on the input's device, and hands raw pointers and the current
 // stream to the C ABI of include/repdl_hip.h.  Host C++ only; built with the host compiler
@@ -256,6 +257,77 @@ torch::Tensor cross_entropy(const torch::Tensor &input, const torch::Tensor &tar
        "repdl_hip_cross_entropy");
     return out;
 }
+namespace
+{
+// [N,C,H,W] or [B,F] with per-channel vectors -> outer, channels, inner
+void bn_geometry(const torch::Tensor &x, std::initializer_list<torch::Tensor> vectors, int64_t &outer, int64_t &channels,
+                 int64_t &inner)
+{
+    TORCH_CHECK(x.dim() == 4 || x.dim() == 2, "batch norm takes 2-D or 4-D tensors, got ", x.dim(), " dimensions");
+    outer = x.size(0);
+    channels = x.size(1);
+    inner = x.dim() == 4 ? x.size(2) * x.size(3) : 1;
+    for (const auto &v : vectors)
+    {
+        TORCH_CHECK(v.numel() == channels, "a per-channel vector has ", v.numel(), " elements for ", channels, " channels");
+        same_device(v, x);
+    }
+}
+} // namespace
+
+// ((input - mean) / std) * weight + bias per channel, every operation rounded (repdl/nn/batchnorm.py:25-32)
+torch::Tensor bn_apply(const torch::Tensor &input, const torch::Tensor &mean, const torch::Tensor &std,
+                       const torch::Tensor &weight, const torch::Tensor &bias)
+{
+    const auto x = checked(input, "input", -1);
+    const auto m = checked(mean, "mean", 1), s = checked(std, "std", 1), w = checked(weight, "weight", 1),
+               b = checked(bias, "bias", 1);
+    int64_t outer, channels, inner;
+    bn_geometry(x, {m, s, w, b}, outer, channels, inner);
+    const DeviceGuard guard(x.device());
+    auto out = torch::empty_like(x);
+    ok(repdl_hip_bn_apply(x.data_ptr<float>(), m.data_ptr<float>(), s.data_ptr<float>(), w.data_ptr<float>(),
+                          b.data_ptr<float>(), out.data_ptr<float>(), outer, channels, inner, current_stream()),
+       "repdl_hip_bn_apply");
+    return out;
+}
+
+// (grad_output * (mean - input)) * coef per channel: what grad_var sums (repdl/nn/batchnorm.py:56-58)
+torch::Tensor bn_gvar_term(const torch::Tensor &grad_output, const torch::Tensor &input, const torch::Tensor &mean,
+                           const torch::Tensor &coef)
+{
+    const auto g = checked(grad_output, "grad_output", -1), x = checked(input, "input", -1);
+    const auto m = checked(mean, "mean", 1), c = checked(coef, "coef", 1);
+    TORCH_CHECK(g.sizes() == x.sizes(), "grad_output and input differ in shape");
+    same_device(g, x);
+    int64_t outer, channels, inner;
+    bn_geometry(x, {m, c}, outer, channels, inner);
+    const DeviceGuard guard(x.device());
+    auto out = torch::empty_like(x);
+    ok(repdl_hip_bn_gvar_term(g.data_ptr<float>(), x.data_ptr<float>(), m.data_ptr<float>(), c.data_ptr<float>(),
+                              out.data_ptr<float>(), outer, channels, inner, current_stream()),
+       "repdl_hip_bn_gvar_term");
+    return out;
+}
+
+// ((input - mean) / std) * grad_output per channel: what grad_weight sums (repdl/nn/batchnorm.py:60-61)
+torch::Tensor bn_gweight_term(const torch::Tensor &input, const torch::Tensor &mean, const torch::Tensor &std,
+                              const torch::Tensor &grad_output)
+{
+    const auto x = checked(input, "input", -1), g = checked(grad_output, "grad_output", -1);
+    const auto m = checked(mean, "mean", 1), s = checked(std, "std", 1);
+    TORCH_CHECK(g.sizes() == x.sizes(), "grad_output and input differ in shape");
+    same_device(g, x);
+    int64_t outer, channels, inner;
+    bn_geometry(x, {m, s}, outer, channels, inner);
+    const DeviceGuard guard(x.device());
+    auto out = torch::empty_like(x);
+    ok(repdl_hip_bn_gweight_term(x.data_ptr<float>(), m.data_ptr<float>(), s.data_ptr<float>(), g.data_ptr<float>(),
+                                 out.data_ptr<float>(), outer, channels, inner, current_stream()),
+       "repdl_hip_bn_gweight_term");
+    return out;
+}
+
 } // namespace hip
 } // namespace repdl
 
@@ -279,4 +351,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("div_scalar", &h::div_scalar);
     m.def("mm_bias", &h::mm_bias);
     m.def("conv2d_bias", &h::conv2d_bias);
+    m.def("bn_apply", &h::bn_apply);
+    m.def("bn_gvar_term", &h::bn_gvar_term);
+    m.def("bn_gweight_term", &h::bn_gweight_term);
 }

@@ -148,18 +148,11 @@ class _BatchNorm(torch.autograd.Function):
     def forward(ctx, x, mean, var, weight, bias, eps):
         std = ops.sqrt(var + eps)
         ctx.save_for_backward(x, mean, std, weight)
-        y = ops.div(x - _per_channel(mean, x), _per_channel(std, x).expand_as(x))
-        if x.dim() == 4:
-            y *= _per_channel(weight, x)
-            y += _per_channel(bias, x)
-        else:
-            y = weight * y + bias
-        return y
+        return ops.bn_apply(x, mean, std, weight, bias)  # ((x - mean) / std) * weight + bias, four roundings
 
     @staticmethod
     def backward(ctx, gy):
         x, mean, std, weight = ctx.saved_tensors
-        mean_b, std_b, weight_b = (_per_channel(t, gy) for t in (mean, std, weight))
         reduce = ops.sum4d_dim023 if gy.dim() == 4 else ops.sum2d_dim0
         need = ctx.needs_input_grad
         w_over_std = ops.div(weight, std)
@@ -169,8 +162,8 @@ class _BatchNorm(torch.autograd.Function):
         gx, rgy, gvar, gweight = _side_by_side(gy.device, [
             (lambda: _per_channel(w_over_std, gy) * gy) if need[0] else None,
             (lambda: reduce(gy)) if need[1] or need[4] else None,
-            (lambda: reduce(gy * (mean_b - x) * _per_channel(coef, gy))) if need[2] else None,
-            (lambda: reduce(ops.div(x - mean_b, std_b.expand_as(x)) * gy)) if need[3] else None])
+            (lambda: reduce(ops.bn_gvar_term(gy, x, mean, coef))) if need[2] else None,      # gy * (mean - x) * coef
+            (lambda: reduce(ops.bn_gweight_term(x, mean, std, gy))) if need[3] else None])  # (x - mean) / std * gy
         gmean = (-w_over_std) * rgy if need[1] else None
         gbias = rgy if need[4] else None
         return gx, gmean, gvar, gweight, gbias, None

@@ -132,3 +132,21 @@ def sum(input: torch.Tensor, dim=None, keepdim: bool = False, average: bool = Fa
     if nd == 4 and dim is not None and tuple(dim) == (0, 2, 3):
         return sum4d_dim023(input, keepdim, average)
     raise NotImplementedError("sum over dim=%r of a %d-D tensor has no reproducible operator" % (dim, nd))
+
+
+def bn_apply(input: torch.Tensor, mean: torch.Tensor, std: torch.Tensor, weight: torch.Tensor,
+             bias: torch.Tensor) -> torch.Tensor:
+    """``((input - mean) / std) * weight + bias`` with the per-channel vectors broadcast over a
+    [N,C,H,W] or [B,F] input: the four rounded operations of the reference's forward
+    (nn/batchnorm.py:25-32) in one pass.  Not in the reference's ``ops``."""
+    return _backend(input).bn_apply(input, mean, std, weight, bias)
+
+
+def bn_gvar_term(grad_output: torch.Tensor, input: torch.Tensor, mean: torch.Tensor, coef: torch.Tensor) -> torch.Tensor:
+    """``(grad_output * (mean - input)) * coef``: the tensor that grad_var sums (nn/batchnorm.py:56-58)."""
+    return _backend(input).bn_gvar_term(grad_output, input, mean, coef)
+
+
+def bn_gweight_term(input: torch.Tensor, mean: torch.Tensor, std: torch.Tensor, grad_output: torch.Tensor) -> torch.Tensor:
+    """``((input - mean) / std) * grad_output``: the tensor that grad_weight sums (nn/batchnorm.py:60-61)."""
+    return _backend(input).bn_gweight_term(input, mean, std, grad_output)

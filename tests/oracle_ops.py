@@ -44,6 +44,30 @@ class _OracleBackend:
             y += bias.unsqueeze(-1).unsqueeze(-1)
         return y
 
+    # the reference's own compositions (repdl/nn/batchnorm.py:25-32, 56-58, 60-61); its divisions go through
+    # the oracle's div, which is PyTorch's CPU division
+    @staticmethod
+    def _bc(v, like):
+        return v.unsqueeze(-1).unsqueeze(-1) if like.dim() == 4 else v
+
+    @staticmethod
+    def bn_apply(x, mean, std, weight, bias):
+        bc = _OracleBackend._bc
+        y = _OracleBackend.div(x - bc(mean, x), bc(std, x))
+        y *= bc(weight, x)
+        y += bc(bias, x)
+        return y
+
+    @staticmethod
+    def bn_gvar_term(gy, x, mean, coef):
+        bc = _OracleBackend._bc
+        return gy * (bc(mean, x) - x) * bc(coef, x)
+
+    @staticmethod
+    def bn_gweight_term(x, mean, std, gy):
+        bc = _OracleBackend._bc
+        return _OracleBackend.div(x - bc(mean, x), bc(std, x)) * gy
+
     @staticmethod
     def div(a, b):
         shape = torch.broadcast_shapes(a.shape, b.shape)
