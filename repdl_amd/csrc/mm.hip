@@ -467,9 +467,14 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_fast_kernel(const float
 {
     constexpr int NTH = 64 * WGM * WGN;
     constexpr int TM = 32 * FM * WGM, TN = 32 * FN * WGN;
-    constexpr int LDA_ = TM + 4, LDB_ = TN + 4;
-    constexpr int NVA = TM * BK / 4 / NTH, NVB = TN * BK / 4 / NTH;
     constexpr bool A_KC = !TA, B_KC = TB;
+    constexpr int LDA_ = TM + 4, LDB_ = TN + 4;
+    // Tiles of one wave per SIMD (64x64, 128x128) run the software-pipelined loop below: a lone
+    // wave has nobody to cover its LDS latency after a barrier (1024^3: 31 -> 25-29 us, 1536^2 x
+    // 4096: +7 %).  With two waves per SIMD (256x256) the plain loop is the faster one by 3-4 %.
+    constexpr bool PIPE = FM * FN <= 4;
+    constexpr int PIPE_STORE_AT = 4; // k-pair after which the next k-tile goes to LDS
+    constexpr int NVA = TM * BK / 4 / NTH, NVB = TN * BK / 4 / NTH;
     typedef float v4f __attribute__((ext_vector_type(4)));
     extern __shared__ __attribute__((aligned(16))) float smem[];
     float *const As = smem;                 // [2][BK * LDA_]
@@ -711,6 +716,53 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_fast_kernel(const float
         store_tiles(0);
     }
     __syncthreads();
+    if constexpr (PIPE)
+    {
+        // Software pipeline over the k-pairs of a k-tile: the operands of pair kp + 1 are read
+        // while the matrix instructions of pair kp run, the next k-tile is stored to the other
+        // LDS buffer mid-way, and the barrier sits before the last pair, whose instructions cover
+        // the first operand reads of the next k-tile.  One barrier per k-tile is enough: every read
+        // of a buffer is issued before the barrier that precedes the next stores into it.
+        float pa[2][FM], pb[2][FN];
+        auto read_ops = [&](int buf, int kp, float(&a)[FM], float(&b)[FN]) {
+            const float *as = As + buf * BK * LDA_ + a_off, *bs = Bs + buf * BK * LDB_ + b_off;
+#pragma unroll
+            for (int i = 0; i < FM; i++)
+                a[i] = as[2 * kp * LDA_ + 32 * i];
+#pragma unroll
+            for (int j = 0; j < FN; j++)
+                b[j] = bs[2 * kp * LDB_ + 32 * j];
+        };
+        if (nkt > 0)
+            read_ops(0, 0, pa[0], pb[0]);
+        for (int64_t kt = 0; kt < nkt; kt++)
+        {
+            const int cur = (int)(kt & 1);
+            const bool more = kt + 1 < nkt;
+            if (more)
+                load_any(kt + 1);
+#pragma unroll
+            for (int kp = 0; kp < BK / 2; kp++)
+            {
+                if (kp + 1 < BK / 2)
+                    read_ops(cur, kp + 1, pa[(kp + 1) & 1], pb[(kp + 1) & 1]);
+                else if (more)
+                    read_ops(cur ^ 1, 0, pa[0], pb[0]);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < FM; i++)
+#pragma unroll
+                    for (int j = 0; j < FN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[kp & 1][i], pb[kp & 1][j], acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (kp == PIPE_STORE_AT && more)
+                    store_tiles(cur ^ 1);
+                if (kp == BK / 2 - 2)
+                    __syncthreads();
+            }
+        }
+    }
+    else
     for (int64_t kt = 0; kt < nkt; kt++)
     {
         const int cur = (int)(kt & 1);
