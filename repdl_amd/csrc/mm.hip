@@ -882,18 +882,18 @@ REPDL_API int repdl_hip_mm_bias(const float *A, const float *B, const float *bia
     hipStream_t s = repdl_stream(stream);
     if (repdl_mfma_exact())
     {
-        // Tile choice: tiles run in rounds over the 256 CUs (workgroups that share a CU share its
-        // matrix pipes), so a configuration costs rounds x tile area / efficiency.  Measured rates per CU
-        // relative to the 256x256 tile (135 TFLOP/s when every CU has one or more): 128x128 tiles 0.77
-        // with one per CU, 0.86 with two or three, 0.92 from four on; 64x64 tiles 0.8 up to three per
-        // CU, 0.52 in large launches (twice the operand traffic per flop).  A 4096x4096 output is 256
-        // tiles of 256x256, one per CU, at the full rate (4096x4096x32768: 8.77 -> 8.11 ms against
-        // 128x128 tiles).
-        auto rounds = [&](int64_t tm, int64_t tn) { return repdl_cdiv(repdl_cdiv(M, tm) * repdl_cdiv(N, tn), 256); };
-        const int64_t r256 = rounds(256, 256), r128 = rounds(128, 128), r64 = rounds(64, 64);
+        // Tile choice.  A CU runs its tiles one after the other (256x256: one workgroup fills it) or
+        // side by side (smaller tiles), so a configuration costs (most tiles on any CU) x tile area
+        // / rate, with the rates measured per configuration and tiles per CU, relative to the
+        // 256x256 tile (135 TFLOP/s chip-wide): 128x128 0.785 alone on its CU, 0.92 with two, 0.955
+        // from three on; 64x64 0.555 alone, 0.76 with two, 0.85 with three or four, 0.88 beyond
+        // (4096^3: 1.03 / 1.08 / 1.13 ms with 256 / 128 / 64 tiles; 3072^2 x 4096, 144 / 576 / 2304
+        // tiles: 1.02 / 0.79 / 0.65 ms; 1024^3: 0.26 / 0.080 / 0.029 ms).
+        auto per_cu = [&](int64_t tm, int64_t tn) { return repdl_cdiv(repdl_cdiv(M, tm) * repdl_cdiv(N, tn), 256); };
+        const int64_t r256 = per_cu(256, 256), r128 = per_cu(128, 128), r64 = per_cu(64, 64);
         const double c256 = (double)r256 * 65536.0;
-        const double c128 = (double)r128 * 16384.0 / (r128 >= 4 ? 0.92 : r128 >= 2 ? 0.86 : 0.77);
-        const double c64 = (double)r64 * 4096.0 / (r64 <= 3 ? 0.8 : 0.52);
+        const double c128 = (double)r128 * 16384.0 / (r128 >= 3 ? 0.955 : r128 == 2 ? 0.92 : 0.785);
+        const double c64 = (double)r64 * 4096.0 / (r64 >= 5 ? 0.88 : r64 >= 3 ? 0.85 : r64 == 2 ? 0.76 : 0.555);
         if (c256 <= c128 && c256 <= c64)
             return launch_mfma<4, 2, 2, 4>(A, B, C, bias, M, N, K, transA, transB, avec, bvec, s);
         if (c128 <= c64)
