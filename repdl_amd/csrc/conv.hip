@@ -858,6 +858,10 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
     // LDS it saves is a tenth workgroup per CU and worth more than the barrier.
     constexpr int LDBF = TBN;
     constexpr int NA = PB == 2 ? 2 : 1;
+    // 128-pixel tiles run the software-pipelined loop (112x112 forward 0.729 -> 0.697 ms, 128
+    // channels at 28x28 0.219 -> 0.208); with 64-pixel tiles it needs the second kernel buffer
+    // and loses more with the tenth workgroup than it gains (56x56 forward 0.203 -> 0.212 ms).
+    constexpr bool PIPE = PB == 2;
     __shared__ __attribute__((aligned(16))) float As[NA][BK * LDA];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDBF];
 
@@ -951,6 +955,52 @@ __global__ __launch_bounds__(2 * BM) void conv_gemm_fast_kernel(const float *__r
     if (has_bias && tid < BM)
         bias_s[tid] = bias_r;
     __syncthreads();
+    if constexpr (PIPE)
+    {
+        // Software pipeline over the k-pairs of a k-tile: the operands of pair kp + 1 are read
+        // while the matrix instructions of pair kp run, the next k-tile goes to the other LDS
+        // buffers mid-way, and the barrier sits before the last pair, whose instructions cover
+        // the first operand reads of the next k-tile.  Every read of a buffer is issued before
+        // the barrier that precedes the next stores into it, so one barrier per k-tile is enough.
+        float pa[2][2], pb[2][PB];
+        auto read_ops = [&](int buf, int kp, float(&a)[2], float(&b)[PB]) {
+            const float *as = As[buf] + a_off, *bs = Bs[buf] + b_off;
+            a[0] = as[2 * kp * LDA];
+            a[1] = as[2 * kp * LDA + 32];
+#pragma unroll
+            for (int j = 0; j < PB; j++)
+                b[j] = bs[2 * kp * LDBF + 32 * j];
+        };
+        if (nkt > 0)
+            read_ops(0, 0, pa[0], pb[0]);
+        for (int kt = 0; kt < nkt; kt++)
+        {
+            const int cur = kt & 1;
+            const bool more = kt + 1 < nkt;
+            if (more)
+                load_tiles(kt + 1);
+#pragma unroll
+            for (int kp = 0; kp < BK / 2; kp++)
+            {
+                if (kp + 1 < BK / 2)
+                    read_ops(cur, kp + 1, pa[(kp + 1) & 1], pb[(kp + 1) & 1]);
+                else if (more)
+                    read_ops(cur ^ 1, 0, pa[0], pb[0]);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < PB; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[kp & 1][i], pb[kp & 1][j], acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (kp == 4 && more)
+                    store_tiles(cur ^ 1);
+                if (kp == BK / 2 - 2)
+                    __syncthreads();
+            }
+        }
+    }
+    else
     for (int kt = 0; kt < nkt; kt++)
     {
         const int cur = kt & 1;
