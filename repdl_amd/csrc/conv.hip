@@ -752,19 +752,37 @@ __global__ __launch_bounds__(256) void conv_pad_kernel(const float *__restrict__
     {
         const float *__restrict__ sp = src + pl * H * W;
         float *__restrict__ dp = dst + pl * plane;
-        for (int hp = wave; hp < Hp; hp += 4)
+        // eight rows per wave and pass: their loads are all issued before the first store (one
+        // row in flight per wave left the copy at 3.2 TB/s)
+        constexpr int U = 8;
+        for (int wp = lane; wp < Wp; wp += 64)
         {
             // source element (h, w) lands at (PT + h*dH, PL + w*dW); everything else is zero
-            const int hd = hp - PT;
-            const int h = dH == 1 ? hd : hd / dH;
-            const bool hin = hd >= 0 && h < H && (dH == 1 || h * dH == hd);
-            for (int wp = lane; wp < Wp; wp += 64)
+            const int wd = wp - PL;
+            const int w = dW == 1 ? wd : wd / dW;
+            const bool win = wd >= 0 && w < W && (dW == 1 || w * dW == wd);
+            for (int hp0 = wave; hp0 < Hp; hp0 += 4 * U)
             {
-                const int wd = wp - PL;
-                const int w = dW == 1 ? wd : wd / dW;
-                const float v = (hin && wd >= 0 && w < W && (dW == 1 || w * dW == wd)) ? sp[h * W + w] : 0.0f;
-                dp[hp * Wp + wp] = v;
-                m = guard_min(m, guard_bits(v));
+                float v[U];
+#pragma unroll
+                for (int u = 0; u < U; u++)
+                {
+                    const int hp = hp0 + 4 * u;
+                    const int hd = hp - PT;
+                    const int h = dH == 1 ? hd : hd / dH;
+                    const bool hin = hp < Hp && hd >= 0 && h < H && (dH == 1 || h * dH == hd);
+                    v[u] = (hin && win) ? sp[h * W + w] : 0.0f;
+                }
+#pragma unroll
+                for (int u = 0; u < U; u++)
+                {
+                    const int hp = hp0 + 4 * u;
+                    if (hp < Hp)
+                    {
+                        dp[hp * Wp + wp] = v[u];
+                        m = guard_min(m, guard_bits(v[u]));
+                    }
+                }
             }
         }
     }
