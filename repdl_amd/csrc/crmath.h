@@ -270,10 +270,10 @@ CRM_FN float crm_log(float x, crm_log_tables tab)
     // zeros, negatives, infinities and NaNs run through the core harmlessly (the
     // table index is masked) and are overridden
     const uint32_t gen = crm_f2u(crm_d2f(crm_log64_core((double)x, tab)));
-    const uint32_t ax = ux & 0x7FFFFFFFu;
-    uint32_t sp = CRM_QNAN_NEG;                        // log(negative), log(-inf): (x-x)/(x-x) on x86
-    sp = (ux == 0x7F800000u) ? 0x7F800000u : sp;       // log(+inf)
-    sp = (ax == 0u) ? 0xFF800000u : sp;                // log(+-0) = -inf
-    sp = (ax > 0x7F800000u) ? (ux | 0x00400000u) : sp; // NaN: sign and payload kept, quieted
+    // the special inputs in three selects: x + x is +inf for +inf and, for a NaN, the same
+    // NaN quieted (sign and payload kept); a NaN compares false both times
+    uint32_t sp = crm_f2u(x + x);
+    sp = (x < 0.0f) ? CRM_QNAN_NEG : sp;  // log(negative), log(-inf): (x-x)/(x-x) on x86
+    sp = (x == 0.0f) ? 0xFF800000u : sp;  // log(+-0) = -inf
     return crm_u2f((ux - 1u >= 0x7F7FFFFFu) ? sp : gen);
 }
