@@ -36,10 +36,10 @@ HBM_PEAK_GBS = 8000.0
 # reads 524300 for 1 GiB (factor 1.99995 KiB per count), WRITE_SIZE 1048576 (factor 1.0).  Summary:
 # profiles/hbm_traffic_counters.txt.  Valid for the default workload sizes only.
 MEASURED_TRAFFIC_BYTES = {
-    "mm": 5482423 * 1.99995 * 1024 + 262148 * 1024,       # 1.15e10: operand panels re-read behind L2 (35 % L2 hit rate)
-    "exp": 524335 * 1.99995 * 1024 + 1048599 * 1024,      # 2.147e9 = the algorithmic 8 B/element
+    "mm": 5426902 * 1.99995 * 1024 + 262155 * 1024,       # 1.14e10: operand panels re-read behind L2 (35 % L2 hit rate)
+    "exp": 524335 * 1.99995 * 1024 + 1048586 * 1024,      # 2.147e9 = the algorithmic 8 B/element
     "sum2d_dim1": 524389 * 1.99995 * 1024 + 64 * 1024,    # 1.074e9 = the algorithmic 4 B/element
-    "adam_step": 524363 * 1.99995 * 1024 + 786446 * 1024,  # 1.879e9 = the algorithmic 28 B/element (2^26 elements)
+    "adam_step": 524363 * 1.99995 * 1024 + 786443 * 1024,  # 1.879e9 = the algorithmic 28 B/element (2^26 elements)
 }
 
 
