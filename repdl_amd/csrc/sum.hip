@@ -211,21 +211,32 @@ __global__ __launch_bounds__(RT) void rowchain_kernel(const float *__restrict__ 
 // fewer when columns are scarce so that the CUs still get several workgroups each)
 // and moves down in tiles of (RTILE / CW) rows x CW columns = 32 KiB.  All waves
 // stream the next tile into registers (16-byte non-temporal loads; a row of the
-// tile is CW*4 contiguous bytes) while one wave walks the current tile in LDS,
-// lane = column, one ds_read_b32 and one dependent v_add_f32 per row.
+// tile is CW*4 contiguous bytes) and store it transposed, [column][row], while one wave
+// walks the current tile in LDS, lane = column, one ds_read_b128 and four dependent
+// v_add_f32 per four rows (a ds_read_b32 per row cost 14 clocks per row, this 9).
 // ---------------------------------------------------------------------------
 template <int CW, bool VEC>
-__global__ __launch_bounds__(256) void coltile_kernel(const float *__restrict__ in, float *__restrict__ out,
+__global__ __launch_bounds__(320) void coltile_kernel(const float *__restrict__ in, float *__restrict__ out,
                                                       int64_t M, int64_t N, float factor)
 {
     constexpr int TR = RTILE / CW;      // rows per tile
     constexpr int C4 = CW / 4;          // float4 per tile row
     constexpr int RV = RTILE / 4 / 256; // float4 per thread and tile
-    __shared__ __attribute__((aligned(16))) float tile[RTILE];
+    constexpr int TRP = TR + 4;         // LDS words per column (the pad spreads the walk's 16-byte reads over the banks)
+    __shared__ __attribute__((aligned(16))) float tile[CW * TRP]; // [column][row]: the walk reads four rows at once
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int walker = blockIdx.x % 4;
-    const int64_t col0 = (int64_t)blockIdx.x * CW;
+    constexpr int walker = 4; // waves 0-3 move the tiles, wave 4 only walks (as a mover too it walked 12.6 clocks per row)
+    // Which columns?  With 16 columns a row of the tile is half a 128-byte line, and the
+    // workgroup that takes the other half should sit behind the same L2 or the line comes
+    // from memory twice.  Workgroups go to the 8 XCDs round-robin by id, so inside every whole
+    // group of 16 ids, ids b and b + 8 (same XCD, dispatched back to back) take the two halves
+    // of one line; the loads then keep the default cache policy instead of the streaming one.
+    constexpr bool HALF_LINE = CW == 16;
+    int64_t cg = blockIdx.x;
+    if (HALF_LINE && (cg | 15) < (int64_t)gridDim.x)
+        cg = (cg & ~(int64_t)15) + ((cg & 7) << 1) + ((cg >> 3) & 1);
+    const int64_t col0 = cg * CW;
     const int64_t ntiles = (M + TR - 1) / TR;
 
     float acc = 0.0f;
@@ -242,7 +253,8 @@ __global__ __launch_bounds__(256) void coltile_kernel(const float *__restrict__ 
             {
                 const float *p = in + r * N + c;
                 if (VEC && c + 3 < N)
-                    v = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(p));
+                    v = HALF_LINE ? *reinterpret_cast<const v4f *>(p)
+                                  : __builtin_nontemporal_load(reinterpret_cast<const v4f *>(p));
                 else
                 {
                     if (c + 0 < N) v.x = p[0];
@@ -257,10 +269,18 @@ __global__ __launch_bounds__(256) void coltile_kernel(const float *__restrict__ 
     auto store = [&]() {
 #pragma unroll
         for (int i = 0; i < RV; i++)
-            *reinterpret_cast<v4f *>(&tile[(tid + 256 * i) << 2]) = stage[i]; // [row][column], CW floats per row
+        {
+            const int idx = tid + 256 * i;
+            float *q = &tile[((idx % C4) << 2) * TRP + idx / C4]; // transposed on the way in
+            q[0 * TRP] = stage[i].x;
+            q[1 * TRP] = stage[i].y;
+            q[2 * TRP] = stage[i].z;
+            q[3 * TRP] = stage[i].w;
+        }
     };
 
-    if (ntiles > 0)
+    const bool mover = wave < 4;
+    if (ntiles > 0 && mover)
     {
         load(0);
         store();
@@ -269,45 +289,57 @@ __global__ __launch_bounds__(256) void coltile_kernel(const float *__restrict__ 
     for (int64_t t = 0; t < ntiles; t++)
     {
         const bool more = t + 1 < ntiles;
-        if (more)
+        if (more && mover)
             load(t + 1);
         if (wave == walker && lane < CW)
         {
             const int64_t rem = M - t * TR; // rows of this tile that exist; the rest must not be added
-            const float *colp = &tile[lane];
+            const float *colp = &tile[lane * TRP];
             if (rem >= TR)
             {
-                float va[16], vb[16];
+                // 16 rows ahead: the reads of the next 16 are issued before the adds of these
+                const v4f *cp = reinterpret_cast<const v4f *>(colp);
+                v4f va[4], vb[4];
 #pragma unroll
-                for (int u = 0; u < 16; u++)
-                    va[u] = colp[u * CW];
+                for (int u = 0; u < 4; u++)
+                    va[u] = cp[u];
                 for (int r = 0; r < TR; r += 32)
                 {
 #pragma unroll
-                    for (int u = 0; u < 16; u++)
-                        vb[u] = colp[(r + 16 + u) * CW];
+                    for (int u = 0; u < 4; u++)
+                        vb[u] = cp[(r + 16) / 4 + u];
 #pragma unroll
-                    for (int u = 0; u < 16; u++)
-                        acc = acc + va[u];
+                    for (int u = 0; u < 4; u++)
+                    {
+                        acc = acc + va[u].x;
+                        acc = acc + va[u].y;
+                        acc = acc + va[u].z;
+                        acc = acc + va[u].w;
+                    }
                     if (r + 32 < TR)
                     {
 #pragma unroll
-                        for (int u = 0; u < 16; u++)
-                            va[u] = colp[(r + 32 + u) * CW];
+                        for (int u = 0; u < 4; u++)
+                            va[u] = cp[(r + 32) / 4 + u];
                     }
 #pragma unroll
-                    for (int u = 0; u < 16; u++)
-                        acc = acc + vb[u];
+                    for (int u = 0; u < 4; u++)
+                    {
+                        acc = acc + vb[u].x;
+                        acc = acc + vb[u].y;
+                        acc = acc + vb[u].z;
+                        acc = acc + vb[u].w;
+                    }
                 }
             }
             else
             {
                 for (int r = 0; r < (int)rem; r++)
-                    acc = acc + colp[r * CW];
+                    acc = acc + colp[r];
             }
         }
         __syncthreads(); // the walk of tile t is over: the buffer may be overwritten
-        if (more)
+        if (more && mover)
             store();
         __syncthreads();
     }
@@ -437,9 +469,9 @@ REPDL_API int repdl_hip_sum2d_dim0(const float *in, float *out, int64_t M, int64
     do                                                                                                  \
     {                                                                                                   \
         if (vec)                                                                                        \
-            hipLaunchKernelGGL((coltile_kernel<CWv, true>), g, dim3(256), 0, st, in, out, M, N, factor); \
+            hipLaunchKernelGGL((coltile_kernel<CWv, true>), g, dim3(320), 0, st, in, out, M, N, factor); \
         else                                                                                            \
-            hipLaunchKernelGGL((coltile_kernel<CWv, false>), g, dim3(256), 0, st, in, out, M, N, factor); \
+            hipLaunchKernelGGL((coltile_kernel<CWv, false>), g, dim3(320), 0, st, in, out, M, N, factor); \
     } while (0)
     if (cw == 64)
         REPDL_COLTILE(64);
