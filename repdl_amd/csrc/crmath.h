@@ -129,6 +129,15 @@ typedef struct
     const float *logc_lo;
 } crm_log_tables;
 
+// the same tables with invc and logc_lo widened to binary64 (exact), for kernels that fill their
+// own copy once per workgroup
+typedef struct
+{
+    const double *invc;
+    const double *logc_hi;
+    const double *logc_lo;
+} crm_log_tables_wide;
+
 typedef struct
 {
     double db, y;
@@ -236,17 +245,21 @@ CRM_FN float crm_exp(float x, const uint64_t *tab)
 // log(x) = k ln2 + logc + log1p(r), summed as an exact head
 // w = k*LN2_HI + logc_hi, a compensated hi + lo, and a degree-9 polynomial.
 // Tables (crmath_tables.h): invc[128] binary32, logc_hi[128] binary64, logc_lo[128] binary32.
-CRM_FN double crm_log64_core(double x, crm_log_tables tab)
+// (index, exponent and reduced argument of x; the table entry is fetched by the caller)
+CRM_FN double crm_log64_reduce(double x, uint32_t *idx, int32_t *kexp)
 {
     const uint64_t ix = crm_d2u(x);
     // only the high word takes part in the reduction (the offset has a zero low word)
     const uint32_t hi = (uint32_t)(ix >> 32);
     const uint32_t tmp = hi - 0x3FE60000u;
-    const uint32_t i = (tmp >> 13) & 127u;
-    const int32_t k = (int32_t)tmp >> 20;
+    *idx = (tmp >> 13) & 127u;
+    *kexp = (int32_t)tmp >> 20;
     const uint32_t zhi = hi - (tmp & 0xFFF00000u);
-    const double z = crm_u2d(((uint64_t)zhi << 32) | (ix & 0xFFFFFFFFu));
-    const double invc = (double)tab.invc[i], logc_hi = tab.logc_hi[i], logc_lo = (double)tab.logc_lo[i];
+    return crm_u2d(((uint64_t)zhi << 32) | (ix & 0xFFFFFFFFu));
+}
+
+CRM_FN double crm_log64_eval(double z, int32_t k, double invc, double logc_hi, double logc_lo)
+{
     const double kd = (double)k;
     const double r = crm_fma(z, invc, -1.0);
     const double w = crm_fma(kd, CRM_LN2_HI, logc_hi); // exact
@@ -264,16 +277,43 @@ CRM_FN double crm_log64_core(double x, crm_log_tables tab)
     return hi_sum + crm_fma(r2, p, lo);
 }
 
-CRM_FN float crm_log(float x, crm_log_tables tab)
+CRM_FN double crm_log64_core(double x, crm_log_tables tab)
+{
+    uint32_t i;
+    int32_t k;
+    const double z = crm_log64_reduce(x, &i, &k);
+    return crm_log64_eval(z, k, (double)tab.invc[i], tab.logc_hi[i], (double)tab.logc_lo[i]);
+}
+
+// the same with the two binary32 tables widened beforehand (two conversions less per element)
+CRM_FN double crm_log64_core_wide(double x, crm_log_tables_wide tab)
+{
+    uint32_t i;
+    int32_t k;
+    const double z = crm_log64_reduce(x, &i, &k);
+    return crm_log64_eval(z, k, tab.invc[i], tab.logc_hi[i], tab.logc_lo[i]);
+}
+
+// the special inputs of log in three selects: x + x is +inf for +inf and, for a NaN, the same
+// NaN quieted (sign and payload kept); a NaN compares false both times
+CRM_FN float crm_log_finish(float x, double core)
 {
     const uint32_t ux = crm_f2u(x);
-    // zeros, negatives, infinities and NaNs run through the core harmlessly (the
-    // table index is masked) and are overridden
-    const uint32_t gen = crm_f2u(crm_d2f(crm_log64_core((double)x, tab)));
-    // the special inputs in three selects: x + x is +inf for +inf and, for a NaN, the same
-    // NaN quieted (sign and payload kept); a NaN compares false both times
+    const uint32_t gen = crm_f2u(crm_d2f(core));
     uint32_t sp = crm_f2u(x + x);
     sp = (x < 0.0f) ? CRM_QNAN_NEG : sp;  // log(negative), log(-inf): (x-x)/(x-x) on x86
     sp = (x == 0.0f) ? 0xFF800000u : sp;  // log(+-0) = -inf
     return crm_u2f((ux - 1u >= 0x7F7FFFFFu) ? sp : gen);
+}
+
+CRM_FN float crm_log(float x, crm_log_tables tab)
+{
+    // zeros, negatives, infinities and NaNs run through the core harmlessly (the
+    // table index is masked) and are overridden
+    return crm_log_finish(x, crm_log64_core((double)x, tab));
+}
+
+CRM_FN float crm_log_wide(float x, crm_log_tables_wide tab)
+{
+    return crm_log_finish(x, crm_log64_core_wide((double)x, tab));
 }

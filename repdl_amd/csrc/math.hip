@@ -42,14 +42,14 @@ template <int OP>
 struct Ctx
 {
     const uint64_t *exp_tab;
-    crm_log_tables log_tab;
+    crm_log_tables_wide log_tab;
     crm_divisor divisor;
     __device__ __forceinline__ float apply(float x) const
     {
         if (OP == OP_EXP)
             return crm_exp(x, exp_tab);
         if (OP == OP_LOG)
-            return crm_log(x, log_tab);
+            return crm_log_wide(x, log_tab);
         if (OP == OP_SQRT)
             return crm_sqrt(x);
         return crm_div_by(x, divisor);
@@ -70,12 +70,12 @@ __global__ __launch_bounds__(EW_THREADS) void unary_kernel(const float *__restri
                                                            float *__restrict__ out, int64_t n,
                                                            float scalar, int vec_ok)
 {
-    // exp: 256 words (tail, sbits pairs); log: logc_hi[128] then invc[128], logc_lo[128] as floats
-    __shared__ __attribute__((aligned(16))) uint64_t tab[256];
+    // exp: 256 words (tail, sbits pairs); log: logc_hi[128], invc[128], logc_lo[128], all binary64
+    __shared__ __attribute__((aligned(16))) uint64_t tab[OP == OP_LOG ? 384 : 256];
     Ctx<OP> ctx;
     ctx.exp_tab = tab;
     double *lhi = reinterpret_cast<double *>(tab);
-    float *linvc = reinterpret_cast<float *>(tab + 128), *llo = linvc + 128;
+    double *linvc = lhi + 128, *llo = lhi + (OP == OP_LOG ? 256 : 128);
     ctx.log_tab.invc = linvc;
     ctx.log_tab.logc_hi = lhi;
     ctx.log_tab.logc_lo = llo;
@@ -108,8 +108,8 @@ __global__ __launch_bounds__(EW_THREADS) void unary_kernel(const float *__restri
         if (threadIdx.x < 128)
         {
             lhi[threadIdx.x] = g_log_hi[threadIdx.x];
-            linvc[threadIdx.x] = g_log_invc[threadIdx.x];
-            llo[threadIdx.x] = g_log_lo[threadIdx.x];
+            linvc[threadIdx.x] = (double)g_log_invc[threadIdx.x];
+            llo[threadIdx.x] = (double)g_log_lo[threadIdx.x];
         }
         __syncthreads();
     }
