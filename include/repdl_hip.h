@@ -49,17 +49,30 @@ int repdl_hip_abi_version(void);
  * mm and the three convolutions have two implementations of the same chains: one on
  * the binary32 matrix instructions of gfx950 (v_mfma_f32_32x32x2_f32 /
  * v_mfma_f32_16x16x4_f32) and one on v_fma_f32.  The matrix instructions are used
- * only after a check on the device itself has found them bit-identical to chains of
- * single-rounding FMAs, k ascending (the first GEMM-shaped call on a device runs
- * about a million comparisons, synchronously, once).
+ * only on a device where a check run on that device has found them bit-identical to
+ * chains of single-rounding FMAs, k ascending; no setting overrides a failed check.
+ *   repdl_hip_init: runs that check (about a million comparisons) for the current
+ *     device, once, and waits for it.  It works on a stream of its own, created
+ *     non-blocking at the default priority, with memory from the stream-ordered
+ *     allocator: it neither waits for nor delays the null stream or any stream of the
+ *     caller.  Returns 0 when the check could run, whatever its verdict.  Call it at
+ *     start-up, outside any stream capture.
+ *   First-call behaviour without repdl_hip_init: the first GEMM-shaped call on a device
+ *     runs the same check in the same way (the calling thread waits about 0.2 ms; the
+ *     caller's stream is not touched).  If the check cannot run at that moment -- the
+ *     thread is capturing a graph, say -- that call takes the v_fma_f32 kernels (same
+ *     bits, slower) and the check is tried again at the next call.
  *   repdl_hip_mfma_selftest: runs waves*trials further comparisons of each
  *     instruction (operand classes cycle with the trial number) and writes the
  *     number of differing results to mismatches[0] (32x32x2) and mismatches[1]
- *     (16x16x4), HOST memory.  Synchronous.
- *   repdl_hip_set_matrix_path: -1 = decide by the check (default), 0 = always the
- *     v_fma_f32 kernels, 1 = always the matrix kernels.  Process-wide.
+ *     (16x16x4), HOST memory.  Synchronous, on a stream of its own.
+ *   repdl_hip_set_matrix_path: 0 = always the v_fma_f32 kernels; -1 (default) and 1 =
+ *     the matrix kernels wherever the check has passed.  Mode 1 also runs the check for
+ *     the current device and returns REPDL_E_UNSUPPORTED, changing nothing, if it did
+ *     not pass there.  Process-wide.
  *   repdl_hip_matrix_path: 1 if GEMM-shaped calls on the current device now take the
  *     matrix kernels, else 0 (runs the check if it has not run yet). */
+int repdl_hip_init(void);
 int repdl_hip_mfma_selftest(int64_t waves, int64_t trials, uint64_t seed, uint64_t *mismatches);
 int repdl_hip_set_matrix_path(int mode);
 int repdl_hip_matrix_path(void);

@@ -89,6 +89,12 @@ def lib() -> ctypes.CDLL:
         handle.repdl_hip_matrix_path.restype = _INT
         handle.repdl_hip_abi_version.argtypes = []
         handle.repdl_hip_abi_version.restype = _INT
+        handle.repdl_hip_init.argtypes = []
+        handle.repdl_hip_init.restype = _INT
+        # The one-time check of the matrix instructions, here rather than inside the first
+        # operator call.  Without a GPU it reports an error, which only matters to callers
+        # that go on to compute (they fail at their first launch).
+        handle.repdl_hip_init()
         _lib = handle
     return _lib
 

@@ -334,6 +334,9 @@ torch::Tensor bn_gweight_term(const torch::Tensor &input, const torch::Tensor &m
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {
     namespace h = repdl::hip;
+    // the one-time check of the matrix instructions, at import instead of inside the first
+    // GEMM-shaped call (an error here -- no device yet -- leaves it to that call)
+    (void)repdl_hip_init();
     m.def("conv2d", &h::conv2d);
     m.def("conv2d_grad_input", &h::conv2d_grad_input);
     m.def("conv2d_grad_kernel", &h::conv2d_grad_kernel);

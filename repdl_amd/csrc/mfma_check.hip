@@ -11,10 +11,11 @@
 // below compare both instructions with __fmaf_rn chains on operands drawn from
 // seven classes (ordinary, any finite, products in the subnormal range, short
 // significands that produce exact ties, overflow, exact cancellation, and a mix
-// of +-0, +-inf, subnormals and extremes).  The first use of a matrix kernel on a
-// device runs a short version of the check; if a single result differs, every
-// GEMM-shaped operator stays on its v_fma_f32 kernel.  repdl_hip_mfma_selftest
-// runs a check of any length on request.
+// of +-0, +-inf, subnormals and extremes).  repdl_hip_init() -- or, failing that, the
+// first use of a matrix kernel on a device -- runs a short version of the check on a
+// stream of its own; if a single result differs, every GEMM-shaped operator stays on
+// its v_fma_f32 kernel, and no setting overrides that.  repdl_hip_mfma_selftest runs a
+// check of any length on request.
 #include <mutex>
 
 #include "common.h"
@@ -155,49 +156,92 @@ __global__ __launch_bounds__(64) void mfma_check_kernel(unsigned long long *coun
         atomicAdd(&counts[1], bad16);
 }
 
+// Runs the comparison on a stream of its own (non-blocking: it neither waits for nor holds up
+// the null stream or the caller's stream), with memory from the stream-ordered allocator, and
+// waits for that stream only.
 int run_check(int64_t blocks, int64_t trials, uint64_t seed, unsigned long long out[2])
 {
-    unsigned long long *d = nullptr;
-    hipError_t e = hipMalloc(&d, 2 * sizeof(unsigned long long));
+    hipStream_t st = nullptr;
+    hipError_t e = hipStreamCreateWithFlags(&st, hipStreamNonBlocking);
     if (e != hipSuccess)
         return (int)e;
-    e = hipMemset(d, 0, 2 * sizeof(unsigned long long));
+    unsigned long long *d = nullptr;
+    e = hipMallocAsync(reinterpret_cast<void **>(&d), 2 * sizeof(unsigned long long), st);
     if (e == hipSuccess)
     {
-        hipLaunchKernelGGL(mfma_check_kernel, dim3((unsigned)blocks), dim3(64), 0, 0, d, (int)trials, seed);
-        e = hipGetLastError();
+        e = hipMemsetAsync(d, 0, 2 * sizeof(unsigned long long), st);
+        if (e == hipSuccess)
+        {
+            hipLaunchKernelGGL(mfma_check_kernel, dim3((unsigned)blocks), dim3(64), 0, st, d, (int)trials, seed);
+            e = hipGetLastError();
+        }
+        if (e == hipSuccess)
+            e = hipMemcpyAsync(out, d, 2 * sizeof(unsigned long long), hipMemcpyDeviceToHost, st);
+        const hipError_t e2 = hipFreeAsync(d, st);
+        if (e == hipSuccess)
+            e = e2;
+        const hipError_t e3 = hipStreamSynchronize(st);
+        if (e == hipSuccess)
+            e = e3;
     }
-    if (e == hipSuccess)
-        e = hipMemcpy(out, d, 2 * sizeof(unsigned long long), hipMemcpyDeviceToHost);
-    hipError_t e2 = hipFree(d);
-    if (e == hipSuccess)
-        e = e2;
+    (void)hipStreamDestroy(st);
     return e == hipSuccess ? REPDL_OK : (int)e;
 }
 
 constexpr int MAX_DEVICES = 64;
 std::mutex g_lock;
-int g_mode = -1;                 // -1 = decide by the check, 0 = never, 1 = always
-int g_verdict[MAX_DEVICES] = {}; // 0 = not checked yet, 1 = exact, 2 = not exact / check failed
+int g_mode = -1;                 // -1 = the matrix kernels where the check passed, 0 = never, 1 = as -1 (see set_matrix_path)
+int g_verdict[MAX_DEVICES] = {}; // 0 = not checked yet, 1 = exact, 2 = not exact
+
+// Verdict of the current device, running the check if it has not run there yet (g_lock held).
+// A check that could not run (no device, or a runtime error such as a stream capture in
+// progress on this thread) leaves the verdict open: the caller then takes the v_fma_f32
+// kernels for this call and the check is tried again at the next one.
+int device_verdict(int *rc_out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES)
+    {
+        if (rc_out)
+            *rc_out = e != hipSuccess ? (int)e : REPDL_E_UNSUPPORTED;
+        return 0;
+    }
+    if (g_verdict[dev] == 0)
+    {
+        unsigned long long bad[2] = {1, 1};
+        // 512 waves x 28 trials x (1024 + 256) results: four trials of every class per wave
+        const int rc = run_check(512, 4 * NCLASS, 0x52657044 /* any fixed seed */, bad);
+        if (rc_out)
+            *rc_out = rc;
+        if (rc != REPDL_OK)
+        {
+            (void)hipGetLastError(); // the failed check must not surface in the caller's next launch check
+            return 0;
+        }
+        g_verdict[dev] = (bad[0] == 0 && bad[1] == 0) ? 1 : 2;
+    }
+    else if (rc_out)
+        *rc_out = REPDL_OK;
+    return g_verdict[dev];
+}
 } // namespace
 
 // Whether the GEMM-shaped operators may use the matrix instructions on the current device.
 bool repdl_mfma_exact()
 {
     std::lock_guard<std::mutex> guard(g_lock);
-    if (g_mode >= 0)
-        return g_mode == 1;
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES)
+    if (g_mode == 0)
         return false;
-    if (g_verdict[dev] == 0)
-    {
-        unsigned long long bad[2] = {1, 1};
-        // 512 waves x 28 trials x (1024 + 256) results: four trials of every class per wave
-        const int rc = run_check(512, 4 * NCLASS, 0x52657044 /* any fixed seed */, bad);
-        g_verdict[dev] = (rc == REPDL_OK && bad[0] == 0 && bad[1] == 0) ? 1 : 2;
-    }
-    return g_verdict[dev] == 1;
+    return device_verdict(nullptr) == 1;
+}
+
+REPDL_API int repdl_hip_init(void)
+{
+    std::lock_guard<std::mutex> guard(g_lock);
+    int rc = REPDL_OK;
+    (void)device_verdict(&rc);
+    return rc;
 }
 
 REPDL_API int repdl_hip_mfma_selftest(int64_t waves, int64_t trials, uint64_t seed, uint64_t *mismatches)
@@ -214,6 +258,14 @@ REPDL_API int repdl_hip_set_matrix_path(int mode)
 {
     REPDL_REQUIRE(mode >= -1 && mode <= 1);
     std::lock_guard<std::mutex> guard(g_lock);
+    if (mode == 1)
+    {
+        // asking for the matrix kernels never bypasses the check: refused where it did not pass
+        int rc = REPDL_OK;
+        const int v = device_verdict(&rc);
+        if (v != 1)
+            return rc != REPDL_OK ? rc : REPDL_E_UNSUPPORTED;
+    }
     g_mode = mode;
     return REPDL_OK;
 }

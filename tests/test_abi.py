@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), n
     other = {"repdl_hip_error_string", "repdl_hip_abi_version", "repdl_hip_sum1d_workspace_bytes",
-             "repdl_hip_matrix_path"}
+             "repdl_hip_matrix_path", "repdl_hip_init"}
     assert set(_lib.SIGNATURES) | other == set(names)
 
 

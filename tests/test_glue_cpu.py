@@ -180,3 +180,28 @@ def test_adam_resumes_from_a_state_dict_with_the_same_bits(amsgrad):
         o3.load_state_dict(o2.state_dict())
         models.train_steps(m2, repdl_amd.nn.CrossEntropyLoss(), o3, x, y, 2)
     assert repdl_amd.utils.get_hash(m1) == repdl_amd.utils.get_hash(m2)
+
+
+def test_readme_initial_model_hash():
+    """The one known answer the reference holds for the glue: README.md:36, the SHA-256 of the
+    LeNet-5 of examples/mnist_trainig.py:12-33 built under torch.manual_seed(0) (:106-108),
+    converted by from_torch_module and hashed by utils.get_hash (parameters in order)."""
+
+    class TorchModel(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.net = torch.nn.Sequential(
+                torch.nn.Conv2d(1, 6, kernel_size=5, padding=2), torch.nn.ReLU(), torch.nn.MaxPool2d(kernel_size=2, stride=2),
+                torch.nn.Conv2d(6, 16, kernel_size=5), torch.nn.ReLU(), torch.nn.MaxPool2d(kernel_size=2, stride=2),
+                torch.nn.Flatten(), torch.nn.Linear(16 * 5 * 5, 120), torch.nn.ReLU(), torch.nn.Linear(120, 84),
+                torch.nn.ReLU(), torch.nn.Linear(84, 10))
+
+        def forward(self, x):
+            return self.net(x)
+
+    torch.manual_seed(0)
+    model = repdl_amd.from_torch_module(TorchModel())
+    assert repdl_amd.utils.get_hash(model) == "2a2d133895b1684e55d0f152ead2914b55adc551d9790a4b4585309b79c60362"
+    kinds = [type(m).__name__ for m in model.net]
+    assert kinds.count("Conv2d") == 2 and kinds.count("Linear") == 3
+    assert all(type(m).__module__.startswith("repdl_amd") for m in model.net if type(m).__name__ in ("Conv2d", "Linear"))

@@ -164,3 +164,23 @@ def test_channel_sums_few_long_chains(shape):
     xd = flat[1:].view(*shape)  # 4 bytes off a 16-byte boundary
     assert xd.data_ptr() % 16 != 0
     assert torch.equal(ops.sum4d_dim023(xd).cpu(), oracle.sum4d_dim023(x))
+
+
+def test_full_size_benchmark_inputs():
+    """The two inputs of the sum configuration at their full sizes: 2^28 uniform multiples of
+    2^-23 in [-1, 1) through sum1d, and row sums of a 16384 x 16384 matrix of N(0,1) values
+    scaled by 2^U[-20,20]; every output bit against the oracle."""
+    from repdl_amd import ops
+
+    x = gen.uniform_pm1(2028, 1 << 28)
+    for avg in (False, True):
+        got = ops.sum1d(x.cuda(), avg).cpu()
+        assert got.view(torch.int32).item() == oracle.sum1d(x, avg).view(torch.int32).item(), avg
+    # a drifting input of the same length: the running sum stops growing at 2^24
+    y = x.abs_()
+    assert ops.sum1d(y.cuda()).cpu().view(torch.int32).item() == oracle.sum1d(y).view(torch.int32).item()
+    del x, y
+    m = gen.scaled_normal(2029, 16384, 16384)
+    got = ops.sum2d_dim1(m.cuda()).cpu()
+    assert torch.equal(got.view(torch.int32), oracle.sum2d_dim1(m).view(torch.int32))
+    assert torch.equal(ops.sum2d_dim0(m.cuda()).cpu().view(torch.int32), oracle.sum2d_dim0(m).view(torch.int32))
