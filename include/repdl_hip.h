@@ -40,6 +40,7 @@ extern "C" {
 #define REPDL_E_ARG (-1)         /* null pointer, negative size, size out of range */
 #define REPDL_E_UNSUPPORTED (-2) /* a combination the reference itself does not define */
 #define REPDL_E_WORKSPACE (-3)   /* workspace missing or too small */
+#define REPDL_E_TOO_LARGE (-4)   /* input beyond the fixed capacity of an entry point that allocates nothing */
 
 const char *repdl_hip_error_string(int code);
 int repdl_hip_abi_version(void);
@@ -149,6 +150,16 @@ int repdl_hip_sum1d(const float *in, float *out, int64_t n, int average, void *s
 size_t repdl_hip_sum1d_workspace_bytes(int64_t n);
 int repdl_hip_sum1d_ws(const float *in, float *out, int64_t n, int average, void *workspace,
                        size_t workspace_bytes, void *stream);
+/* sum1d for callers that cannot allocate (code under graph capture, serving loops, harnesses
+ * that forbid hipMalloc).  No counterpart in the reference.  Same result as repdl_hip_sum1d, bit
+ * for bit, but the scratch memory of the parallel evaluation is a fixed 8 MiB array inside the
+ * library (one per device, held until the process ends) instead of an allocation: the call
+ * makes no hipMalloc / hipFree / stream-ordered allocation.  n may not exceed
+ * repdl_hip_sum1d_static_max_n() (about 16 million elements; REPDL_E_TOO_LARGE beyond).  All
+ * calls on one device share that array: calls that overlap in time on one device (two
+ * streams, two threads) race and must be serialised by the caller. */
+int64_t repdl_hip_sum1d_static_max_n(void);
+int repdl_hip_sum1d_static(const float *in, float *out, int64_t n, int average, void *stream);
 int repdl_hip_sum2d_dim0(const float *in, float *out, int64_t M, int64_t N, int average,
                          void *stream);
 /* sum2d_dim1 and sum4d_dim023 with few long chains (at most 512 chains of at least 49152

@@ -42,6 +42,7 @@ SIGNATURES = {
     "repdl_hip_conv2d_grad_kernel": [_P, _P, _P] + [_I64] * 13 + [_P],
     "repdl_hip_sum1d": [_P, _P, _I64, _INT, _P],
     "repdl_hip_sum1d_ws": [_P, _P, _I64, _INT, _P, ctypes.c_size_t, _P],
+    "repdl_hip_sum1d_static": [_P, _P, _I64, _INT, _P],
     "repdl_hip_sum2d_dim0": [_P, _P, _I64, _I64, _INT, _P],
     "repdl_hip_sum2d_dim1": [_P, _P, _I64, _I64, _INT, _P],
     "repdl_hip_sum4d_dim023": [_P, _P, _I64, _I64, _I64, _I64, _INT, _P],
@@ -89,6 +90,8 @@ def lib() -> ctypes.CDLL:
         handle.repdl_hip_matrix_path.restype = _INT
         handle.repdl_hip_abi_version.argtypes = []
         handle.repdl_hip_abi_version.restype = _INT
+        handle.repdl_hip_sum1d_static_max_n.argtypes = []
+        handle.repdl_hip_sum1d_static_max_n.restype = _I64
         handle.repdl_hip_init.argtypes = []
         handle.repdl_hip_init.restype = _INT
         # The one-time check of the matrix instructions, here rather than inside the first

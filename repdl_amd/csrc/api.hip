@@ -15,6 +15,8 @@ REPDL_API const char *repdl_hip_error_string(int code)
         return "repdl_hip: unsupported combination of arguments";
     case REPDL_E_WORKSPACE:
         return "repdl_hip: workspace missing or too small";
+    case REPDL_E_TOO_LARGE:
+        return "repdl_hip: input exceeds the fixed capacity of this entry point (it allocates nothing; see its *_max_n)";
     default:
         break;
     }

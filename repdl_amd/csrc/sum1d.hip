@@ -33,6 +33,8 @@
 // every applied map is checked against the true state, so the result is the sequential
 // sum bit for bit for every input (NaN, infinities, zeros and subnormal states simply
 // fall through to the replay).
+#include <mutex>
+
 #include "common.h"
 
 namespace
@@ -750,4 +752,66 @@ REPDL_API int repdl_hip_sum1d(const float *in, float *out, int64_t n, int averag
     if (rc != REPDL_OK)
         return rc;
     return e == hipSuccess ? REPDL_OK : (int)e;
+}
+
+// ---- sum1d for callers that cannot allocate ---------------------------------------------------
+// The scratch memory of the parallel evaluation in a file-scope device array instead of an
+// allocation: every device the library runs on holds its own copy of the array until the process
+// ends.  In host code the array's name is only a handle for hipGetSymbolAddress; the address
+// the kernels get is looked up once per device, with that device current.
+namespace
+{
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)8 << 20;
+__device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+constexpr int STATIC_MAX_DEVICES = 64;
+std::mutex g_static_lock;
+void *g_static_ptr[STATIC_MAX_DEVICES] = {};
+
+// largest n whose scratch fits (the need grows monotonically with n)
+int64_t static_max_n()
+{
+    int64_t lo = REPDL_SUM1D_MIN_PARALLEL, hi = (int64_t)STATIC_SCRATCH_BYTES * 8;
+    while (lo < hi)
+    {
+        const int64_t mid = lo + (hi - lo + 1) / 2;
+        if (repdl_sum_chains_workspace_bytes(1, mid) <= STATIC_SCRATCH_BYTES)
+            lo = mid;
+        else
+            hi = mid - 1;
+    }
+    return lo;
+}
+} // namespace
+
+REPDL_API int64_t repdl_hip_sum1d_static_max_n(void)
+{
+    static const int64_t n = static_max_n();
+    return n;
+}
+
+REPDL_API int repdl_hip_sum1d_static(const float *in, float *out, int64_t n, int average, void *stream)
+{
+    REPDL_REQUIRE(n >= 0 && out != nullptr && (n == 0 || in != nullptr));
+    if (n < REPDL_SUM1D_MIN_PARALLEL)
+        return repdl_sum1d_serial(in, out, n, average, stream); // uses no scratch memory
+    if (n > repdl_hip_sum1d_static_max_n())
+        return REPDL_E_TOO_LARGE;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess)
+        return (int)e;
+    REPDL_REQUIRE(dev >= 0 && dev < STATIC_MAX_DEVICES);
+    void *ptr = nullptr;
+    {
+        std::lock_guard<std::mutex> guard(g_static_lock);
+        if (g_static_ptr[dev] == nullptr)
+        {
+            e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+            if (e != hipSuccess)
+                return (int)e;
+            g_static_ptr[dev] = ptr;
+        }
+        ptr = g_static_ptr[dev];
+    }
+    return repdl_hip_sum1d_ws(in, out, n, average, ptr, STATIC_SCRATCH_BYTES, stream);
 }

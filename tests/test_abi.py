@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), n
     other = {"repdl_hip_error_string", "repdl_hip_abi_version", "repdl_hip_sum1d_workspace_bytes",
-             "repdl_hip_matrix_path", "repdl_hip_init"}
+             "repdl_hip_matrix_path", "repdl_hip_init", "repdl_hip_sum1d_static_max_n"}
     assert set(_lib.SIGNATURES) | other == set(names)
 
 
@@ -36,6 +36,7 @@ def test_abi_version_and_error_strings():
     assert lib.repdl_hip_error_string(0) == b"success"
     assert b"invalid argument" in lib.repdl_hip_error_string(-1)
     assert b"workspace" in lib.repdl_hip_error_string(-3)
+    assert b"capacity" in lib.repdl_hip_error_string(-4)
 
 
 def test_bad_arguments_are_rejected_on_the_host():
