@@ -144,9 +144,9 @@ int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float *input, f
 int repdl_hip_sum1d(const float *in, float *out, int64_t n, int average, void *stream);
 /* sum1d with caller-provided scratch memory (same result).  Long inputs are evaluated in
  * parallel -- exactly: the result is the sequential chain's, bit for bit -- which needs
- * repdl_hip_sum1d_workspace_bytes(n) bytes of 16-byte aligned device memory (about n/2
- * bytes; 0 for short inputs).  repdl_hip_sum1d itself takes that memory from the
- * stream-ordered allocator (hipMallocAsync / hipFreeAsync on `stream`). */
+ * repdl_hip_sum1d_workspace_bytes(n) bytes of 16-byte aligned device memory (about 5n/8
+ * bytes; 0 for short inputs).  The memory may hold anything on entry.  repdl_hip_sum1d itself
+ * takes it from the stream-ordered allocator (hipMallocAsync / hipFreeAsync on `stream`). */
 size_t repdl_hip_sum1d_workspace_bytes(int64_t n);
 int repdl_hip_sum1d_ws(const float *in, float *out, int64_t n, int average, void *workspace,
                        size_t workspace_bytes, void *stream);
@@ -155,7 +155,7 @@ int repdl_hip_sum1d_ws(const float *in, float *out, int64_t n, int average, void
  * for bit, but the scratch memory of the parallel evaluation is a fixed 8 MiB array inside the
  * library (one per device, held until the process ends) instead of an allocation: the call
  * makes no hipMalloc / hipFree / stream-ordered allocation.  n may not exceed
- * repdl_hip_sum1d_static_max_n() (about 16 million elements; REPDL_E_TOO_LARGE beyond).  All
+ * repdl_hip_sum1d_static_max_n() (about 13 million elements; REPDL_E_TOO_LARGE beyond).  All
  * calls on one device share that array: calls that overlap in time on one device (two
  * streams, two threads) race and must be serialised by the caller. */
 int64_t repdl_hip_sum1d_static_max_n(void);

@@ -39,13 +39,19 @@ def sources() -> list[str]:
     return sorted(glob(os.path.join(CSRC, "*.hip")))
 
 
-def build(verbose: bool = False) -> str:
+def build(verbose: bool = False, incremental: bool = False, extra_flags: tuple = ()) -> str:
+    """Compiles every source (incremental=True: only those newer than their object, or older
+    than a header) and links the library."""
     os.makedirs(OBJ, exist_ok=True)
     jobs, objs = [], []
+    headers = glob(os.path.join(CSRC, "*.h")) + glob(os.path.join(HERE, "..", "include", "*.h"))
+    newest_header = max(os.path.getmtime(h) for h in headers)
     for src in sources():
         obj = os.path.join(OBJ, os.path.basename(src)[:-4] + ".o")
         objs.append(obj)
-        jobs.append([HIPCC] + FLAGS + ["-c", src, "-o", obj])
+        if incremental and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), newest_header):
+            continue
+        jobs.append([HIPCC] + FLAGS + list(extra_flags) + ["-c", src, "-o", obj])
     with ThreadPoolExecutor(max_workers=6) as ex:
         list(ex.map(_run, jobs))
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
@@ -88,6 +94,6 @@ def build_ext(verbose: bool = False) -> str:
 
 
 if __name__ == "__main__":
-    build(verbose=True)
+    build(verbose=True, incremental="--incremental" in sys.argv)
     build_ext(verbose=True)
     sys.exit(0)

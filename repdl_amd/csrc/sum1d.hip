@@ -33,6 +33,32 @@
 // every applied map is checked against the true state, so the result is the sequential
 // sum bit for bit for every input (NaN, infinities, zeros and subnormal states simply
 // fall through to the replay).
+//
+// Long single chains: step 4 alone is one wave, and on data whose sum wanders across binade
+// boundaries (zero-mean steps) it replays tens of thousands of chunks one after the other.
+// So it is preceded by SPECULATIVE ROUNDS that do the same walk for many candidate states at
+// once, everywhere in parallel:
+//   4a. a NODE is 4 blocks.  One workgroup per node walks it exactly as step 4 would, but
+//       for 256 candidate entry states at once, one per lane: 256 consecutive binary32
+//       bit patterns around the node's predicted entry state.  A map is applied when it is
+//       valid for every lane of a wave, a chunk is replayed with real additions otherwise
+//       (the chunk's elements broadcast from LDS), so every lane ends with the exact exit
+//       state of ITS entry state: a table  candidate -> exit state.
+//   4b. the sixteen node tables of a super-block are composed: exact where each exit state is
+//       again a candidate of the next node, and otherwise an approximate offset (nearest
+//       candidate, the excess carried along).
+//   4c. one workgroup runs the true state through the super-block tables, staged through
+//       LDS, for as long as it finds the state among the candidates (every such step is
+//       exact).  At the first miss it keeps the exact state and position reached (the
+//       FRONT) and goes on with the approximate offsets: they predict the entry state of
+//       every later super-block far better than step 2 could, because they come from real
+//       trajectories that start next to the true one.  The next round builds its tables
+//       around those predictions, and so on for a fixed number of rounds (each a no-op once
+//       the front has reached the end).  On 2^28 zero-mean values the front reaches the end
+//       in four rounds.
+// Whatever the rounds leave (nothing, as a rule) step 4 walks from the front.  Only exact
+// table entries ever touch the true state, so the result is still the sequential sum for
+// every input.
 #include <mutex>
 
 #include "common.h"
@@ -46,6 +72,11 @@ constexpr int HYP_NONE = -1;      // no usable hypothesis: replay
 constexpr int HYP_ANY = 0x200;    // every element is +-0: the identity for any state
 constexpr int BIG = 1 << 26;      // "leaves the binade for sure"
 constexpr int SAT = 1 << 28;      // saturation bound of all tuple fields
+constexpr int SUP = 64;           // blocks per super-block
+constexpr int NODEB = 4;          // blocks per node (the unit of the speculative rounds)
+constexpr int NPS = SUP / NODEB;  // nodes per super-block
+constexpr int CAND = 256;         // candidate entry states per node
+constexpr int HB = 16;            // super-blocks per hyper-block (the unit the resolver steps through)
 
 struct __attribute__((aligned(16))) Tup
 {
@@ -53,7 +84,7 @@ struct __attribute__((aligned(16))) Tup
     int lo0, hi0; // over all prefixes: min of (offset + X) before rounding, max of offset after
     int lo1, hi1;
     int hyp;      // (sign << 8) | biased exponent of the state this tuple assumes, or HYP_*
-    int pad;
+    int heavy;    // chunks below this node whose map does not even hold for the predicted state (an estimate of the replays)
 };
 
 __device__ __forceinline__ int clampi(int v) { return v < -SAT ? -SAT : (v > SAT ? SAT : v); }
@@ -63,7 +94,7 @@ __device__ __forceinline__ Tup tup_identity(int hyp)
     Tup t;
     t.t0 = t.t1 = t.lo0 = t.hi0 = t.lo1 = t.hi1 = 0;
     t.hyp = hyp;
-    t.pad = 0;
+    t.heavy = 0;
     return t;
 }
 
@@ -82,7 +113,7 @@ __device__ __forceinline__ Tup tup_compose(const Tup &a, const Tup &b)
     c.lo1 = clampi(min(a.lo1, a.t1 + blo1));
     c.hi1 = clampi(max(a.hi1, a.t1 + bhi1));
     c.hyp = a.hyp;
-    c.pad = 0;
+    c.heavy = a.heavy + b.heavy;
     return c;
 }
 
@@ -141,7 +172,7 @@ __device__ __forceinline__ Tup tup_shfl_down(const Tup &t, int delta)
     r.lo1 = __shfl_down(t.lo1, delta, 64);
     r.hi1 = __shfl_down(t.hi1, delta, 64);
     r.hyp = __shfl_down(t.hyp, delta, 64);
-    r.pad = 0;
+    r.heavy = __shfl_down(t.heavy, delta, 64);
     return r;
 }
 
@@ -283,37 +314,58 @@ __global__ __launch_bounds__(256) void sum1d_blocksum_kernel(const float *__rest
         bsum[blockIdx.x] = (part[0] + part[1]) + (part[2] + part[3]);
 }
 
-// ---- step 2: exclusive prefix of the block sums (one workgroup) ---------------------------
-__global__ __launch_bounds__(256) void sum1d_prefix_kernel(const double *__restrict__ bsum,
-                                                           double *__restrict__ prefix, int64_t nblk)
+// ---- step 2: exclusive prefix of the block sums (one workgroup per row) --------------------
+// Tiles of 8192 sums: a thread owns eight consecutive ones, the workgroup scans the thread totals.
+__global__ __launch_bounds__(1024) void sum1d_prefix_kernel(const double *__restrict__ bsum,
+                                                            double *__restrict__ prefix, int64_t nblk)
 {
-    __shared__ double seg[256];
-    const int tid = threadIdx.x;
+    constexpr int PER = 8;
+    __shared__ double wsum[2][16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     bsum += (int64_t)blockIdx.x * nblk; // one workgroup per row
     prefix += (int64_t)blockIdx.x * nblk;
-    const int64_t per = (nblk + 255) / 256;
-    const int64_t b0 = tid * per, b1 = (b0 + per < nblk) ? b0 + per : nblk;
-    double s = 0.0;
-    for (int64_t b = b0; b < b1; b++)
-        s += bsum[b];
-    seg[tid] = s;
-    __syncthreads();
-    if (tid == 0)
+    double carry = 0.0;
+    int par = 0;
+    for (int64_t base = 0; base < nblk; base += PER * 1024)
     {
-        double run = 0.0;
-        for (int t = 0; t < 256; t++)
+        const int64_t i0 = base + (int64_t)tid * PER;
+        double v[PER];
+        double tot = 0.0;
+#pragma unroll
+        for (int d = 0; d < PER; d++)
         {
-            const double v = seg[t];
-            seg[t] = run;
-            run += v;
+            v[d] = i0 + d < nblk ? bsum[i0 + d] : 0.0;
+            tot += v[d];
         }
-    }
-    __syncthreads();
-    double run = seg[tid];
-    for (int64_t b = b0; b < b1; b++)
-    {
-        prefix[b] = run;
-        run += bsum[b];
+        double inc = tot;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1)
+        {
+            const double o = __shfl_up(inc, off, 64);
+            if (lane >= off)
+                inc += o;
+        }
+        if (lane == 63)
+            wsum[par][wave] = inc;
+        __syncthreads(); // (the other half of wsum is not written before everyone has passed the next barrier)
+        double before = 0.0, total = 0.0;
+#pragma unroll
+        for (int w = 0; w < 16; w++)
+        {
+            const double t = wsum[par][w];
+            before += w < wave ? t : 0.0;
+            total += t;
+        }
+        double run = carry + before + (inc - tot);
+#pragma unroll
+        for (int d = 0; d < PER; d++)
+        {
+            if (i0 + d < nblk)
+                prefix[i0 + d] = run;
+            run += v[d];
+        }
+        carry += total;
+        par ^= 1;
     }
 }
 
@@ -386,6 +438,14 @@ __global__ __launch_bounds__(256) void sum1d_tuple_kernel(const float *__restric
     // ordered reduction: 4 lanes -> chunk
     t = tup_compose(t, tup_shfl_down(t, 1));
     t = tup_compose(t, tup_shfl_down(t, 2));
+    {
+        // does the chunk's map hold for the state predicted at its start?  (counted up the tree:
+        // the speculative rounds walk the nodes with the most such chunks first)
+        const uint32_t S0 = (us & 0x7FFFFFu) | 0x800000u;
+        const int lo = (S0 & 1u) ? t.lo1 : t.lo0, hi = (S0 & 1u) ? t.hi1 : t.hi0;
+        const bool holds = hyp == HYP_ANY || (hyp >= 0 && (int)S0 + lo >= 0x800000 && (int)S0 + hi <= 0xFFFFFF);
+        t.heavy = holds ? 0 : 1;
+    }
     if ((lane & 3) == 0)
         T1[blk * (BLK / CH) + (tid >> 2)] = t;
     // 8 chunks -> group, 2 groups -> wave, 4 waves -> block (hypotheses merged on the way)
@@ -456,22 +516,60 @@ __device__ __forceinline__ bool lane_tup_apply(uint32_t &s, const LaneTup &l, in
     return ok;
 }
 
-// ---- step 3b: tuples of super-blocks (64 blocks) --------------------------------------------
-constexpr int SUP = 64; // blocks per super-block
+// ---- step 3b: tuples of nodes (16 blocks) and super-blocks (64 blocks) -------------------------
+// Per row: where the true state is known exactly so far (a super-block index and the state
+// there); nsup once the whole chain is resolved.
+struct Ctl
+{
+    int front;
+    uint32_t s;
+};
 
-__global__ __launch_bounds__(256) void sum1d_super_kernel(const Tup *__restrict__ T2, Tup *__restrict__ T3, int64_t nblk,
+// Per round of the speculative stage: the list of nodes that have to be walked.  The plan kernel
+// puts the nodes that promise long walks at the front (`count` of them, filled upwards from entry
+// 0) and the others at the back (`light`, filled downwards from the last entry); walkers take
+// the front ones first, so that the longest walks start first.  `next`: entries handed out.
+constexpr int MAX_ROUNDS = 12;
+constexpr int HEAVY_CHUNKS = 24; // predicted replays from which a node counts as a long walk
+struct Work
+{
+    int count;
+    int light;
+    int next;
+    int unused;
+};
+
+__global__ __launch_bounds__(256) void sum1d_super_kernel(const Tup *__restrict__ T2, Tup *__restrict__ TN, Tup *__restrict__ T3,
+                                                          Ctl *__restrict__ ctl, Work *__restrict__ work, int64_t nblk, int64_t nnode,
                                                           int64_t nsup)
 {
     const int lane = threadIdx.x & 63;
     const int64_t sb = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+    {
+        ctl[blockIdx.y].front = 0; // nothing resolved yet; the chain starts at +0.0f
+        ctl[blockIdx.y].s = 0u;
+    }
+    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x < MAX_ROUNDS)
+    {
+        work[threadIdx.x].count = 0; // the lists of walks of all rounds start empty
+        work[threadIdx.x].light = 0;
+        work[threadIdx.x].next = 0;
+    }
     if (sb >= nsup)
         return;
     T2 += (int64_t)blockIdx.y * nblk; // row
+    TN += (int64_t)blockIdx.y * nnode;
     T3 += (int64_t)blockIdx.y * nsup;
     const int64_t b = sb * SUP + lane;
     Tup t = b < nblk ? T2[b] : tup_identity(HYP_ANY);
 #pragma unroll
-    for (int off = 1; off < 64; off <<= 1)
+    for (int off = 1; off < NODEB; off <<= 1)
+        t = tup_join(t, tup_shfl_down(t, off)); // lanes 0, 4, 8, ...: the blocks of a node in order
+    if ((lane & (NODEB - 1)) == 0 && sb * NPS + lane / NODEB < nnode)
+        TN[sb * NPS + lane / NODEB] = t;
+#pragma unroll
+    for (int off = NODEB; off < 64; off <<= 1)
         t = tup_join(t, tup_shfl_down(t, off)); // lane 0: the 64 blocks in order
     if (lane == 0)
         T3[sb] = t;
@@ -571,7 +669,8 @@ __global__ __launch_bounds__(64) void sum1d_walk_kernel(const float *__restrict_
                                                         const Tup *__restrict__ T1,
                                                         const Tup *__restrict__ TG,
                                                         const Tup *__restrict__ T2,
-                                                        const Tup *__restrict__ T3, float factor,
+                                                        const Tup *__restrict__ T3,
+                                                        const Ctl *__restrict__ ctl, float factor,
                                                         float *__restrict__ out, int vec)
 {
     __shared__ __attribute__((aligned(16))) float xd[BLK + 2 * CH]; // + what the read-ahead overshoots
@@ -583,21 +682,27 @@ __global__ __launch_bounds__(64) void sum1d_walk_kernel(const float *__restrict_
     T2 += row * nblk;
     T3 += row * nsup;
     out += row;
-    uint32_t s = 0u; // +0.0f; wave-uniform throughout
-    BlockRegs pf;    // the block requested ahead
+    // Where the speculative rounds got to (super-block `first`, state there); 0 and +0.0f
+    // without rounds; nothing to do if they resolved the whole chain.
+    const int64_t first = __builtin_amdgcn_readfirstlane(ctl[row].front);
+    if (first >= nsup)
+        return;
+    uint32_t s = __builtin_amdgcn_readfirstlane(ctl[row].s); // wave-uniform throughout
+    BlockRegs pf;                                            // the block requested ahead
     int64_t pf_blk = -1;
     load_block(pf, x, c, T1, TG, 0, lane, vec); // (any valid block: the registers are then defined)
     pf_blk = 0;
-    Tup nsup_t = (lane < nsup) ? T3[lane] : tup_identity(HYP_ANY);
+    const int64_t gfirst = first & ~(int64_t)63;
+    Tup nsup_t = (gfirst + lane < nsup) ? T3[gfirst + lane] : tup_identity(HYP_ANY);
     // block tuples of the super-block being tried, and of the next one
-    Tup blk_next = (lane < nblk) ? T2[lane] : tup_identity(HYP_ANY);
-    for (int64_t g0 = 0; g0 < nsup; g0 += 64)
+    Tup blk_next = (first * SUP + lane < nblk) ? T2[first * SUP + lane] : tup_identity(HYP_ANY);
+    for (int64_t g0 = gfirst; g0 < nsup; g0 += 64)
     {
         const LaneTup ls = lane_tup(nsup_t);
         if (g0 + 64 < nsup) // the next 64 super-block tuples, loaded while these are walked
             nsup_t = (g0 + 64 + lane < nsup) ? T3[g0 + 64 + lane] : tup_identity(HYP_ANY);
         const int cnt = (nsup - g0 < 64) ? (int)(nsup - g0) : 64;
-        for (int i = 0; i < cnt; i++)
+        for (int i = (g0 == gfirst ? (int)(first - gfirst) : 0); i < cnt; i++)
         {
             const int64_t sb = g0 + i;
             const Tup blk_cur = blk_next;
@@ -653,6 +758,615 @@ __global__ __launch_bounds__(64) void sum1d_walk_kernel(const float *__restrict_
         out[0] = factor * __uint_as_float(s);
 }
 
+// ---- step 4a: a node walked for 256 candidate entry states ------------------------------------
+// A state is a binary32 bit pattern; candidate k of a node is base + k (any 32-bit pattern is a
+// state, and the walk below is exact for every one of them).
+
+// nearest candidate of the state whose bits are yb, for a window that starts at base
+__device__ __forceinline__ uint32_t nearest_candidate(uint32_t yb, uint32_t base, bool &hit)
+{
+    const uint32_t d = yb - base;
+    hit = d < (uint32_t)CAND;
+    return hit ? d : (d < 0x80000000u ? (uint32_t)(CAND - 1) : 0u);
+}
+
+// The window of candidates for a predicted state: CAND consecutive bit patterns around it, moved
+// where necessary to stay inside its binade (same sign and exponent).  The maps of a chunk assume
+// one binade, so candidates beyond its edge would be replayed element by element all the way --
+// for nothing when the sum sits exactly on the edge, as a sum of positive numbers does once it
+// has stopped growing at a power of two.  A true state on the far side of the edge is a miss, and
+// the next round's window lies there.
+__device__ __forceinline__ uint32_t window_base(uint32_t centre)
+{
+    const uint32_t lo = centre & 0xFF800000u, hi = centre | 0x007FFFFFu;
+    uint32_t base = centre - lo < (uint32_t)(CAND / 2) ? lo : centre - (uint32_t)(CAND / 2);
+    if (hi - base < (uint32_t)(CAND - 1))
+        base = hi - (uint32_t)(CAND - 1);
+    return base;
+}
+
+// One approximate step: the state sa (binary64, so that it can carry an excess over the
+// candidate it is snapped to) through a table.
+__device__ __forceinline__ double approx_step(double sa, uint32_t base, const uint32_t *__restrict__ tab)
+{
+    bool hit;
+    const uint32_t idx = nearest_candidate(__float_as_uint((float)sa), base, hit);
+    const double e = sa - (double)__uint_as_float(base + idx);
+    const double t = (double)__uint_as_float(tab[idx]);
+    return (e == e && e - e == 0.0) ? t + e : t; // a non-finite excess is dropped
+}
+
+// The test of lane_tup_apply for a whole wave of different states: the map (wave-uniform) is
+// applied if it is valid for every lane's state.
+__device__ __forceinline__ bool apply_all(uint32_t &s, const LaneTup &l)
+{
+    const bool odd = (s & 1u) != 0u;
+    const uint32_t smin = odd ? l.smin1 : l.smin0, smax = odd ? l.smax1 : l.smax0;
+    const bool ok = s >= smin && s <= smax;
+    if (!__all(ok))
+        return false;
+    s += (uint32_t)(odd ? l.t1 : l.t0);
+    return true;
+}
+
+// half a chunk (32 elements) from LDS, the same for every lane
+__device__ __forceinline__ void read_half(const float *__restrict__ xg, int h, f4v (&v)[CH / 8])
+{
+    const f4v *p = reinterpret_cast<const f4v *>(xg + h * (CH / 2));
+#pragma unroll
+    for (int k = 0; k < CH / 8; k++)
+        v[k] = p[k];
+}
+
+// 32 real additions, each lane on its own state
+__device__ __forceinline__ uint32_t add_half(uint32_t s, const f4v (&v)[CH / 8])
+{
+    float acc = __uint_as_float(s);
+#pragma unroll
+    for (int k = 0; k < CH / 8; k++)
+    {
+        acc = acc + v[k].x;
+        acc = acc + v[k].y;
+        acc = acc + v[k].z;
+        acc = acc + v[k].w;
+    }
+    return __float_as_uint(acc);
+}
+
+struct NodeRegs
+{
+    float4 f[BLK / 1024]; // this thread's 16 elements of the block
+    LaneTup lt;           // threads 0..63: a chunk map, 64..71: a group map, 72: the block map
+};
+
+// Thread tid's share of block blk (blocks past the end of the chain: -0.0f, which changes no state,
+// and identity maps).
+__device__ __forceinline__ void load_node_block(NodeRegs &r, const float *__restrict__ x, const Chains &c,
+                                                const Tup *__restrict__ T1, const Tup *__restrict__ TG,
+                                                const Tup *__restrict__ T2, int64_t blk, int tid, int vec)
+{
+    const int64_t n = c.n;
+    Tup t = tup_identity(HYP_ANY);
+    if (blk < c.nblk)
+    {
+        if (tid < BLK / CH)
+            t = T1[blk * (BLK / CH) + tid];
+        else if (tid < BLK / CH + GROUPS)
+            t = TG[blk * GROUPS + (tid - BLK / CH)];
+        else if (tid == BLK / CH + GROUPS)
+            t = T2[blk];
+    }
+    r.lt = lane_tup(t);
+    const int64_t e0 = blk * BLK;
+#pragma unroll
+    for (int q = 0; q < BLK / 1024; q++)
+    {
+        const int64_t idx = e0 + (int64_t)(q * 256 + tid) * 4;
+        if (vec && idx + 3 < n)
+            r.f[q] = *reinterpret_cast<const float4 *>(chain_ptr(x, c, idx)); // (segments are multiples of 16 long)
+        else
+        {
+            r.f[q].x = (idx + 0 < n) ? *chain_ptr(x, c, idx + 0) : -0.0f;
+            r.f[q].y = (idx + 1 < n) ? *chain_ptr(x, c, idx + 1) : -0.0f;
+            r.f[q].z = (idx + 2 < n) ? *chain_ptr(x, c, idx + 2) : -0.0f;
+            r.f[q].w = (idx + 3 < n) ? *chain_ptr(x, c, idx + 3) : -0.0f;
+        }
+    }
+}
+
+// Plan of a round: one wave per super-block that is not resolved yet.
+//   - the window of each of its nodes: round 0 centres it on the binary64 prediction of step 2,
+//     later rounds on the super-block centre the resolver left in sc[], taken through the previous
+//     round's tables node by node;
+//   - a node whose window has not moved keeps its table; a node whose own map holds for all its
+//     candidates gets its table from that map; every other node goes on the list of walks.
+// tab_*: [rows][nnode][CAND] exit states, nbase_*: [rows][nnode] first candidate of each window.
+__global__ __launch_bounds__(64) void sum1d_plan_kernel(const double *__restrict__ prefix, const Tup *__restrict__ TN,
+                                                        const Ctl *__restrict__ ctl, const float *__restrict__ sc,
+                                                        const float *__restrict__ hc, const float *__restrict__ SA,
+                                                        const uint32_t *__restrict__ sbase,
+                                                        const uint32_t *__restrict__ nbase_old, const uint32_t *__restrict__ tab_old,
+                                                        uint32_t *__restrict__ nbase_new, uint32_t *__restrict__ tab_new,
+                                                        int *__restrict__ worklist, Work *__restrict__ work, int64_t nblk,
+                                                        int64_t nnode, int64_t nsup, int round)
+{
+    const int lane = threadIdx.x;
+    const int64_t row = blockIdx.y, sb = blockIdx.x;
+    const int cap = (int)(nnode * gridDim.y); // entries of the list
+    const int64_t front = ctl[row].front;
+    if (front >= nsup || sb < front)
+        return; // resolved already
+    prefix += row * nblk;
+    TN += row * nnode;
+    sc += row * nsup;
+    hc += row * ((nsup + HB - 1) / HB);
+    SA += row * nsup * CAND;
+    sbase += row * nsup;
+    nbase_old += row * nnode;
+    nbase_new += row * nnode;
+    tab_old += row * nnode * CAND;
+    tab_new += row * nnode * CAND;
+    const int64_t n0 = sb * NPS;
+    const int cnt = nnode - n0 < NPS ? (int)(nnode - n0) : NPS;
+    float centre = 0.0f; // lane i: node n0 + i
+    if (round == 0)
+    {
+        if (lane < cnt)
+            centre = (float)prefix[(n0 + lane) * NODEB];
+    }
+    else
+    {
+        // (wave-uniform chain)  The resolver left a centre for every super-block of the hyper-block
+        // the front lies in, and for the first super-block of every later hyper-block; from
+        // there the centre goes through the approximate offsets of the super-blocks before this one.
+        double sa;
+        if (sb / HB == front / HB)
+            sa = (double)sc[sb];
+        else
+        {
+            sa = (double)hc[sb / HB];
+            for (int64_t j = sb / HB * HB; j < sb; j++)
+            {
+                bool hit;
+                const uint32_t idx = nearest_candidate(__float_as_uint((float)sa), sbase[j], hit);
+                sa += (double)SA[j * CAND + idx];
+            }
+        }
+        for (int i = 0; i < cnt; i++)
+        {
+            centre = lane == i ? (float)sa : centre;
+            sa = approx_step(sa, nbase_old[n0 + i], tab_old + (n0 + i) * CAND);
+        }
+    }
+    int kind = -1; // 0: keep the old table, 1: the node's own map, 2: walk
+    uint32_t base = 0u;
+    int t0 = 0, t1 = 0;
+    if (lane < cnt)
+    {
+        base = window_base(__float_as_uint(centre));
+        nbase_new[n0 + lane] = base;
+        const LaneTup ln = lane_tup(TN[n0 + lane]);
+        t0 = ln.t0;
+        t1 = ln.t1;
+        // candidates base .. base + CAND - 1: the even ones and the odd ones each inside their interval
+        const uint32_t e0 = base + (base & 1u), e1 = base + CAND - 2 + (base & 1u);
+        const uint32_t o0 = base + 1 - (base & 1u), o1 = base + CAND - 1 - (base & 1u);
+        const bool whole = e0 >= ln.smin0 && e1 <= ln.smax0 && o0 >= ln.smin1 && o1 <= ln.smax1 && e1 >= e0 && o1 >= o0;
+        kind = (round != 0 && nbase_old[n0 + lane] == base) ? 0 : (whole ? 1 : 2);
+        if (kind == 2)
+        {
+            const int gn = (int)(row * nnode + n0 + lane);
+            if (TN[n0 + lane].heavy >= HEAVY_CHUNKS)
+                worklist[atomicAdd(&work[round].count, 1)] = gn;
+            else
+                worklist[cap - 1 - atomicAdd(&work[round].light, 1)] = gn;
+        }
+    }
+    for (int i = 0; i < cnt; i++)
+    {
+        const int k = __shfl(kind, i, 64);
+        if (k == 2)
+            continue;
+        const uint32_t b = (uint32_t)__shfl((int)base, i, 64);
+        const int a0 = __shfl(t0, i, 64), a1 = __shfl(t1, i, 64);
+#pragma unroll
+        for (int q = 0; q < CAND / 64; q++)
+        {
+            const int c = q * 64 + lane;
+            const uint32_t st = b + (uint32_t)c;
+            tab_new[(n0 + i) * CAND + c] = k == 0 ? tab_old[(n0 + i) * CAND + c] : st + (uint32_t)((st & 1u) ? a1 : a0);
+        }
+    }
+}
+
+#ifdef REPDL_DEBUG_HOOKS
+__device__ unsigned long long g_dbg[8]; // wave-level counts: nodes, blocks failed, groups failed, chunk replays
+#define DBG_COUNT(i) do { if ((threadIdx.x & 63) == 0) atomicAdd(&g_dbg[i], 1ull); } while (0)
+#else
+#define DBG_COUNT(i) do { } while (0)
+#endif
+
+// The walks of a round: workgroups of 256 threads take nodes off the list until it is empty
+// (every workgroup leaves the loop: the list's length is fixed before the launch).  Thread t
+// carries candidate t of the node's window.
+__global__ __launch_bounds__(256) void sum1d_cand_walk_kernel(
+    const float *__restrict__ x, Chains c, const Tup *__restrict__ T1, const Tup *__restrict__ TG,
+    const Tup *__restrict__ T2, const uint32_t *__restrict__ nbase, uint32_t *__restrict__ tab,
+    const int *__restrict__ worklist, Work *__restrict__ work, int64_t nnode, int cap, int round, int vec)
+{
+    __shared__ __attribute__((aligned(16))) float xd[2][BLK];
+    __shared__ __attribute__((aligned(16))) LaneTup lmap[2][BLK / CH + GROUPS + 1];
+    __shared__ int item_s;
+    const int tid = threadIdx.x;
+    const int front_count = work[round].count, count = front_count + work[round].light;
+    for (;;)
+    {
+        if (tid == 0)
+            item_s = atomicAdd(&work[round].next, 1);
+        __syncthreads();
+        const int item = item_s;
+        __syncthreads(); // (everyone has read item_s, and has finished with the LDS of the previous node)
+        if (item >= count)
+            break;
+        const int64_t gn = worklist[item < front_count ? item : cap - 1 - (item - front_count)], row = gn / nnode,
+                      nd = gn - row * nnode;
+        const float *xr = x + row * c.row_stride;
+        const Tup *T1r = T1 + row * c.nblk * (BLK / CH), *TGr = TG + row * c.nblk * GROUPS, *T2r = T2 + row * c.nblk;
+        uint32_t s = nbase[gn] + (uint32_t)tid;
+        NodeRegs r;
+        load_node_block(r, xr, c, T1r, TGr, T2r, nd * NODEB, tid, vec);
+        for (int b = 0; b < NODEB; b++)
+        {
+            const int buf = b & 1;
+#pragma unroll
+            for (int q = 0; q < BLK / 1024; q++)
+                *reinterpret_cast<float4 *>(&xd[buf][(q * 256 + tid) * 4]) = r.f[q];
+            if (tid <= BLK / CH + GROUPS)
+                lmap[buf][tid] = r.lt;
+            // One barrier per block is enough: a wave that stores block b + 1 into the other buffer
+            // has passed this barrier, so every wave has finished walking block b - 1 in it.
+            __syncthreads();
+            if (b + 1 < NODEB)
+                load_node_block(r, xr, c, T1r, TGr, T2r, nd * NODEB + b + 1, tid, vec);
+            DBG_COUNT(0);
+            if (apply_all(s, lmap[buf][BLK / CH + GROUPS]))
+                continue;
+            DBG_COUNT(1);
+            // Where the sum is small against its elements nothing applies, block after block; a
+            // test costs a quarter of a replay there, and a replay is always right.  So after two
+            // failures in a row the rest of the unit (the groups of a block, the chunks of a group)
+            // is taken without testing.
+            int gfail = 0;
+            for (int gr = 0; gr < GROUPS; gr++)
+            {
+                if (gfail < 2 && apply_all(s, lmap[buf][BLK / CH + gr]))
+                {
+                    gfail = 0;
+                    continue;
+                }
+                gfail++;
+                DBG_COUNT(2);
+                constexpr int CG = BLK / CH / GROUPS; // 8 chunks; their data is read half a chunk ahead of the additions
+                const float *xg = &xd[buf][gr * CG * CH];
+                f4v ha[CH / 8], hb[CH / 8];
+                int cfail = 0;
+                read_half(xg, 0, ha);
+#pragma unroll
+                for (int j = 0; j < CG; j++)
+                {
+                    read_half(xg, 2 * j + 1, hb);
+                    const bool replay = cfail >= 2 || !apply_all(s, lmap[buf][gr * CG + j]);
+                    if (replay)
+                    {
+                        DBG_COUNT(3);
+                        s = add_half(s, ha);
+                    }
+                    if (j + 1 < CG)
+                        read_half(xg, 2 * j + 2, ha);
+                    if (replay)
+                        s = add_half(s, hb);
+                    cfail = replay ? cfail + 1 : 0;
+                }
+            }
+        }
+        tab[gn * CAND + tid] = s;
+    }
+}
+
+// ---- step 4b: the node tables of a super-block composed ----------------------------------------
+// grid (super-blocks, rows), 256 threads: thread k takes candidate k of the super-block's first
+// node through the tables of its nodes.  SE[k]: the exit state, exact if bit k of SOK is set
+// (every intermediate state was a candidate of the next node); SA[k]: exit minus entry as a
+// binary32 offset, approximate where a state had to be snapped to the nearest candidate.
+__global__ __launch_bounds__(256) void sum1d_compose_kernel(const uint32_t *__restrict__ nbase, const uint32_t *__restrict__ tab,
+                                                            const Ctl *__restrict__ ctl, uint32_t *__restrict__ SE,
+                                                            float *__restrict__ SA, uint32_t *__restrict__ SOK,
+                                                            uint32_t *__restrict__ sbase, int64_t nnode, int64_t nsup)
+{
+    const int tid = threadIdx.x;
+    const int64_t row = blockIdx.y, sb = blockIdx.x;
+    const int64_t front = ctl[row].front;
+    if (front >= nsup || sb < front)
+        return;
+    nbase += row * nnode;
+    tab += row * nnode * CAND;
+    SE += (row * nsup + sb) * CAND;
+    SA += (row * nsup + sb) * CAND;
+    SOK += (row * nsup + sb) * (CAND / 32);
+    const int64_t n0 = sb * NPS;
+    const uint32_t base0 = nbase[n0];
+    uint32_t y = base0 + (uint32_t)tid; // exact while ok
+    bool ok = true;
+    double sa = 0.0; // the approximate state once a window was missed
+    for (int i = 0; i < NPS && n0 + i < nnode; i++)
+    {
+        const uint32_t b = nbase[n0 + i];
+        const uint32_t *t = tab + (n0 + i) * CAND;
+        if (ok)
+        {
+            const uint32_t d = y - b;
+            if (d < (uint32_t)CAND)
+            {
+                y = t[d];
+                continue;
+            }
+            ok = false;
+            sa = (double)__uint_as_float(y);
+        }
+        sa = approx_step(sa, b, t);
+    }
+    const double entry = (double)__uint_as_float(base0 + (uint32_t)tid);
+    SE[tid] = y;
+    SA[tid] = (float)((ok ? (double)__uint_as_float(y) : sa) - entry);
+    const unsigned long long m = __ballot(ok);
+    if ((tid & 63) == 0)
+    {
+        SOK[(tid >> 6) * 2] = (uint32_t)m;
+        SOK[(tid >> 6) * 2 + 1] = (uint32_t)(m >> 32);
+    }
+    if (tid == 0)
+        sbase[row * nsup + sb] = base0;
+}
+
+// ---- step 4b': the super-block tables of a hyper-block composed ----------------------------------
+// The same composition one level up: grid (hyper-blocks, rows), 256 threads; thread k takes candidate
+// k of the hyper-block's first unresolved super-block through its super-blocks.  HE / HOK / HA as
+// SE / SOK / SA.
+__global__ __launch_bounds__(256) void sum1d_compose2_kernel(const uint32_t *__restrict__ SE, const float *__restrict__ SA,
+                                                             const uint32_t *__restrict__ SOK, const uint32_t *__restrict__ sbase,
+                                                             const Ctl *__restrict__ ctl, uint32_t *__restrict__ HE,
+                                                             float *__restrict__ HA, uint32_t *__restrict__ HOK,
+                                                             uint32_t *__restrict__ hbase, int64_t nsup, int64_t nhyp)
+{
+    const int tid = threadIdx.x;
+    const int64_t row = blockIdx.y, h = blockIdx.x;
+    const int64_t front = ctl[row].front;
+    if (front >= nsup || h < front / HB)
+        return;
+    SE += row * nsup * CAND;
+    SA += row * nsup * CAND;
+    SOK += row * nsup * (CAND / 32);
+    sbase += row * nsup;
+    HE += (row * nhyp + h) * CAND;
+    HA += (row * nhyp + h) * CAND;
+    HOK += (row * nhyp + h) * (CAND / 32);
+    const int64_t j0 = h * HB > front ? h * HB : front, j1 = (h + 1) * HB < nsup ? (h + 1) * HB : nsup;
+    const uint32_t base0 = sbase[j0];
+    uint32_t y = base0 + (uint32_t)tid; // exact while ok
+    bool ok = true;
+    double sa = 0.0;
+    for (int64_t j = j0; j < j1; j++)
+    {
+        const uint32_t b = sbase[j];
+        if (ok)
+        {
+            const uint32_t d = y - b;
+            if (d < (uint32_t)CAND && ((SOK[j * (CAND / 32) + (d >> 5)] >> (d & 31u)) & 1u) != 0u)
+            {
+                y = SE[j * CAND + d];
+                continue;
+            }
+            ok = false;
+            sa = (double)__uint_as_float(y);
+        }
+        bool hit;
+        const uint32_t idx = nearest_candidate(__float_as_uint((float)sa), b, hit);
+        sa += (double)SA[j * CAND + idx];
+    }
+    const double entry = (double)__uint_as_float(base0 + (uint32_t)tid);
+    HE[tid] = y;
+    HA[tid] = (float)((ok ? (double)__uint_as_float(y) : sa) - entry);
+    const unsigned long long m = __ballot(ok);
+    if ((tid & 63) == 0)
+    {
+        HOK[(tid >> 6) * 2] = (uint32_t)m;
+        HOK[(tid >> 6) * 2 + 1] = (uint32_t)(m >> 32);
+    }
+    if (tid == 0)
+        hbase[row * nhyp + h] = base0;
+}
+
+// ---- step 4c: the true state through the tables --------------------------------------------------
+// One workgroup of 256 threads per row; every thread runs the same chain (all reads are LDS
+// broadcasts), so that the workgroup can stage tables together wherever the chain needs them.
+// The state steps through the hyper-block tables (RB at a time in LDS, requested RD batches
+// ahead) while it finds itself among the candidates and the entry is exact.  At the first miss
+// the sixteen super-block tables of that hyper-block come into LDS and the state steps through
+// those up to the super-block that misses: the new front.  From there the chain is approximate
+// (nearest candidate, the excess kept in binary64) and leaves the predictions of the next round:
+// sc[] for the rest of this hyper-block, hc[] for every later hyper-block.
+constexpr int RB = 4; // hyper-blocks per batch
+constexpr int RD = 4; // batches in flight
+
+__global__ __launch_bounds__(256) void sum1d_resolve_kernel(
+    const uint32_t *__restrict__ HE, const float *__restrict__ HA, const uint32_t *__restrict__ HOK,
+    const uint32_t *__restrict__ hbase, const uint32_t *__restrict__ SE, const float *__restrict__ SA,
+    const uint32_t *__restrict__ SOK, const uint32_t *__restrict__ sbase, float *__restrict__ sc, float *__restrict__ hc,
+    Ctl *__restrict__ ctl, float factor, float *__restrict__ out, int64_t nsup, int64_t nhyp)
+{
+    __shared__ __attribute__((aligned(16))) uint32_t lhe[2][RB][CAND];
+    __shared__ __attribute__((aligned(16))) float lha[2][RB][CAND];
+    __shared__ uint32_t lhok[2][RB][CAND / 32];
+    __shared__ uint32_t lhbase[2][RB];
+    __shared__ __attribute__((aligned(16))) uint32_t dse[HB][CAND];
+    __shared__ __attribute__((aligned(16))) float dsa[HB][CAND];
+    __shared__ uint32_t dok[HB][CAND / 32];
+    __shared__ uint32_t dbase[HB];
+    const int tid = threadIdx.x;
+    const int64_t row = blockIdx.x;
+    const int64_t front = ctl[row].front;
+    if (front >= nsup)
+        return;
+    HE += row * nhyp * CAND;
+    HA += row * nhyp * CAND;
+    HOK += row * nhyp * (CAND / 32);
+    hbase += row * nhyp;
+    SE += row * nsup * CAND;
+    SA += row * nsup * CAND;
+    SOK += row * nsup * (CAND / 32);
+    sbase += row * nsup;
+    sc += row * nsup;
+    hc += row * nhyp;
+    const int64_t h0 = front / HB;
+    const int64_t nbatch = (nhyp - h0 + RB - 1) / RB;
+    // this thread's part of a batch: 16 bytes of each hyper-block's exact and approximate table
+    // (tid: hyper-block tid / 64, piece tid % 64), one word of the masks / bases
+    const int wh = tid >> 6, wq = tid & 63;
+    uint4 pfe[RD], pfa[RD];
+    uint32_t pfw[RD];
+    auto request = [&](int64_t bt, uint4 &ve, uint4 &va, uint32_t &word) {
+        ve = va = make_uint4(0u, 0u, 0u, 0u);
+        word = 0u;
+        if (bt >= nbatch)
+            return;
+        const int64_t h = h0 + bt * RB + wh;
+        if (h < nhyp)
+        {
+            ve = reinterpret_cast<const uint4 *>(HE + h * CAND)[wq];
+            va = reinterpret_cast<const uint4 *>(HA + h * CAND)[wq];
+        }
+        if (tid < RB * (CAND / 32))
+        {
+            const int64_t hh = h0 + bt * RB + tid / (CAND / 32);
+            word = hh < nhyp ? HOK[hh * (CAND / 32) + tid % (CAND / 32)] : 0u;
+        }
+        else if (tid < RB * (CAND / 32) + RB)
+        {
+            const int64_t hh = h0 + bt * RB + (tid - RB * (CAND / 32));
+            word = hh < nhyp ? hbase[hh] : 0u;
+        }
+    };
+#pragma unroll
+    for (int d = 0; d < RD; d++)
+        request(d, pfe[d], pfa[d], pfw[d]);
+    uint32_t s = ctl[row].s;
+    bool exact = true;
+    double sa = 0.0;
+    int64_t new_front = nsup;
+    uint32_t s_front = 0u;
+    for (int64_t bt0 = 0; bt0 < nbatch; bt0 += RD)
+    {
+#pragma unroll
+        for (int d = 0; d < RD; d++)
+        {
+            const int64_t bt = bt0 + d;
+            if (bt >= nbatch) // (uniform)
+                break;
+            const int buf = d & 1; // RD is even
+            reinterpret_cast<uint4 *>(&lhe[buf][wh][0])[wq] = pfe[d];
+            reinterpret_cast<uint4 *>(&lha[buf][wh][0])[wq] = pfa[d];
+            if (tid < RB * (CAND / 32))
+                lhok[buf][tid / (CAND / 32)][tid % (CAND / 32)] = pfw[d];
+            else if (tid < RB * (CAND / 32) + RB)
+                lhbase[buf][tid - RB * (CAND / 32)] = pfw[d];
+            // (this batch's buffer was last read two batches ago, and a barrier lies in between)
+            __syncthreads();
+            request(bt + RD, pfe[d], pfa[d], pfw[d]);
+            for (int i = 0; i < RB; i++)
+            {
+                const int64_t h = h0 + bt * RB + i;
+                if (h >= nhyp)
+                    break;
+                const uint32_t base = lhbase[buf][i];
+                if (exact)
+                {
+                    const uint32_t dd = s - base;
+                    const uint32_t k = dd < (uint32_t)CAND ? dd : 0u;
+                    const uint32_t nxt = lhe[buf][i][k];
+                    const uint32_t okw = lhok[buf][i][k >> 5];
+                    if (dd < (uint32_t)CAND && ((okw >> (k & 31u)) & 1u) != 0u)
+                    {
+                        s = nxt; // an exact step over a whole hyper-block
+                        continue;
+                    }
+                    // somewhere inside this hyper-block the state is not among the candidates:
+                    // its super-block tables, together
+                    const int64_t j0 = h * HB > front ? h * HB : front, j1 = (h + 1) * HB < nsup ? (h + 1) * HB : nsup;
+                    const int cnt = (int)(j1 - j0);
+                    __syncthreads(); // (whoever still reads the tables of an earlier descent)
+                    for (int q = tid; q < cnt * (CAND / 4); q += 256)
+                    {
+                        const int jj = q / (CAND / 4), pc = q % (CAND / 4);
+                        reinterpret_cast<uint4 *>(&dse[jj][0])[pc] = reinterpret_cast<const uint4 *>(SE + (j0 + jj) * CAND)[pc];
+                        reinterpret_cast<uint4 *>(&dsa[jj][0])[pc] = reinterpret_cast<const uint4 *>(SA + (j0 + jj) * CAND)[pc];
+                    }
+                    if (tid < cnt * (CAND / 32))
+                        dok[tid / (CAND / 32)][tid % (CAND / 32)] = SOK[(j0 + tid / (CAND / 32)) * (CAND / 32) + tid % (CAND / 32)];
+                    else if (tid >= 128 && tid < 128 + cnt)
+                        dbase[tid - 128] = sbase[j0 + tid - 128];
+                    __syncthreads();
+                    int jj = 0;
+                    for (; jj < cnt; jj++)
+                    {
+                        const uint32_t d2 = s - dbase[jj];
+                        const uint32_t k2 = d2 < (uint32_t)CAND ? d2 : 0u;
+                        if (!(d2 < (uint32_t)CAND && ((dok[jj][k2 >> 5] >> (k2 & 31u)) & 1u) != 0u))
+                            break;
+                        s = dse[jj][k2];
+                    }
+                    if (jj == cnt)
+                        continue; // (every super-block hit after all)
+                    exact = false;
+                    new_front = j0 + jj;
+                    s_front = s;
+                    sa = (double)__uint_as_float(s);
+                    for (; jj < cnt; jj++)
+                    {
+                        const float f = (float)sa;
+                        if (tid == 0)
+                            sc[j0 + jj] = f;
+                        bool hit;
+                        const uint32_t idx = nearest_candidate(__float_as_uint(f), dbase[jj], hit);
+                        sa += (double)dsa[jj][idx];
+                    }
+                    continue;
+                }
+                // approximate from here on: predictions for the next round
+                const float f = (float)sa;
+                if (tid == 0)
+                    hc[h] = f;
+                bool hit;
+                const uint32_t idx = nearest_candidate(__float_as_uint(f), base, hit);
+                sa += (double)lha[buf][i][idx];
+            }
+        }
+    }
+    if (tid == 0)
+    {
+        if (exact)
+        {
+            ctl[row].front = (int)nsup;
+            ctl[row].s = s;
+            out[row] = factor * __uint_as_float(s);
+        }
+        else
+        {
+            ctl[row].front = (int)new_front;
+            ctl[row].s = s_front;
+        }
+    }
+}
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 inline size_t round256(size_t v) { return (v + 255) & ~(size_t)255; }
 } // namespace
@@ -660,29 +1374,91 @@ inline size_t round256(size_t v) { return (v + 255) & ~(size_t)255; }
 // serial single-chain kernel of sum.hip
 int repdl_sum1d_serial(const float *in, float *out, int64_t n, int average, void *stream);
 
-// Scratch for `rows` chains of n elements.
-size_t repdl_sum_chains_workspace_bytes(int64_t rows, int64_t n)
+// Number of speculative rounds for `rows` chains of n elements (0: step 4 alone).  Rounds pay
+// from a few million elements on; chains that come in rows are short and many, and their walks
+// already run side by side.
+#ifdef REPDL_DEBUG_HOOKS
+static int g_debug_rounds = -1;
+#endif
+static int spec_rounds(int64_t rows, int64_t n)
 {
-    const size_t nblk = (size_t)repdl_cdiv(n, BLK) * (size_t)rows;
-    const size_t nsup = (size_t)repdl_cdiv(repdl_cdiv(n, BLK), SUP) * (size_t)rows;
-    return round256(nblk * sizeof(double)) * 2 + round256(nsup * sizeof(Tup)) + round256(nblk * sizeof(Tup)) +
-           round256(nblk * GROUPS * sizeof(Tup)) + round256(nblk * (BLK / CH) * sizeof(Tup));
+    if (rows != 1 || n < ((int64_t)1 << 22))
+        return 0;
+#ifdef REPDL_DEBUG_HOOKS
+    if (g_debug_rounds >= 0)
+        return g_debug_rounds;
+#endif
+    return n < ((int64_t)1 << 24) ? 4 : (n < ((int64_t)1 << 26) ? 8 : MAX_ROUNDS);
 }
+
+namespace
+{
+struct Layout
+{
+    size_t bsum, prefix, T3, TN, T2, TG, T1, ctl, work, sc, nbase[2], tab[2], worklist, SE, SA, SOK, sbase, HE, HA, HOK, hbase, hc, total;
+};
+
+Layout layout(int64_t rows, int64_t n)
+{
+    const size_t nblk = (size_t)repdl_cdiv(n, BLK), nnode = (size_t)repdl_cdiv((int64_t)nblk, NODEB),
+                 nsup = (size_t)repdl_cdiv((int64_t)nblk, SUP), r = (size_t)rows;
+    Layout l;
+    size_t at = 0;
+    auto take = [&](size_t bytes) {
+        const size_t here = at;
+        at += round256(bytes);
+        return here;
+    };
+    l.bsum = take(r * nblk * sizeof(double));
+    l.prefix = take(r * nblk * sizeof(double));
+    l.T3 = take(r * nsup * sizeof(Tup));
+    l.TN = take(r * nnode * sizeof(Tup));
+    l.T2 = take(r * nblk * sizeof(Tup));
+    l.TG = take(r * nblk * GROUPS * sizeof(Tup));
+    l.T1 = take(r * nblk * (BLK / CH) * sizeof(Tup));
+    l.ctl = take(r * sizeof(Ctl));
+    l.work = take(MAX_ROUNDS * sizeof(Work));
+    const bool spec = spec_rounds(rows, n) > 0;
+    l.sc = take(spec ? r * nsup * sizeof(float) : 0);
+    for (int i = 0; i < 2; i++)
+        l.nbase[i] = take(spec ? r * nnode * sizeof(uint32_t) : 0);
+    for (int i = 0; i < 2; i++)
+        l.tab[i] = take(spec ? r * nnode * CAND * sizeof(uint32_t) : 0);
+    l.worklist = take(spec ? r * nnode * sizeof(int) : 0);
+    l.SE = take(spec ? r * nsup * CAND * sizeof(uint32_t) : 0);
+    l.SA = take(spec ? r * nsup * CAND * sizeof(float) : 0);
+    l.SOK = take(spec ? r * nsup * (CAND / 32) * sizeof(uint32_t) : 0);
+    l.sbase = take(spec ? r * nsup * sizeof(uint32_t) : 0);
+    const size_t nhyp = (nsup + HB - 1) / HB;
+    l.HE = take(spec ? r * nhyp * CAND * sizeof(uint32_t) : 0);
+    l.HA = take(spec ? r * nhyp * CAND * sizeof(float) : 0);
+    l.HOK = take(spec ? r * nhyp * (CAND / 32) * sizeof(uint32_t) : 0);
+    l.hbase = take(spec ? r * nhyp * sizeof(uint32_t) : 0);
+    l.hc = take(spec ? r * nhyp * sizeof(float) : 0);
+    l.total = at;
+    return l;
+}
+} // namespace
+
+// Scratch for `rows` chains of n elements.
+size_t repdl_sum_chains_workspace_bytes(int64_t rows, int64_t n) { return layout(rows, n).total; }
 
 // out[r] = factor * (the sequential sum of chain r), r < rows, by the parallel evaluation.
 // Chain r: nseg segments of seglen contiguous floats, segment s at in + r*row_stride +
 // s*seg_stride.  The caller has checked: n = nseg*seglen >= 1, rows in [1, 65535], and for
 // nseg > 1 that seglen is a multiple of 16 and n < 2^31.
+// Every word of the scratch memory that is read has been written earlier in the same call, so
+// it may hold anything on entry.
 int repdl_sum_chains(const float *in, float *out, int64_t rows, int64_t nseg, int64_t seglen, int64_t row_stride,
                      int64_t seg_stride, float factor, void *workspace, size_t workspace_bytes, void *stream)
 {
     const int64_t n = nseg * seglen;
     REPDL_REQUIRE(rows >= 1 && rows <= 65535 && n >= 1 && in != nullptr && out != nullptr);
     REPDL_REQUIRE(nseg == 1 || (seglen % 16 == 0 && n <= REPDL_I32_MAX));
-    if (workspace == nullptr || workspace_bytes < repdl_sum_chains_workspace_bytes(rows, n) ||
-        (reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
+    const Layout l = layout(rows, n);
+    if (workspace == nullptr || workspace_bytes < l.total || (reinterpret_cast<uintptr_t>(workspace) & 15) != 0)
         return REPDL_E_WORKSPACE;
-    const int64_t nblk = repdl_cdiv(n, BLK), nsup = repdl_cdiv(nblk, SUP);
+    const int64_t nblk = repdl_cdiv(n, BLK), nnode = repdl_cdiv(nblk, NODEB), nsup = repdl_cdiv(nblk, SUP);
     REPDL_REQUIRE(nblk <= REPDL_I32_MAX);
     Chains c;
     c.n = n;
@@ -693,30 +1469,55 @@ int repdl_sum_chains(const float *in, float *out, int64_t rows, int64_t nseg, in
     c.seglen = nseg > 1 ? (int)seglen : 0;
     c.segmented = nseg > 1;
     char *w = static_cast<char *>(workspace);
-    double *bsum = reinterpret_cast<double *>(w);
-    w += round256(rows * nblk * sizeof(double));
-    double *prefix = reinterpret_cast<double *>(w);
-    w += round256(rows * nblk * sizeof(double));
-    Tup *T3 = reinterpret_cast<Tup *>(w);
-    w += round256(rows * nsup * sizeof(Tup));
-    Tup *T2 = reinterpret_cast<Tup *>(w);
-    w += round256(rows * nblk * sizeof(Tup));
-    Tup *TG = reinterpret_cast<Tup *>(w);
-    w += round256(rows * nblk * GROUPS * sizeof(Tup));
-    Tup *T1 = reinterpret_cast<Tup *>(w);
+    double *bsum = reinterpret_cast<double *>(w + l.bsum), *prefix = reinterpret_cast<double *>(w + l.prefix);
+    Tup *T3 = reinterpret_cast<Tup *>(w + l.T3), *TN = reinterpret_cast<Tup *>(w + l.TN), *T2 = reinterpret_cast<Tup *>(w + l.T2),
+        *TG = reinterpret_cast<Tup *>(w + l.TG), *T1 = reinterpret_cast<Tup *>(w + l.T1);
+    Ctl *ctl = reinterpret_cast<Ctl *>(w + l.ctl);
+    Work *work = reinterpret_cast<Work *>(w + l.work);
     hipStream_t s = repdl_stream(stream);
     // 16-byte loads: every row and segment starts on a 16-byte boundary
     const int vec = aligned16(in) && (rows == 1 || row_stride % 4 == 0) && (nseg == 1 || seg_stride % 4 == 0);
     const dim3 g2((unsigned)nblk, (unsigned)rows);
     hipLaunchKernelGGL(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(nullptr), bsum, vec);
-    hipLaunchKernelGGL(sum1d_prefix_kernel, dim3((unsigned)rows), dim3(256), 0, s, bsum, prefix, nblk);
+    hipLaunchKernelGGL(sum1d_prefix_kernel, dim3((unsigned)rows), dim3(1024), 0, s, bsum, prefix, nblk);
     // one refinement of the prediction (see quantum_of)
     hipLaunchKernelGGL(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(prefix), bsum, vec);
-    hipLaunchKernelGGL(sum1d_prefix_kernel, dim3((unsigned)rows), dim3(256), 0, s, bsum, prefix, nblk);
+    hipLaunchKernelGGL(sum1d_prefix_kernel, dim3((unsigned)rows), dim3(1024), 0, s, bsum, prefix, nblk);
     hipLaunchKernelGGL(sum1d_tuple_kernel, g2, dim3(256), 0, s, in, c, prefix, T1, TG, T2, vec);
-    hipLaunchKernelGGL(sum1d_super_kernel, dim3((unsigned)repdl_cdiv(nsup, 4), (unsigned)rows), dim3(256), 0, s, T2, T3, nblk,
-                       nsup);
-    hipLaunchKernelGGL(sum1d_walk_kernel, dim3((unsigned)rows), dim3(64), 0, s, in, c, T1, TG, T2, T3, factor, out, vec);
+    hipLaunchKernelGGL(sum1d_super_kernel, dim3((unsigned)repdl_cdiv(nsup, 4), (unsigned)rows), dim3(256), 0, s, T2, TN, T3, ctl,
+                       work, nblk, nnode, nsup);
+    const int rounds = spec_rounds(rows, n);
+    if (rounds > 0)
+    {
+        float *sc = reinterpret_cast<float *>(w + l.sc);
+        uint32_t *nbase[2] = {reinterpret_cast<uint32_t *>(w + l.nbase[0]), reinterpret_cast<uint32_t *>(w + l.nbase[1])};
+        uint32_t *tab[2] = {reinterpret_cast<uint32_t *>(w + l.tab[0]), reinterpret_cast<uint32_t *>(w + l.tab[1])};
+        uint32_t *SE = reinterpret_cast<uint32_t *>(w + l.SE), *SOK = reinterpret_cast<uint32_t *>(w + l.SOK),
+                 *sbase = reinterpret_cast<uint32_t *>(w + l.sbase);
+        float *SA = reinterpret_cast<float *>(w + l.SA);
+        int *worklist = reinterpret_cast<int *>(w + l.worklist);
+        const int64_t nhyp = repdl_cdiv(nsup, HB);
+        uint32_t *HE = reinterpret_cast<uint32_t *>(w + l.HE), *HOK = reinterpret_cast<uint32_t *>(w + l.HOK),
+                 *hbase = reinterpret_cast<uint32_t *>(w + l.hbase);
+        float *HA = reinterpret_cast<float *>(w + l.HA), *hc = reinterpret_cast<float *>(w + l.hc);
+        for (int r = 0; r < rounds; r++)
+        {
+            const int cur = r & 1, old = cur ^ 1;
+            hipLaunchKernelGGL(sum1d_plan_kernel, dim3((unsigned)nsup, (unsigned)rows), dim3(64), 0, s, prefix, TN, ctl, sc, hc, SA, sbase,
+                               nbase[old], tab[old], nbase[cur], tab[cur], worklist, work, nblk, nnode, nsup, r);
+            const int64_t walkers = nnode * rows < 1024 ? nnode * rows : 1024; // four workgroups per CU
+            hipLaunchKernelGGL(sum1d_cand_walk_kernel, dim3((unsigned)walkers), dim3(256), 0, s, in, c, T1, TG, T2, nbase[cur], tab[cur],
+                               worklist, work, nnode, (int)(nnode * rows), r, vec);
+            hipLaunchKernelGGL(sum1d_compose_kernel, dim3((unsigned)nsup, (unsigned)rows), dim3(256), 0, s, nbase[cur], tab[cur], ctl,
+                               SE, SA, SOK, sbase, nnode, nsup);
+            hipLaunchKernelGGL(sum1d_compose2_kernel, dim3((unsigned)nhyp, (unsigned)rows), dim3(256), 0, s, SE, SA, SOK, sbase, ctl, HE,
+                               HA, HOK, hbase, nsup, nhyp);
+            hipLaunchKernelGGL(sum1d_resolve_kernel, dim3((unsigned)rows), dim3(256), 0, s, HE, HA, HOK, hbase, SE, SA, SOK, sbase, sc,
+                               hc, ctl, factor, out, nsup, nhyp);
+        }
+    }
+    // whatever the rounds left (everything, without rounds), from the front
+    hipLaunchKernelGGL(sum1d_walk_kernel, dim3((unsigned)rows), dim3(64), 0, s, in, c, T1, TG, T2, T3, ctl, factor, out, vec);
     return repdl_launch_status();
 }
 
@@ -815,3 +1616,35 @@ REPDL_API int repdl_hip_sum1d_static(const float *in, float *out, int64_t n, int
     }
     return repdl_hip_sum1d_ws(in, out, n, average, ptr, STATIC_SCRATCH_BYTES, stream);
 }
+
+#ifdef REPDL_DEBUG_HOOKS
+// Development only (not built into the library): force the number of rounds, read a row's front.
+REPDL_API void repdl_debug_sum1d_rounds(int r) { g_debug_rounds = r; }
+REPDL_API int repdl_debug_sum1d_front(const void *workspace, int64_t n)
+{
+    const Layout l = layout(1, n);
+    Ctl c;
+    hipDeviceSynchronize();
+    hipMemcpy(&c, static_cast<const char *>(workspace) + l.ctl, sizeof(c), hipMemcpyDeviceToHost);
+    return c.front;
+}
+REPDL_API void repdl_debug_sum1d_counts(unsigned long long *c, int reset)
+{
+    hipDeviceSynchronize();
+    hipMemcpyFromSymbol(c, HIP_SYMBOL(g_dbg), sizeof(g_dbg));
+    if (reset)
+    {
+        unsigned long long z[8] = {};
+        hipMemcpyToSymbol(HIP_SYMBOL(g_dbg), z, sizeof(z));
+    }
+}
+REPDL_API void repdl_debug_sum1d_work(const void *workspace, int64_t n, int *counts)
+{
+    const Layout l = layout(1, n);
+    Work w[MAX_ROUNDS];
+    hipDeviceSynchronize();
+    hipMemcpy(w, static_cast<const char *>(workspace) + l.work, sizeof(w), hipMemcpyDeviceToHost);
+    for (int i = 0; i < MAX_ROUNDS; i++)
+        counts[i] = w[i].count + w[i].light;
+}
+#endif

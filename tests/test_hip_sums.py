@@ -184,3 +184,66 @@ def test_full_size_benchmark_inputs():
     got = ops.sum2d_dim1(m.cuda()).cpu()
     assert torch.equal(got.view(torch.int32), oracle.sum2d_dim1(m).view(torch.int32))
     assert torch.equal(ops.sum2d_dim0(m.cuda()).cpu().view(torch.int32), oracle.sum2d_dim0(m).view(torch.int32))
+
+
+def _long_cases():
+    """Inputs long enough for the speculative rounds of the single-chain evaluation (2^22 elements
+    and more), built to make the rounds miss: sums that cross zero and many binades, that fall from
+    a large magnitude to a small one, that stop growing at a power of two, that pass through
+    infinities and NaNs, all-zero stretches, and lengths that fill the last block, node or
+    super-block only partly."""
+    r = _rng(31)
+    n = (1 << 22) + 12345
+    yield "uniform_pm1_ragged", gen.uniform_pm1(41, n).numpy()
+    yield "exactly_2^22", gen.uniform_pm1(42, 1 << 22).numpy()
+    yield "one_node_short", gen.uniform_pm1(43, (1 << 23) - 16384 + 7).numpy()
+    yield "normal_full_mantissa", r.standard_normal(n).astype(np.float32)
+    down = np.concatenate([[3.0e6], -np.abs(r.standard_normal(3_000_000)).astype(np.float32) * 1.2, r.standard_normal(1_500_000)])
+    yield "descent", down.astype(np.float32)
+    yield "stagnation_at_2^24", (0.25 + 0.75 * r.random(1 << 25)).astype(np.float32)
+    z = r.standard_normal(n).astype(np.float32)
+    z[1_000_000:1_300_000] = 0.0
+    z[2_000_000:2_000_064] = -0.0
+    yield "zero_stretches", z
+    w = r.standard_normal(n).astype(np.float32)
+    w[3_000_001] = np.inf
+    yield "inf_late", w
+    v = r.standard_normal(n).astype(np.float32)
+    v[2_500_000], v[2_500_777] = np.inf, -np.inf
+    yield "nan_midway", v
+    yield "scaled_normal", gen.scaled_normal(44, n).numpy()
+    yield "tiny_values", (r.standard_normal(n) * 2.0**-140).astype(np.float32)
+    yield "huge_values", (r.standard_normal(n) * 2.0**100).astype(np.float32)
+
+
+@pytest.mark.parametrize("name,x", list(_long_cases()), ids=[n for n, _ in _long_cases()])
+def test_sum1d_speculative_rounds(name, x):
+    from repdl_amd import ops
+
+    t = torch.from_numpy(np.ascontiguousarray(x))
+    got = ops.sum1d(t.cuda(), name == "descent").cpu()
+    want = oracle.sum1d(t, name == "descent")
+    assert got.view(torch.int32).item() == want.view(torch.int32).item() or (torch.isnan(got) and torch.isnan(want)), name
+
+
+def test_sum1d_long_unaligned_and_workspace():
+    """A long chain from a pointer 4 bytes off a 16-byte boundary, and the same through the entry point
+    that takes the caller's scratch memory (deliberately filled with junk first)."""
+    import ctypes
+
+    from repdl_amd import _lib, ops
+
+    n = (1 << 22) + 999
+    buf = gen.uniform_pm1(51, n + 1).cuda()
+    x = buf[1:]
+    assert x.data_ptr() % 16 != 0
+    want = oracle.sum1d(x.cpu())
+    assert torch.equal(ops.sum1d(x).cpu(), want)
+    nb = _lib.lib().repdl_hip_sum1d_workspace_bytes(n)
+    ws = torch.randint(0, 255, (nb,), dtype=torch.uint8, device="cuda")
+    out = torch.empty((), dtype=torch.float32, device="cuda")
+    for _ in range(2):  # the second call finds the first call's leftovers
+        _lib.call("repdl_hip_sum1d_ws", ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(out.data_ptr()), n, 0,
+                  ctypes.c_void_p(ws.data_ptr()), ctypes.c_size_t(nb), None)
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu(), want)

@@ -186,3 +186,140 @@ def test_composition_is_associative():
     for t in reversed(ts[:-1]):
         right = compose(t, right)
     assert left == right
+
+
+# ---- speculative rounds -------------------------------------------------------------------
+# The second stage of the GPU evaluation (sum1d.hip: sum1d_cand_walk_kernel, sum1d_compose_kernel,
+# sum1d_resolve_kernel), restated.  The chain is cut into nodes; for every node a TABLE holds the
+# exact exit state (a real float32 replay) for each of C candidate entry states, the C consecutive
+# float32 bit patterns around a predicted entry state.  Groups of nodes ("super-blocks") compose
+# their tables: exact where every intermediate state is again a candidate of the next node, and an
+# approximate offset (nearest candidate + the excess carried along) where not.  A serial resolver
+# runs the true state through the super-block tables while it finds it among the candidates; at
+# the first miss it keeps the exact state reached, continues with the approximate offsets to
+# predict the entry states of everything after, and the next round builds its tables around those.
+# Only exact table entries ever reach the result; what is left after the last round is summed
+# literally.
+
+def _bits(f):
+    return int(np.float32(f).view(np.uint32))
+
+
+def _flt(b):
+    return np.uint32(b & 0xFFFFFFFF).view(np.float32)
+
+
+def _window_base(centre_bits, C):
+    """C consecutive bit patterns around the centre, moved to stay inside its binade"""
+    lo, hi = centre_bits & 0xFF800000, centre_bits | 0x007FFFFF
+    base = lo if centre_bits - lo < C // 2 else centre_bits - C // 2
+    if hi - base < C - 1:
+        base = hi - (C - 1)
+    return base
+
+
+def _clamp_index(yb, base, C):
+    d = (yb - base) & 0xFFFFFFFF
+    if d < C:
+        return d, True
+    return (C - 1 if d < (1 << 31) else 0), False
+
+
+def speculative_sum(x, node=32, per_super=4, C=8, rounds=3):
+    n = len(x)
+    nnode = (n + node - 1) // node
+    nsup = (nnode + per_super - 1) // per_super
+    pred = np.concatenate([[0.0], np.cumsum(x.astype(np.float64))])  # the prediction: a binary64 prefix
+    with np.errstate(all="ignore"):
+        pred = np.nan_to_num(pred, nan=0.0, posinf=3e38, neginf=-3e38)
+
+    def table(nd, base):
+        seg = x[nd * node:(nd + 1) * node]
+        out = []
+        for k in range(C):
+            acc = _flt(base + k)
+            with np.errstate(all="ignore"):
+                for v in seg:
+                    acc = np.float32(acc + v)
+            out.append(_bits(acc))
+        return out
+
+    def chain(sa, nodes, bases, tabs):
+        """approximate state `sa` (a Python float) through `nodes`: nearest candidate, excess kept;
+        returns the final value, whether every step was an exact hit, and the state before each node"""
+        exact, before = True, []
+        for nd in nodes:
+            before.append(sa)
+            with np.errstate(all="ignore"):
+                f = np.float32(sa)
+            k, hit = _clamp_index(_bits(f), bases[nd], C)
+            cand = float(_flt(bases[nd] + k))
+            exact = exact and hit and float(f) == sa
+            with np.errstate(all="ignore"):
+                sa = float(_flt(tabs[nd][k])) + (sa - cand) if np.isfinite(sa - cand) else float(_flt(tabs[nd][k]))
+        return sa, exact, before
+
+    front, s_exact = 0, 0  # super-block index, state bits
+    centre = [float(np.float32(pred[min(j * per_super * node, n)])) for j in range(nsup)]
+    old_bases, old_tabs = None, None
+    stats = []
+    for _ in range(rounds):
+        if front >= nsup:
+            break
+        bases, tabs = {}, {}
+        for j in range(front, nsup):
+            nodes = [nd for nd in range(j * per_super, min((j + 1) * per_super, nnode))]
+            if old_tabs is None:
+                cs = [float(np.float32(pred[nd * node])) for nd in nodes]
+                cs[0] = centre[j]
+            else:
+                _, _, cs = chain(centre[j], nodes, old_bases, old_tabs)
+            for nd, c in zip(nodes, cs):
+                with np.errstate(all="ignore"):
+                    bases[nd] = _window_base(_bits(np.float32(c)), C)
+                tabs[nd] = table(nd, bases[nd])
+        # compose + resolve
+        s, exact, new_front, sa = s_exact, True, None, None
+        for j in range(front, nsup):
+            nodes = [nd for nd in range(j * per_super, min((j + 1) * per_super, nnode))]
+            if exact:
+                out, ok, _ = chain(float(_flt(s)), nodes, bases, tabs)
+                if ok and not np.isnan(out):
+                    s = _bits(np.float32(out))
+                    continue
+                if ok:  # NaN states: a hit with a NaN result (float(nan) != nan breaks `ok` upstream; keep exact bits)
+                    pass
+                exact, new_front, s_exact, sa = False, j, s, float(_flt(s))
+            centre[j] = sa
+            sa, _, _ = chain(sa, nodes, bases, tabs)
+        stats.append(front)
+        if exact:
+            front, s_exact = nsup, s
+        else:
+            front = new_front
+        old_bases, old_tabs = bases, tabs
+    # what the rounds did not resolve: literally
+    acc = _flt(s_exact)
+    with np.errstate(all="ignore"):
+        for v in x[front * per_super * node:]:
+            acc = np.float32(acc + v)
+    return _bits(acc), front, nsup
+
+
+@pytest.mark.parametrize("name,x", list(datasets()), ids=[n for n, _ in datasets()])
+def test_speculative_rounds_equal_sequential(name, x):
+    x = x[:2500]
+    for node, per_super, C, rounds in ((32, 4, 8, 3), (16, 2, 4, 6), (64, 4, 16, 1)):
+        got, front, nsup = speculative_sum(x, node, per_super, C, rounds)
+        want = sequential(x)
+        assert got == want or (np.isnan(_flt(got)) and np.isnan(_flt(want))), (name, node, C, rounds)
+
+
+def test_speculative_rounds_resolve_most_of_a_random_walk():
+    """On the benchmark's kind of data (zero-mean steps, the sum wanders across binade boundaries)
+    a few rounds resolve everything: nothing is left to the literal tail."""
+    r = _rng(5)
+    x = (r.integers(-2**23, 2**23, 20000) / 2.0**23).astype(np.float32)
+    got, front, nsup = speculative_sum(x, node=64, per_super=4, C=64, rounds=4)
+    assert got == sequential(x)
+    assert front == nsup
