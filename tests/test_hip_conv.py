@@ -34,6 +34,16 @@ FWD = [
     (40, 128, 15, 15, 128, 3, 3, 2, 2, 1, 1, 1),   # (forward only: its 15x15 input is too large for grad-input to take this route)
     (32, 128, 9, 9, 128, 5, 3, 2, 1, 2, 1, 1),     # strides in grad-input: input 9x9, output 5x9
     (32, 512, 8, 8, 128, 1, 1, 1, 1, 0, 0, 1),
+    # 3x3 at stride 1 on images 32 to 62 wide, channels in fours, rows in 64s: the input-patch kernel
+    (2, 64, 20, 40, 64, 3, 3, 1, 1, 1, 1, 1),      # 800 pixels: 6.25 tiles, tiles that start mid-row
+    (1, 8, 9, 33, 128, 3, 3, 1, 1, 0, 2, 1),       # two row tiles, no padding above / two columns left, 7x35 output
+    (3, 64, 35, 32, 64, 3, 3, 1, 1, 2, 0, 1),      # narrowest image: a tile spans five rows; output 37x30 (below 32: falls back)
+    (2, 12, 5, 62, 64, 3, 3, 1, 1, 1, 1, 1),       # widest image, three chunks of four channels, few rows
+    (1, 64, 34, 34, 64, 3, 3, 1, 1, 0, 0, 1),      # forward skips no tap (32x32 output), grad-input does
+    # 1x1 at stride 1 without padding on images of 1024 pixels and more: the kernel that streams both operands
+    (2, 32, 33, 40, 64, 1, 1, 1, 1, 0, 0, 1),      # 1320 pixels: 10.3 tiles
+    (1, 16, 32, 32, 128, 1, 1, 1, 1, 0, 0, 1),     # two row tiles forward, 16 channels: one step of the stream
+    (3, 64, 30, 45, 64, 1, 1, 1, 1, 0, 0, 1),      # 1350 pixels, the last tile half full
 ]
 
 
