@@ -215,15 +215,19 @@ __global__ __launch_bounds__(RT) void rowchain_kernel(const float *__restrict__ 
 // walks the current tile in LDS, lane = column, one ds_read_b128 and four dependent
 // v_add_f32 per four rows (a ds_read_b32 per row cost 14 clocks per row, this 9).
 // ---------------------------------------------------------------------------
-template <int CW, bool VEC>
+// NB = 2 (used when the workgroups are so few that each one's walk is the critical path): half-size
+// tiles in two LDS buffers, so that the walk never waits for the movers' stores -- one barrier per
+// tile, and the walking wave goes from one tile straight into the next.
+template <int CW, bool VEC, int NB>
 __global__ __launch_bounds__(320) void coltile_kernel(const float *__restrict__ in, float *__restrict__ out,
                                                       int64_t M, int64_t N, float factor)
 {
-    constexpr int TR = RTILE / CW;      // rows per tile
-    constexpr int C4 = CW / 4;          // float4 per tile row
-    constexpr int RV = RTILE / 4 / 256; // float4 per thread and tile
-    constexpr int TRP = TR + 4;         // LDS words per column (the pad spreads the walk's 16-byte reads over the banks)
-    __shared__ __attribute__((aligned(16))) float tile[CW * TRP]; // [column][row]: the walk reads four rows at once
+    constexpr int TFLOATS = RTILE / NB;  // floats per tile
+    constexpr int TR = TFLOATS / CW;     // rows per tile
+    constexpr int C4 = CW / 4;           // float4 per tile row
+    constexpr int RV = TFLOATS / 4 / 256; // float4 per thread and tile
+    constexpr int TRP = TR + 4;          // LDS words per column (the pad spreads the walk's 16-byte reads over the banks)
+    __shared__ __attribute__((aligned(16))) float tile[NB][CW * TRP]; // [column][row]: the walk reads four rows at once
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     constexpr int walker = 4; // waves 0-3 move the tiles, wave 4 only walks (as a mover too it walked 12.6 clocks per row)
@@ -266,16 +270,62 @@ __global__ __launch_bounds__(320) void coltile_kernel(const float *__restrict__ 
             stage[i] = v;
         }
     };
-    auto store = [&]() {
+    auto store = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < RV; i++)
         {
             const int idx = tid + 256 * i;
-            float *q = &tile[((idx % C4) << 2) * TRP + idx / C4]; // transposed on the way in
+            float *q = &tile[buf][((idx % C4) << 2) * TRP + idx / C4]; // transposed on the way in
             q[0 * TRP] = stage[i].x;
             q[1 * TRP] = stage[i].y;
             q[2 * TRP] = stage[i].z;
             q[3 * TRP] = stage[i].w;
+        }
+    };
+    auto walk = [&](int64_t t, int buf) {
+        const int64_t rem = M - t * TR; // rows of this tile that exist; the rest must not be added
+        const float *colp = &tile[buf][lane * TRP];
+        if (rem >= TR)
+        {
+            // 16 rows ahead: the reads of the next 16 are issued before the adds of these
+            const v4f *cp = reinterpret_cast<const v4f *>(colp);
+            v4f va[4], vb[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                va[u] = cp[u];
+            for (int r = 0; r < TR; r += 32)
+            {
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+                    vb[u] = cp[(r + 16) / 4 + u];
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+                {
+                    acc = acc + va[u].x;
+                    acc = acc + va[u].y;
+                    acc = acc + va[u].z;
+                    acc = acc + va[u].w;
+                }
+                if (r + 32 < TR)
+                {
+#pragma unroll
+                    for (int u = 0; u < 4; u++)
+                        va[u] = cp[(r + 32) / 4 + u];
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+                {
+                    acc = acc + vb[u].x;
+                    acc = acc + vb[u].y;
+                    acc = acc + vb[u].z;
+                    acc = acc + vb[u].w;
+                }
+            }
+        }
+        else
+        {
+            for (int r = 0; r < (int)rem; r++)
+                acc = acc + colp[r];
         }
     };
 
@@ -283,65 +333,36 @@ __global__ __launch_bounds__(320) void coltile_kernel(const float *__restrict__ 
     if (ntiles > 0 && mover)
     {
         load(0);
-        store();
+        store(0);
+        if (NB == 2 && ntiles > 1)
+            load(1);
     }
     __syncthreads();
     for (int64_t t = 0; t < ntiles; t++)
     {
-        const bool more = t + 1 < ntiles;
-        if (more && mover)
-            load(t + 1);
-        if (wave == walker && lane < CW)
+        if (NB == 2)
         {
-            const int64_t rem = M - t * TR; // rows of this tile that exist; the rest must not be added
-            const float *colp = &tile[lane * TRP];
-            if (rem >= TR)
-            {
-                // 16 rows ahead: the reads of the next 16 are issued before the adds of these
-                const v4f *cp = reinterpret_cast<const v4f *>(colp);
-                v4f va[4], vb[4];
-#pragma unroll
-                for (int u = 0; u < 4; u++)
-                    va[u] = cp[u];
-                for (int r = 0; r < TR; r += 32)
-                {
-#pragma unroll
-                    for (int u = 0; u < 4; u++)
-                        vb[u] = cp[(r + 16) / 4 + u];
-#pragma unroll
-                    for (int u = 0; u < 4; u++)
-                    {
-                        acc = acc + va[u].x;
-                        acc = acc + va[u].y;
-                        acc = acc + va[u].z;
-                        acc = acc + va[u].w;
-                    }
-                    if (r + 32 < TR)
-                    {
-#pragma unroll
-                        for (int u = 0; u < 4; u++)
-                            va[u] = cp[(r + 32) / 4 + u];
-                    }
-#pragma unroll
-                    for (int u = 0; u < 4; u++)
-                    {
-                        acc = acc + vb[u].x;
-                        acc = acc + vb[u].y;
-                        acc = acc + vb[u].z;
-                        acc = acc + vb[u].w;
-                    }
-                }
-            }
-            else
-            {
-                for (int r = 0; r < (int)rem; r++)
-                    acc = acc + colp[r];
-            }
+            // tile t + 1 (in registers since the previous round) into the other buffer, tile t + 2 requested
+            if (mover && t + 1 < ntiles)
+                store((int)((t + 1) & 1));
+            if (mover && t + 2 < ntiles)
+                load(t + 2);
+            if (wave == walker && lane < CW)
+                walk(t, (int)(t & 1));
+            __syncthreads(); // tile t + 1 is complete, the walk of tile t is over
         }
-        __syncthreads(); // the walk of tile t is over: the buffer may be overwritten
-        if (more && mover)
-            store();
-        __syncthreads();
+        else
+        {
+            const bool more = t + 1 < ntiles;
+            if (more && mover)
+                load(t + 1);
+            if (wave == walker && lane < CW)
+                walk(t, 0);
+            __syncthreads(); // the walk of tile t is over: the buffer may be overwritten
+            if (more && mover)
+                store(0);
+            __syncthreads();
+        }
     }
     if (wave == walker && lane < CW && col0 + lane < N)
         out[col0 + lane] = factor * acc;
@@ -465,20 +486,24 @@ REPDL_API int repdl_hip_sum2d_dim0(const float *in, float *out, int64_t M, int64
     const dim3 g((unsigned)grid);
     hipStream_t st = repdl_stream(stream);
     const float factor = repdl_sum_factor(average, M);
-#define REPDL_COLTILE(CWv)                                                                               \
-    do                                                                                                  \
-    {                                                                                                   \
-        if (vec)                                                                                        \
-            hipLaunchKernelGGL((coltile_kernel<CWv, true>), g, dim3(320), 0, st, in, out, M, N, factor); \
-        else                                                                                            \
-            hipLaunchKernelGGL((coltile_kernel<CWv, false>), g, dim3(320), 0, st, in, out, M, N, factor); \
+    // few workgroups, long columns: the walk of each is the critical path -- two LDS buffers
+    const bool two = grid <= 512 && M >= 4096;
+#define REPDL_COLTILE(CWv, NBv)                                                                               \
+    do                                                                                                       \
+    {                                                                                                        \
+        if (vec)                                                                                             \
+            hipLaunchKernelGGL((coltile_kernel<CWv, true, NBv>), g, dim3(320), 0, st, in, out, M, N, factor); \
+        else                                                                                                 \
+            hipLaunchKernelGGL((coltile_kernel<CWv, false, NBv>), g, dim3(320), 0, st, in, out, M, N, factor); \
     } while (0)
     if (cw == 64)
-        REPDL_COLTILE(64);
+        REPDL_COLTILE(64, 1);
     else if (cw == 32)
-        REPDL_COLTILE(32);
+        REPDL_COLTILE(32, 1);
+    else if (two)
+        REPDL_COLTILE(16, 2);
     else
-        REPDL_COLTILE(16);
+        REPDL_COLTILE(16, 1);
 #undef REPDL_COLTILE
     return repdl_launch_status();
 }
