@@ -50,7 +50,7 @@ TRAFFIC_JSON = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 # --write-traffic.  The first entry is the leg's anchor: it runs exactly once per call, so the
 # number of calls in a profiled run is its dispatch count.
 LEG_KERNELS = {
-    "mm": ["mm_mfma_fast_kernel<false, true, 4, 2, 2, 4"],
+    "mm": ["mm_dma_kernel<false, true, 4, 2, 2, 4"],
     "mm_fma": ["mm_kernel<false, true"],
     "sum2d_dim1": ["rowchain_kernel"],
     "sum2d_dim0": ["coltile_kernel"],
@@ -121,7 +121,7 @@ def write_traffic(fetch_dir: str, write_dir: str) -> None:
         hits = [(k, v) for (k, c), v in agg.items() if c == counter and sub in k]
         return hits
 
-    probe = "vectorized_elementwise_kernel"
+    probe = "trunc"
     pf, pw = mean_of(fetch, probe, "FETCH_SIZE"), mean_of(write, probe, "WRITE_SIZE")
     if not pf or not pw:
         raise SystemExit("the copy-probe kernel is missing from the counter runs (run bench.py with --copy-probe)")
@@ -139,7 +139,7 @@ def write_traffic(fetch_dir: str, write_dir: str) -> None:
         detail[leg] = {"read_bytes_per_call": round(rd), "written_bytes_per_call": round(wr), "calls_profiled": calls_f}
     out = {"source": "rocprofv3 --pmc FETCH_SIZE / --pmc WRITE_SIZE over `bench.py --copy-probe`, one run per counter",
            "calibration": {"fetch_bytes_per_count": f_unit, "write_bytes_per_count": w_unit,
-                           "probe": "torch.add(x, 0) on 2^28 floats: 1 GiB read, 1 GiB written per dispatch"},
+                           "probe": "torch.trunc(x, out=y) on 2^28 floats: 1 GiB read, 1 GiB written per dispatch"},
            "bytes_per_call": legs, "detail": detail}
     with open(TRAFFIC_JSON, "w") as f:
         json.dump(out, f, indent=1, sort_keys=True)
@@ -242,7 +242,7 @@ def main() -> int:
                                                "exp,log,sqrt,div,loss,conv,linear,adam,cnn)")
     ap.add_argument("--size", type=int, default=8192, help="mm size (M=N=K); the metric is quoted at 8192")
     ap.add_argument("--copy-probe", action="store_true",
-                    help="also run a plain 1 GiB elementwise copy kernel (torch.add(x, 0)), the known-size kernel "
+                    help="also run a plain 1 GiB elementwise kernel (torch.trunc(x, out=y)), the known-size kernel "
                          "against which FETCH_SIZE / WRITE_SIZE counters are calibrated")
     ap.add_argument("--summarise-trace", metavar="DIR")
     ap.add_argument("--summarise-counters", metavar="DIR", nargs="+")
@@ -331,8 +331,8 @@ def main() -> int:
     del y_gpu, out_holder
 
     if _lib.lib().repdl_hip_matrix_path() == 1:
-        kernel_name = "mm_mfma_fast_kernel<NT, 256x256x16 tile, 512 threads>"
-        kernel_note = ("fp32 matrix-instruction peak; v_mfma_f32_32x32x2_f32, checked on this device to be a "
+        kernel_name = "mm_dma_kernel<NT, 128x128x16 tile, 512 threads, operands DMA'd global->LDS>"
+        kernel_note = ("fp32 matrix-instruction peak; v_mfma_f32_16x16x4_f32, checked on this device to be a "
                        "k-ascending chain of single-rounding FMAs before use")
     else:
         kernel_name = "mm_kernel<NT>"
@@ -658,7 +658,7 @@ def main() -> int:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)
         for _ in range(3):
-            torch.add(src, 0.0, out=dst)  # an elementwise kernel: reads 1 GiB, writes 1 GiB
+            torch.trunc(src, out=dst)  # an elementwise kernel no leg uses: reads 1 GiB, writes 1 GiB
         torch.cuda.synchronize()
 
     print(json.dumps(result))

@@ -6,11 +6,13 @@
 // operands are staged are free; the order along K is not, so K is never split
 // across threads.
 //
-// Two kernels implement it.  mm_mfma_kernel feeds v_mfma_f32_32x32x2_f32, which on
-// gfx950 evaluates exactly such a chain (two k per instruction, ascending; checked
-// on the device before first use, see mfma_check.hip).  mm_kernel is the same
-// computation with one v_fma_f32 per term; it runs when that check fails or the
-// matrix path is switched off.
+// Three families of kernels implement it.  The matrix-instruction kernels feed
+// v_mfma_f32_16x16x4_f32 (mm_dma_kernel: whole-tile shapes, operands moved from global memory
+// straight into LDS) or v_mfma_f32_32x32x2_f32 (mm_mfma_fast_kernel, mm_mfma_kernel: tile edges,
+// K tails, unaligned operands), which on gfx950 evaluate exactly such a chain (four or two k per
+// instruction, ascending; checked on the device before first use, see mfma_check.hip).
+// mm_kernel is the same computation with one v_fma_f32 per term; it runs when that check
+// fails or the matrix path is switched off.
 //
 // mm_kernel layout: a workgroup of 256 threads computes a 128x128 tile of C; each thread
 // an 8x8 micro-tile held in registers (rows ty*4+{0..3} and 64+ty*4+{0..3},
@@ -801,6 +803,255 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_fast_kernel(const float
         }
 }
 
+// ---------------------------------------------------------------------------------------------
+// mm_dma_kernel: whole-tile shapes with 16-byte aligned operands.
+//
+// The operands never pass through registers on their way to LDS: global_load_lds_dwordx4 moves 16
+// bytes per lane from global memory straight into LDS, at consecutive lanes' consecutive 16-byte
+// slots from an LDS base in M0.  So the layout of a k-tile in LDS is whatever order the lanes are
+// given, and both operand orientations have an order that the matrix instruction can read without
+// bank conflicts.  The instruction is v_mfma_f32_16x16x4_f32: lane l supplies row (column) l%16 of
+// its 16-row block at k = 4q + l/16 and the instruction adds k = 4q .. 4q+3 in ascending order.  A
+// k-tile is NQ such quads.  With T = rows of C (A operand) or columns of C (B operand) per tile:
+//
+//   k contiguous in memory (A of NN/NT, B of NT/TT): lane -> (row r, quad q), 16 bytes = 4 consecutive
+//     k of one row; LDS word q*4T + 4r + k%4.  A lane of the matrix instruction reads word
+//     q*4T + 4r + l/16: 64 lanes, 64 banks.
+//   r contiguous in memory (A of TN/TT, B of NN/TN): lane -> (k%4, group of 4 rows), 16 bytes = 4
+//     consecutive rows at one k; LDS word q*4T + 16(r/4) + 4(k%4) + r%4, again one bank per lane.
+//
+// NB >= 3 LDS buffers per operand.  Quad by quad a wave reads its operands D quads ahead of the
+// matrix instructions that use them (a ring of D+1 register sets); the one barrier per k-tile sits
+// D quads before the tile's end, where the next tile's first reads begin, and is followed by the
+// DMA of the tile NB-1 ahead into the buffer whose reads ended a whole tile ago -- so nobody waits
+// on LDS reads at the barrier, and a DMA has NB-2 tiles of matrix work to land in (small tiles need
+// several: a 64x64x32 tile is 0.4 us of matrix work, less than one trip to HBM).  The loop holds no
+// vector ALU instruction at all.
+__device__ __forceinline__ void dma16(const void *base, uint32_t voff, uint32_t lds_byte)
+{
+    // M0 = LDS byte address of lane 0's slot
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(base), "s"(lds_byte)
+                 : "memory", "m0");
+}
+
+template <bool TA, bool TB, int FM, int FN, int WGM, int WGN, int NQ, int D, int NB>
+__global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__restrict__ A, const float *__restrict__ B,
+                                                               float *__restrict__ C, const float *__restrict__ bias,
+                                                               int64_t M, int64_t N, int64_t K, int64_t gx, int64_t gy,
+                                                               int64_t ntiles8)
+{
+    constexpr int NW = WGM * WGN;
+    constexpr int TM = 16 * FM * WGM, TN = 16 * FN * WGN;
+    constexpr bool A_KC = !TA, B_KC = TB;
+    constexpr int QSA = 4 * TM, QSB = 4 * TN;     // LDS words per quad
+    constexpr int OPA = NQ * QSA, OPB = NQ * QSB; // LDS words per k-tile
+    constexpr int R = D + 1;                      // register sets in the ring
+    static_assert(NQ % R == 0 && D >= 1 && D < NQ, "ring must divide the k-tile");
+    static_assert(NB >= 3, "a buffer being read, one landed or landing, one being filled");
+    static_assert((TM * NQ) % 64 == 0 && (TN * NQ) % 64 == 0, "a DMA instruction fills 64 slots");
+    constexpr int NIA = TM * NQ / 64, NIB = TN * NQ / 64; // DMA instructions per k-tile
+    constexpr int CA = (NIA + NW - 1) / NW, CB = (NIB + NW - 1) / NW;
+    static_assert(NB == 3 || (NIA % NW == 0 && NIB % NW == 0), "every wave must issue the same number of loads per tile");
+    constexpr int INFLIGHT = (NB - 3) * (CA + CB); // loads of later tiles that may still be under way at a barrier
+    static_assert(INFLIGHT < 64, "vmcnt is a 6-bit counter");
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    extern __shared__ __attribute__((aligned(16))) float smem[]; // [NB][OPA] then [NB][OPB]
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave % WGM, wn = wave / WGM;
+    const int l16 = lane & 15, g = lane >> 4;
+
+    int64_t tile = blockIdx.x;
+    if (tile < ntiles8)
+        tile = (tile & 7) * (ntiles8 >> 3) + (tile >> 3);
+    const int64_t group_sz = (int64_t)GROUP_M * gx;
+    const int64_t group = tile / group_sz;
+    const int64_t first_row = group * GROUP_M;
+    const int64_t rows_here = (gy - first_row < GROUP_M) ? gy - first_row : GROUP_M;
+    const int64_t in_group = tile - group * group_sz;
+    const int64_t trow = first_row + in_group % rows_here, tcol = in_group / rows_here;
+    const int64_t m0 = trow * TM, n0 = tcol * TN;
+    const int64_t lda = TA ? M : K, ldb = TB ? K : N;
+
+    // DMA instruction e of an operand with T rows: 64 consecutive 16-byte slots of the tile's LDS
+    // image, i.e. slots [64e, 64e+64) of NQ*T; slot s = quad (s / T), position w = s % T in the quad.
+    uint32_t va[CA], vb[CB];
+    uint32_t la[CA], lb[CB];
+#pragma unroll
+    for (int t = 0; t < CA; t++)
+    {
+        const int e = wave + NW * t, s = 64 * e + lane, q = s / TM, w = s % TM;
+        va[t] = A_KC ? (uint32_t)(((int64_t)w * lda + 4 * q) * 4) : (uint32_t)(((int64_t)(4 * q + (w & 3)) * lda + (w & ~3)) * 4);
+        la[t] = __builtin_amdgcn_readfirstlane(64 * e * 16);
+    }
+#pragma unroll
+    for (int t = 0; t < CB; t++)
+    {
+        const int e = wave + NW * t, s = 64 * e + lane, q = s / TN, w = s % TN;
+        vb[t] = B_KC ? (uint32_t)(((int64_t)w * ldb + 4 * q) * 4) : (uint32_t)(((int64_t)(4 * q + (w & 3)) * ldb + (w & ~3)) * 4);
+        lb[t] = __builtin_amdgcn_readfirstlane(NB * OPA * 4 + 64 * e * 16);
+    }
+    const char *a_base = reinterpret_cast<const char *>(A_KC ? A + m0 * lda : A + m0);
+    const char *b_base = reinterpret_cast<const char *>(B_KC ? B + n0 * ldb : B + n0);
+    const int64_t a_step = (A_KC ? (int64_t)(4 * NQ) : (int64_t)(4 * NQ) * lda) * 4;
+    const int64_t b_step = (B_KC ? (int64_t)(4 * NQ) : (int64_t)(4 * NQ) * ldb) * 4;
+    auto issue = [&](int buf) {
+#pragma unroll
+        for (int t = 0; t < CA; t++)
+            if (NIA % NW == 0 || wave + NW * t < NIA)
+                dma16(a_base, va[t], la[t] + buf * OPA * 4);
+#pragma unroll
+        for (int t = 0; t < CB; t++)
+            if (NIB % NW == 0 || wave + NW * t < NIB)
+                dma16(b_base, vb[t], lb[t] + buf * OPB * 4);
+        a_base += a_step;
+        b_base += b_step;
+    };
+
+    v4f acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+            acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    const int ma = wm * 16 * FM + l16, nb = wn * 16 * FN + l16;
+    const float *ra = smem + (A_KC ? 4 * ma + g : 16 * (ma >> 2) + 4 * g + (ma & 3));
+    const float *rb = smem + NB * OPA + (B_KC ? 4 * nb + g : 16 * (nb >> 2) + 4 * g + (nb & 3));
+    float xa[R][FM], xb[R][FN];
+    auto read_q = [&](int buf, int q, float(&a)[FM], float(&b)[FN]) {
+#pragma unroll
+        for (int i = 0; i < FM; i++)
+            a[i] = ra[buf * OPA + q * QSA + 64 * i];
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+            b[j] = rb[buf * OPB + q * QSB + 64 * j];
+    };
+    auto mfma_q = [&](float(&a)[FM], float(&b)[FN]) {
+#pragma unroll
+        for (int i = 0; i < FM; i++)
+#pragma unroll
+            for (int j = 0; j < FN; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], b[j], acc[i][j], 0, 0, 0);
+    };
+
+    const int64_t nkt = K / (4 * NQ);
+    if (nkt > 0)
+    {
+#pragma unroll
+        for (int u = 0; u < NB - 1; u++)
+            if (u < nkt)
+                issue(u);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < D; q++)
+            read_q(0, q, xa[q], xb[q]);
+    }
+    for (int64_t kt = 0; kt < nkt; kt += NB)
+    {
+#pragma unroll
+        for (int u = 0; u < NB; u++)
+        {
+            if (kt + u >= nkt)
+                break;
+            const bool more1 = kt + u + 1 < nkt, more_dma = kt + u + NB - 1 < nkt;
+#pragma unroll
+            for (int q = 0; q < NQ; q++)
+            {
+                if (q == NQ - D)
+                {
+                    // the next tile (this wave's share) has landed; after the barrier everyone's has,
+                    // and every read of the tile before this one has long been consumed
+                    if (INFLIGHT > 0 && kt + u + NB - 2 < nkt)
+                        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(INFLIGHT) : "memory");
+                    else
+                        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    __builtin_amdgcn_s_barrier();
+                    asm volatile("" ::: "memory");
+                    if (more_dma)
+                        issue((u + NB - 1) % NB);
+                }
+                const int qq = q + D;
+                if (qq < NQ)
+                    read_q(u, qq, xa[qq % R], xb[qq % R]);
+                else if (more1)
+                    read_q((u + 1) % NB, qq - NQ, xa[qq % R], xb[qq % R]);
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_q(xa[q % R], xb[q % R]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+
+    // bias: one rounded add per output after its chain; a lane owns FN columns
+    float bv[FN];
+#pragma unroll
+    for (int j = 0; j < FN; j++)
+        bv[j] = bias != nullptr ? bias[n0 + wn * 16 * FN + 16 * j + l16] : 0.0f;
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+        {
+            const int64_t m = m0 + wm * 16 * FM + 16 * i + 4 * g + r;
+#pragma unroll
+            for (int j = 0; j < FN; j++)
+            {
+                const int64_t nn = n0 + wn * 16 * FN + 16 * j + l16;
+                __builtin_nontemporal_store(bias != nullptr ? acc[i][j][r] + bv[j] : acc[i][j][r], &C[m * N + nn]);
+            }
+        }
+}
+
+// Whether mm_dma_kernel with this tile can take the product, and its launch.
+template <int FM, int FN, int WGM, int WGN, int NQ>
+bool dma_applies(int64_t M, int64_t N, int64_t K, int transA, int transB, int avec, int bvec)
+{
+    constexpr int TM = 16 * FM * WGM, TN = 16 * FN * WGN, BKQ = 4 * NQ;
+    if (!avec || !bvec || M % TM || N % TN || K % BKQ || K < BKQ)
+        return false;
+    const int64_t lda = transA ? M : K, ldb = transB ? K : N;
+    // per-lane byte offsets inside an operand tile are 32-bit
+    const int64_t ea = transA ? (int64_t)BKQ * lda + TM : (int64_t)TM * lda + BKQ;
+    const int64_t eb = transB ? (int64_t)TN * ldb + BKQ : (int64_t)BKQ * ldb + TN;
+    return ea * 4 < (1LL << 32) && eb * 4 < (1LL << 32) && (M / TM) * (N / TN) <= REPDL_I32_MAX;
+}
+
+template <bool TA, bool TB, int FM, int FN, int WGM, int WGN, int NQ, int D, int NB>
+int launch_dma_t(const float *A, const float *B, float *C, const float *bias, int64_t M, int64_t N, int64_t K, hipStream_t s)
+{
+    constexpr int TM = 16 * FM * WGM, TN = 16 * FN * WGN;
+    constexpr size_t shmem = (size_t)NB * NQ * 4 * (TM + TN) * sizeof(float);
+    static_assert(shmem <= 160 * 1024, "LDS of one CU");
+    const int64_t gx = N / TN, gy = M / TM;
+    const int64_t ntiles8 = (gx * gy) & ~(int64_t)7;
+    auto kern = &mm_dma_kernel<TA, TB, FM, FN, WGM, WGN, NQ, D, NB>;
+    if (shmem > 48 * 1024)
+    {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)shmem);
+        if (e != hipSuccess)
+            return (int)e;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)(gx * gy)), dim3(64 * WGM * WGN), shmem, s, A, B, C, bias, M, N, K, gx, gy, ntiles8);
+    return repdl_launch_status();
+}
+
+template <int FM, int FN, int WGM, int WGN, int NQ, int D, int NB>
+int launch_dma(const float *A, const float *B, float *C, const float *bias, int64_t M, int64_t N, int64_t K, int transA,
+               int transB, hipStream_t s)
+{
+    if (!transA && !transB)
+        return launch_dma_t<false, false, FM, FN, WGM, WGN, NQ, D, NB>(A, B, C, bias, M, N, K, s);
+    if (transA && !transB)
+        return launch_dma_t<true, false, FM, FN, WGM, WGN, NQ, D, NB>(A, B, C, bias, M, N, K, s);
+    if (!transA && transB)
+        return launch_dma_t<false, true, FM, FN, WGM, WGN, NQ, D, NB>(A, B, C, bias, M, N, K, s);
+    return launch_dma_t<true, true, FM, FN, WGM, WGN, NQ, D, NB>(A, B, C, bias, M, N, K, s);
+}
+
 template <bool TA, bool TB, int FM, int FN, int WGM, int WGN>
 int launch_mfma_t(const float *A, const float *B, float *C, const float *bias, int64_t M, int64_t N, int64_t K, int avec,
                   int bvec, hipStream_t s)
@@ -882,7 +1133,64 @@ REPDL_API int repdl_hip_mm_bias(const float *A, const float *B, const float *bia
     hipStream_t s = repdl_stream(stream);
     if (repdl_mfma_exact())
     {
-        // Tile choice.  A CU runs its tiles one after the other (256x256: one workgroup fills it) or
+        // Whole-tile shapes with aligned operands: mm_dma_kernel.  Its configurations, with the share
+        // of the chip's matrix rate (145 TFLOP/s on the 128x128 tile with many tiles per CU) each was
+        // measured at, by tiles per CU r (a CU holds up to three workgroups of either tile at once):
+        //   128x128, 8 waves of 64x32, k-tile 16:   r = 1 0.76, 2 0.92, 3 0.97, more 0.99
+        //   64x64, 4 waves of 32x32, k-tile 32/16:  r = 1 0.60, 2 0.76, 3..5 0.83, 6..11 0.89, more 0.94
+        //   64x16 or 16x64, 4 waves of 16x16, k-tile 64, five buffers: 0.35 (one 16x16 block per SIMD is
+        //     a chain of dependent instructions; for C with fewer 64x64 tiles than CUs)
+        // (8192^3 NT: 145 / 138 TFLOP/s on the first two; 3072^2 x 4096: 108 / 129; 2048^3: 110 / 121;
+        // 1536^2 x 4096: 75 / 96; 1024^3: - / 87; 64 x 4096 x 4096: 28 on 64x64, 51 on 64x16.)
+        if (avec && bvec)
+        {
+            auto rounds = [&](int64_t tm, int64_t tn) { return repdl_cdiv((M / tm) * (N / tn), 256); };
+            double best = 1e300;
+            int pick = 0;
+            if (dma_applies<4, 2, 2, 4, 4>(M, N, K, transA, transB, avec, bvec))
+            {
+                const int64_t r = rounds(128, 128);
+                const double c = (double)r * 16384.0 / (r >= 4 ? 0.99 : r == 3 ? 0.97 : r == 2 ? 0.92 : 0.76);
+                if (c < best)
+                    best = c, pick = 1;
+            }
+            if (dma_applies<2, 2, 2, 2, 4>(M, N, K, transA, transB, avec, bvec))
+            {
+                const int64_t r = rounds(64, 64);
+                const double c = (double)r * 4096.0 / (r >= 12 ? 0.94 : r >= 6 ? 0.89 : r >= 3 ? 0.83 : r == 2 ? 0.76 : 0.60);
+                // the deeper k-tile pays when a CU has one workgroup; the shallower one lets six share a CU
+                if (c < best)
+                    best = c, pick = (r == 1 && dma_applies<2, 2, 2, 2, 8>(M, N, K, transA, transB, avec, bvec)) ? 2 : 3;
+            }
+            if (dma_applies<1, 1, 4, 1, 16>(M, N, K, transA, transB, avec, bvec))
+            {
+                const double c = (double)rounds(64, 16) * 1024.0 / 0.35;
+                if (c < best)
+                    best = c, pick = 4;
+            }
+            else if (dma_applies<1, 1, 1, 4, 16>(M, N, K, transA, transB, avec, bvec))
+            {
+                const double c = (double)rounds(16, 64) * 1024.0 / 0.35;
+                if (c < best)
+                    best = c, pick = 5;
+            }
+            switch (pick)
+            {
+            case 1:
+                return launch_dma<4, 2, 2, 4, 4, 1, 3>(A, B, C, bias, M, N, K, transA, transB, s);
+            case 2:
+                return launch_dma<2, 2, 2, 2, 8, 1, 3>(A, B, C, bias, M, N, K, transA, transB, s);
+            case 3:
+                return launch_dma<2, 2, 2, 2, 4, 1, 3>(A, B, C, bias, M, N, K, transA, transB, s);
+            case 4:
+                return launch_dma<1, 1, 4, 1, 16, 7, 5>(A, B, C, bias, M, N, K, transA, transB, s);
+            case 5:
+                return launch_dma<1, 1, 1, 4, 16, 7, 5>(A, B, C, bias, M, N, K, transA, transB, s);
+            default:
+                break;
+            }
+        }
+        // Every other shape: the kernels that stage operands through registers.  A CU runs its tiles one after the other (256x256: one workgroup fills it) or
         // side by side (smaller tiles), so a configuration costs (most tiles on any CU) x tile area
         // / rate, with the rates measured per configuration and tiles per CU, relative to the
         // 256x256 tile (135 TFLOP/s chip-wide): 128x128 0.785 alone on its CU, 0.92 with two, 0.955

@@ -23,6 +23,40 @@ def test_layouts_and_edges(shape, tA, tB):
     assert torch.equal(got, oracle.mm(a, b, bool(tA), bool(tB)))
 
 
+# Whole-tile shapes with aligned operands take the kernels that move operands from global memory
+# straight into LDS; one shape per tile configuration (128x128; 64x64 with the shallow and the
+# deep k-tile; 64x16; 16x64), each in all four layouts.
+WHOLE_TILE_SHAPES = [(4096, 4096, 48), (2048, 2048, 80), (512, 512, 96), (512, 512, 48), (64, 1024, 128), (48, 1024, 192),
+                     (256, 192, 128), (128, 128, 2048)]
+
+
+@pytest.mark.parametrize("tA,tB", [(0, 0), (1, 0), (0, 1), (1, 1)])
+@pytest.mark.parametrize("shape", WHOLE_TILE_SHAPES, ids=str)
+def test_whole_tile_shapes(shape, tA, tB):
+    """Operands with zeros of both signs, subnormals, huge and tiny magnitudes and infinities
+    (NaN results only have to be NaN), then well-scaled operands with a bias."""
+    from repdl_amd import ops
+
+    M, N, K = shape
+    a = gen.elementwise_mix(M + 3 * K, M * K).view((K, M) if tA else (M, K))
+    b = gen.elementwise_mix(N + 5 * K, N * K).view((N, K) if tB else (K, N))
+    a = torch.where(torch.isnan(a), torch.zeros_like(a), a)
+    b = torch.where(torch.isnan(b), torch.full_like(b, -0.0), b)
+    got = ops.mm(a.cuda(), b.cuda(), bool(tA), bool(tB)).cpu()
+    assert _same_bits_or_both_nan(got, oracle.mm(a, b, bool(tA), bool(tB)))
+    a = gen.scaled_normal(M * 7 + K, *((K, M) if tA else (M, K)), lo=-6, hi=6)
+    b = gen.normal_like(N * 3 + K, *((N, K) if tB else (K, N)))
+    bias = gen.scaled_normal(N + 1, N, lo=-30, hi=30)
+    bias[::5] = 0.0
+    bias[1::7] = -0.0
+    want = oracle.mm(a, b, bool(tA), bool(tB))
+    got = ops.mm(a.cuda(), b.cuda(), bool(tA), bool(tB)).cpu()
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+    want += bias
+    got = ops.mm_bias(a.cuda(), b.cuda(), bias.cuda(), bool(tA), bool(tB)).cpu()
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+
+
 @pytest.mark.parametrize("tA,tB", [(0, 1), (0, 0), (1, 0), (1, 1)])
 @pytest.mark.parametrize("shape", SHAPES + [(512, 768, 256), (300, 1000, 64)], ids=str)
 def test_bias_in_the_epilogue(shape, tA, tB):
