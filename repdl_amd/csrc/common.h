@@ -50,6 +50,15 @@ int repdl_sum_chains(const float *in, float *out, int64_t rows, int64_t nseg, in
 // the GEMM-shaped operators then use them, otherwise their v_fma_f32 kernels.
 bool repdl_mfma_exact();
 
+// mm.hip: a batch of `nbatch` products C_b[M][N] = op(A_b)[M][K] . op(B_b)[K][N] on the kernel that moves
+// operands from global memory straight into LDS; operand b lies `stride` elements behind operand b-1
+// (0: one operand shared by all).  row_bias[M], if not null, is added to every column of C after the
+// chains.  REPDL_E_UNSUPPORTED, and nothing launched, where that kernel cannot take the operands
+// (rows off 16-byte boundaries, the matrix path switched off).
+int repdl_mm_batched(const float *A, const float *B, float *C, const float *row_bias, int64_t M, int64_t N, int64_t K,
+                     int transA, int transB, int64_t nbatch, int64_t strideA, int64_t strideB, int64_t strideC,
+                     hipStream_t stream);
+
 __device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
 __device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
 

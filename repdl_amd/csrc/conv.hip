@@ -2235,6 +2235,20 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
     const bool mfma = repdl_mfma_exact();
     if (mfma && patch::applies<MODE>(d, kernel))
         return patch::launch<MODE>(gathered, kernel, out, d, s);
+    // (chains of 64 terms or fewer: the streaming kernel, which has no prologue to fill -- batch 64,
+    // 56x56, 64 channels in, 256 out: 0.087 against 0.098 ms)
+    const bool short_chain = K <= 64 && point::applies<MODE>(d);
+    if (mfma && !short_chain && d.groups == 1 && KHW == 1 && d.sH == 1 && d.sW == 1 && d.pH == 0 && d.pW == 0)
+    {
+        // a 1x1 kernel at stride 1: per image Out[M][P] = A[M][C] . Src[C][P], A = W (forward) or W^T
+        // (grad-input) -- a batch of plain products, and the reference skips no tap here (batch 64:
+        // 512 -> 128 at 28x28 0.096 -> 0.072 ms, 1024 -> 256 at 14x14 0.119 -> 0.080, 256 -> 64 at 56x56
+        // 0.079 -> 0.072)
+        const int rc = repdl_mm_batched(kernel, gathered, out, MODE == MODE_FWD ? d.bias : nullptr, M, P, K, MODE == MODE_DGRAD, 0,
+                                        d.N, 0, (int64_t)K * P, (int64_t)M * P, s);
+        if (rc != REPDL_E_UNSUPPORTED)
+            return rc;
+    }
     if (mfma && point::applies<MODE>(d))
         return point::launch<MODE>(gathered, kernel, out, d, s);
     const int64_t gathered_count =

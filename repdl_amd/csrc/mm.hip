@@ -7,9 +7,9 @@
 // across threads.
 //
 // Three families of kernels implement it.  The matrix-instruction kernels feed
-// v_mfma_f32_16x16x4_f32 (mm_dma_kernel: whole-tile shapes, operands moved from global memory
-// straight into LDS) or v_mfma_f32_32x32x2_f32 (mm_mfma_fast_kernel, mm_mfma_kernel: tile edges,
-// K tails, unaligned operands), which on gfx950 evaluate exactly such a chain (four or two k per
+// v_mfma_f32_16x16x4_f32 (mm_dma_kernel: operand rows on 16-byte boundaries, moved from global
+// memory straight into LDS) or v_mfma_f32_32x32x2_f32 (mm_mfma_fast_kernel, mm_mfma_kernel: every
+// other operand, staged through registers), which on gfx950 evaluate exactly such a chain (four or two k per
 // instruction, ascending; checked on the device before first use, see mfma_check.hip).
 // mm_kernel is the same computation with one v_fma_f32 per term; it runs when that check
 // fails or the matrix path is switched off.
@@ -804,7 +804,7 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_fast_kernel(const float
 }
 
 // ---------------------------------------------------------------------------------------------
-// mm_dma_kernel: whole-tile shapes with 16-byte aligned operands.
+// mm_dma_kernel: operands whose rows start on 16-byte boundaries, any M, N, K; a batch of products.
 //
 // The operands never pass through registers on their way to LDS: global_load_lds_dwordx4 moves 16
 // bytes per lane from global memory straight into LDS, at consecutive lanes' consecutive 16-byte
@@ -827,6 +827,18 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_fast_kernel(const float
 // on LDS reads at the barrier, and a DMA has NB-2 tiles of matrix work to land in (small tiles need
 // several: a 64x64x32 tile is 0.4 us of matrix work, less than one trip to HBM).  The loop holds no
 // vector ALU instruction at all.
+//
+// Edges.  A tile that hangs over the lower or right edge of C loads, for the rows it does not have,
+// the operand's last rows again (the lane's address is clamped once, before the loop) and never
+// stores what it computes from them.  A last k-tile of fewer than NQ quads is loaded with the lanes
+// of the missing quads switched off and runs that many quads.  The up to three k past the last
+// whole quad are added afterwards with one v_fma_f32 per term and output, operands read straight
+// from global memory: the same chain step as the matrix instruction's.  So nothing is padded and
+// no accumulator that is -0 is touched.
+//
+// Batch: blockIdx.y selects one of several products with the same shapes, operand b at X + b * stride
+// (stride 0: shared by all).  `cbias` is added per column, `rbias` per row (one rounded addition after
+// the chain, whichever is given; at most one is).
 __device__ __forceinline__ void dma16(const void *base, uint32_t voff, uint32_t lds_byte)
 {
     // M0 = LDS byte address of lane 0's slot
@@ -834,11 +846,16 @@ __device__ __forceinline__ void dma16(const void *base, uint32_t voff, uint32_t 
                  : "memory", "m0");
 }
 
+struct MmBatch
+{
+    int64_t a, b, c; // elements between consecutive products' operands and results
+};
+
 template <bool TA, bool TB, int FM, int FN, int WGM, int WGN, int NQ, int D, int NB>
 __global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__restrict__ A, const float *__restrict__ B,
-                                                               float *__restrict__ C, const float *__restrict__ bias,
-                                                               int64_t M, int64_t N, int64_t K, int64_t gx, int64_t gy,
-                                                               int64_t ntiles8)
+                                                               float *__restrict__ C, const float *__restrict__ cbias,
+                                                               const float *__restrict__ rbias, int64_t M, int64_t N,
+                                                               int64_t K, int64_t gx, int64_t gy, int64_t ntiles8, MmBatch batch)
 {
     constexpr int NW = WGM * WGN;
     constexpr int TM = 16 * FM * WGM, TN = 16 * FN * WGN;
@@ -873,38 +890,76 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__re
     const int64_t trow = first_row + in_group % rows_here, tcol = in_group / rows_here;
     const int64_t m0 = trow * TM, n0 = tcol * TN;
     const int64_t lda = TA ? M : K, ldb = TB ? K : N;
+    A += (int64_t)blockIdx.y * batch.a;
+    B += (int64_t)blockIdx.y * batch.b;
+    C += (int64_t)blockIdx.y * batch.c;
 
     // DMA instruction e of an operand with T rows: 64 consecutive 16-byte slots of the tile's LDS
     // image, i.e. slots [64e, 64e+64) of NQ*T; slot s = quad (s / T), position w = s % T in the quad.
+    // Rows past the operand's last are clamped to rows it has.
     uint32_t va[CA], vb[CB];
     uint32_t la[CA], lb[CB];
+    const int64_t am = M - m0, bn = N - n0; // rows (columns) of C this tile really has, if fewer than the tile's
 #pragma unroll
     for (int t = 0; t < CA; t++)
     {
         const int e = wave + NW * t, s = 64 * e + lane, q = s / TM, w = s % TM;
-        va[t] = A_KC ? (uint32_t)(((int64_t)w * lda + 4 * q) * 4) : (uint32_t)(((int64_t)(4 * q + (w & 3)) * lda + (w & ~3)) * 4);
+        if (A_KC)
+        {
+            const int64_t r = w < am ? w : am - 1;
+            va[t] = (uint32_t)((r * lda + 4 * q) * 4);
+        }
+        else
+        {
+            const int64_t r = (w & ~3) + 3 < am ? (w & ~3) : am - 4;
+            va[t] = (uint32_t)(((int64_t)(4 * q + (w & 3)) * lda + r) * 4);
+        }
         la[t] = __builtin_amdgcn_readfirstlane(64 * e * 16);
     }
 #pragma unroll
     for (int t = 0; t < CB; t++)
     {
         const int e = wave + NW * t, s = 64 * e + lane, q = s / TN, w = s % TN;
-        vb[t] = B_KC ? (uint32_t)(((int64_t)w * ldb + 4 * q) * 4) : (uint32_t)(((int64_t)(4 * q + (w & 3)) * ldb + (w & ~3)) * 4);
+        if (B_KC)
+        {
+            const int64_t r = w < bn ? w : bn - 1;
+            vb[t] = (uint32_t)((r * ldb + 4 * q) * 4);
+        }
+        else
+        {
+            const int64_t r = (w & ~3) + 3 < bn ? (w & ~3) : bn - 4;
+            vb[t] = (uint32_t)(((int64_t)(4 * q + (w & 3)) * ldb + r) * 4);
+        }
         lb[t] = __builtin_amdgcn_readfirstlane(NB * OPA * 4 + 64 * e * 16);
     }
     const char *a_base = reinterpret_cast<const char *>(A_KC ? A + m0 * lda : A + m0);
     const char *b_base = reinterpret_cast<const char *>(B_KC ? B + n0 * ldb : B + n0);
     const int64_t a_step = (A_KC ? (int64_t)(4 * NQ) : (int64_t)(4 * NQ) * lda) * 4;
     const int64_t b_step = (B_KC ? (int64_t)(4 * NQ) : (int64_t)(4 * NQ) * ldb) * 4;
-    auto issue = [&](int buf) {
+    // k-tiles: nkt whole ones, then one of tq < NQ whole quads (if any), whose DMA is predicated
+    // by quad -- the quads it lacks lie past the end of the operands
+    const int64_t nkt = K / (4 * NQ);
+    const int tq = (int)((K / 4) % NQ);
+    const int64_t ntile = nkt + (tq > 0 ? 1 : 0);
+    auto issue = [&](int buf, bool tail) {
 #pragma unroll
         for (int t = 0; t < CA; t++)
             if (NIA % NW == 0 || wave + NW * t < NIA)
-                dma16(a_base, va[t], la[t] + buf * OPA * 4);
+            {
+                if (!tail)
+                    dma16(a_base, va[t], la[t] + buf * OPA * 4);
+                else if ((64 * (wave + NW * t) + lane) / TM < tq)
+                    dma16(a_base, va[t], la[t] + buf * OPA * 4);
+            }
 #pragma unroll
         for (int t = 0; t < CB; t++)
             if (NIB % NW == 0 || wave + NW * t < NIB)
-                dma16(b_base, vb[t], lb[t] + buf * OPB * 4);
+            {
+                if (!tail)
+                    dma16(b_base, vb[t], lb[t] + buf * OPB * 4);
+                else if ((64 * (wave + NW * t) + lane) / TN < tq)
+                    dma16(b_base, vb[t], lb[t] + buf * OPB * 4);
+            }
         a_base += a_step;
         b_base += b_step;
     };
@@ -936,13 +991,12 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__re
                 acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], b[j], acc[i][j], 0, 0, 0);
     };
 
-    const int64_t nkt = K / (4 * NQ);
-    if (nkt > 0)
+    if (ntile > 0)
     {
 #pragma unroll
         for (int u = 0; u < NB - 1; u++)
-            if (u < nkt)
-                issue(u);
+            if (u < ntile)
+                issue(u, u == nkt);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
 #pragma unroll
@@ -956,7 +1010,7 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__re
         {
             if (kt + u >= nkt)
                 break;
-            const bool more1 = kt + u + 1 < nkt, more_dma = kt + u + NB - 1 < nkt;
+            const bool more1 = kt + u + 1 < ntile, more_dma = kt + u + NB - 1 < ntile;
 #pragma unroll
             for (int q = 0; q < NQ; q++)
             {
@@ -971,7 +1025,7 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__re
                     __builtin_amdgcn_s_barrier();
                     asm volatile("" ::: "memory");
                     if (more_dma)
-                        issue((u + NB - 1) % NB);
+                        issue((u + NB - 1) % NB, kt + u + NB - 1 == nkt);
                 }
                 const int qq = q + D;
                 if (qq < NQ)
@@ -984,48 +1038,112 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__re
             }
         }
     }
+    if (tq > 0)
+    {
+        // the last k-tile: its first D quads are in the ring already, it has landed and been
+        // published by the barrier of the tile before it (or by the one above)
+        const int ub = (int)(nkt % NB);
+        const float *rat = ra + ub * OPA, *rbt = rb + ub * OPB;
+#pragma unroll
+        for (int q = 0; q < NQ - 1; q++)
+        {
+            if (q >= tq)
+                break;
+            const int qq = q + D;
+            if (qq < NQ)
+            {
+#pragma unroll
+                for (int i = 0; i < FM; i++)
+                    xa[qq % R][i] = rat[qq * QSA + 64 * i];
+#pragma unroll
+                for (int j = 0; j < FN; j++)
+                    xb[qq % R][j] = rbt[qq * QSB + 64 * j];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_q(xa[q % R], xb[q % R]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
 
-    // bias: one rounded add per output after its chain; a lane owns FN columns
+    const int64_t mw = m0 + wm * 16 * FM + 4 * g, nw = n0 + wn * 16 * FN + l16; // this lane's first row and column
+    // the k past the last whole quad (K not a multiple of 4: neither operand has k contiguous): one
+    // fused multiply-add per term, operands from global memory
+    for (int64_t k = K & ~(int64_t)3; k < K; k++)
+    {
+        float bk[FN];
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+        {
+            const int64_t nn = nw + 16 * j;
+            bk[j] = nn < N ? (B_KC ? B[nn * ldb + k] : B[k * ldb + nn]) : 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < FM; i++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+            {
+                const int64_t m = mw + 16 * i + r;
+                const float av = m < M ? (A_KC ? A[m * lda + k] : A[k * lda + m]) : 0.0f;
+#pragma unroll
+                for (int j = 0; j < FN; j++)
+                    acc[i][j][r] = __builtin_fmaf(av, bk[j], acc[i][j][r]);
+            }
+    }
+
+    // bias: one rounded add per output after its chain; a lane owns FN columns and 4 FM rows
     float bv[FN];
 #pragma unroll
     for (int j = 0; j < FN; j++)
-        bv[j] = bias != nullptr ? bias[n0 + wn * 16 * FN + 16 * j + l16] : 0.0f;
+        bv[j] = cbias != nullptr && nw + 16 * j < N ? cbias[nw + 16 * j] : 0.0f;
 #pragma unroll
     for (int i = 0; i < FM; i++)
 #pragma unroll
         for (int r = 0; r < 4; r++)
         {
-            const int64_t m = m0 + wm * 16 * FM + 16 * i + 4 * g + r;
+            const int64_t m = mw + 16 * i + r;
+            if (m >= M)
+                continue;
+            const float rv = rbias != nullptr ? rbias[m] : 0.0f;
 #pragma unroll
             for (int j = 0; j < FN; j++)
             {
-                const int64_t nn = n0 + wn * 16 * FN + 16 * j + l16;
-                __builtin_nontemporal_store(bias != nullptr ? acc[i][j][r] + bv[j] : acc[i][j][r], &C[m * N + nn]);
+                const int64_t nn = nw + 16 * j;
+                float v = acc[i][j][r];
+                if (cbias != nullptr)
+                    v = v + bv[j];
+                if (rbias != nullptr)
+                    v = v + rv;
+                if (nn < N)
+                    __builtin_nontemporal_store(v, &C[m * N + nn]);
             }
         }
 }
 
-// Whether mm_dma_kernel with this tile can take the product, and its launch.
+// Whether mm_dma_kernel with this tile can take the product: operand rows on 16-byte boundaries,
+// at least four rows (columns) where rows are contiguous (the edge clamp steps back by four), lane
+// offsets inside an operand tile within 32 bits.
 template <int FM, int FN, int WGM, int WGN, int NQ>
-bool dma_applies(int64_t M, int64_t N, int64_t K, int transA, int transB, int avec, int bvec)
+bool dma_applies(int64_t M, int64_t N, int64_t K, int transA, int transB, int avec, int bvec, int64_t nbatch = 1)
 {
     constexpr int TM = 16 * FM * WGM, TN = 16 * FN * WGN, BKQ = 4 * NQ;
-    if (!avec || !bvec || M % TM || N % TN || K % BKQ || K < BKQ)
+    if (!avec || !bvec || M < 1 || N < 1 || K < 1 || nbatch < 1 || nbatch > 65535)
+        return false;
+    if ((transA && M < 4) || (!transB && N < 4))
         return false;
     const int64_t lda = transA ? M : K, ldb = transB ? K : N;
-    // per-lane byte offsets inside an operand tile are 32-bit
     const int64_t ea = transA ? (int64_t)BKQ * lda + TM : (int64_t)TM * lda + BKQ;
     const int64_t eb = transB ? (int64_t)TN * ldb + BKQ : (int64_t)BKQ * ldb + TN;
-    return ea * 4 < (1LL << 32) && eb * 4 < (1LL << 32) && (M / TM) * (N / TN) <= REPDL_I32_MAX;
+    return ea * 4 < (1LL << 32) && eb * 4 < (1LL << 32) && repdl_cdiv(M, TM) * repdl_cdiv(N, TN) <= REPDL_I32_MAX;
 }
 
 template <bool TA, bool TB, int FM, int FN, int WGM, int WGN, int NQ, int D, int NB>
-int launch_dma_t(const float *A, const float *B, float *C, const float *bias, int64_t M, int64_t N, int64_t K, hipStream_t s)
+int launch_dma_t(const float *A, const float *B, float *C, const float *cbias, const float *rbias, int64_t M, int64_t N,
+                 int64_t K, int64_t nbatch, MmBatch batch, hipStream_t s)
 {
     constexpr int TM = 16 * FM * WGM, TN = 16 * FN * WGN;
     constexpr size_t shmem = (size_t)NB * NQ * 4 * (TM + TN) * sizeof(float);
     static_assert(shmem <= 160 * 1024, "LDS of one CU");
-    const int64_t gx = N / TN, gy = M / TM;
+    const int64_t gx = repdl_cdiv(N, TN), gy = repdl_cdiv(M, TM);
     const int64_t ntiles8 = (gx * gy) & ~(int64_t)7;
     auto kern = &mm_dma_kernel<TA, TB, FM, FN, WGM, WGN, NQ, D, NB>;
     if (shmem > 48 * 1024)
@@ -1035,21 +1153,86 @@ int launch_dma_t(const float *A, const float *B, float *C, const float *bias, in
         if (e != hipSuccess)
             return (int)e;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)(gx * gy)), dim3(64 * WGM * WGN), shmem, s, A, B, C, bias, M, N, K, gx, gy, ntiles8);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(gx * gy), (unsigned)nbatch), dim3(64 * WGM * WGN), shmem, s, A, B, C, cbias, rbias, M,
+                       N, K, gx, gy, ntiles8, batch);
     return repdl_launch_status();
 }
 
 template <int FM, int FN, int WGM, int WGN, int NQ, int D, int NB>
-int launch_dma(const float *A, const float *B, float *C, const float *bias, int64_t M, int64_t N, int64_t K, int transA,
-               int transB, hipStream_t s)
+int launch_dma(const float *A, const float *B, float *C, const float *cbias, const float *rbias, int64_t M, int64_t N, int64_t K,
+               int transA, int transB, int64_t nbatch, MmBatch batch, hipStream_t s)
 {
     if (!transA && !transB)
-        return launch_dma_t<false, false, FM, FN, WGM, WGN, NQ, D, NB>(A, B, C, bias, M, N, K, s);
+        return launch_dma_t<false, false, FM, FN, WGM, WGN, NQ, D, NB>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
     if (transA && !transB)
-        return launch_dma_t<true, false, FM, FN, WGM, WGN, NQ, D, NB>(A, B, C, bias, M, N, K, s);
+        return launch_dma_t<true, false, FM, FN, WGM, WGN, NQ, D, NB>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
     if (!transA && transB)
-        return launch_dma_t<false, true, FM, FN, WGM, WGN, NQ, D, NB>(A, B, C, bias, M, N, K, s);
-    return launch_dma_t<true, true, FM, FN, WGM, WGN, NQ, D, NB>(A, B, C, bias, M, N, K, s);
+        return launch_dma_t<false, true, FM, FN, WGM, WGN, NQ, D, NB>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
+    return launch_dma_t<true, true, FM, FN, WGM, WGN, NQ, D, NB>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
+}
+
+// The tile for a batch of products, and its launch; REPDL_E_UNSUPPORTED if mm_dma_kernel cannot
+// take the operands.  Shares of the chip's matrix rate (145 TFLOP/s on the 128x128 tile with many
+// tiles per CU) by tiles per CU r, measured on whole-tile shapes (a CU holds up to three workgroups
+// of the first two tiles at once):
+//   128x128, 8 waves of 64x32, k-tile 16:   r = 1 0.77, 2 0.85, 3 0.88, more 0.97
+//   64x64, 4 waves of 32x32, k-tile 32/16:  r = 1 0.60, 2 0.76, 3 0.86, 4..7 0.88, more 0.92
+//   64x16 or 16x64, 4 waves of 16x16, k-tile 64, five buffers: 0.35 (one 16x16 block per SIMD is a
+//     chain of dependent instructions; for C with fewer 64x64 tiles than CUs)
+// (8192^3 NT: 145 / 138 TFLOP/s on the first two; 3072^2 x 4096: 96 / 133; 2048^2 x 4096: 112 / 128;
+// 1408^2 x 4096: 57 / 105; 1024^3: - / 87; 64 x 4096 x 4096: 28 on 64x64, 51 on 64x16.)  A tile that
+// hangs over an edge costs what a whole one does.
+#ifdef REPDL_DEBUG_HOOKS
+int g_force_tile = 0; // 1..5: that configuration whatever the shape
+#endif
+int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias, const float *rbias, int64_t M, int64_t N,
+                    int64_t K, int transA, int transB, int avec, int bvec, int64_t nbatch, MmBatch batch, hipStream_t s)
+{
+    auto rounds = [&](int64_t tm, int64_t tn) { return repdl_cdiv(repdl_cdiv(M, tm) * repdl_cdiv(N, tn) * nbatch, 256); };
+    double best = 1e300;
+    int pick = 0;
+    if (dma_applies<4, 2, 2, 4, 4>(M, N, K, transA, transB, avec, bvec, nbatch))
+    {
+        const int64_t r = rounds(128, 128);
+        const double c = (double)r * 16384.0 / (r >= 4 ? 0.97 : r == 3 ? 0.88 : r == 2 ? 0.85 : 0.77);
+        if (c < best)
+            best = c, pick = 1;
+    }
+    if (dma_applies<2, 2, 2, 2, 8>(M, N, K, transA, transB, avec, bvec, nbatch))
+    {
+        const int64_t r = rounds(64, 64);
+        const double c = (double)r * 4096.0 / (r >= 8 ? 0.92 : r >= 4 ? 0.88 : r == 3 ? 0.86 : r == 2 ? 0.76 : 0.60);
+        // the deeper k-tile pays when a CU has one workgroup; the shallower one lets six share a CU
+        if (c < best)
+            best = c, pick = r == 1 ? 2 : 3;
+    }
+    if (dma_applies<1, 1, 4, 1, 16>(M, N, K, transA, transB, avec, bvec, nbatch))
+    {
+        // 64x16 or 16x64: whichever makes fewer tiles
+        const int64_t r1 = rounds(64, 16), r2 = rounds(16, 64);
+        const double c = (double)(r1 <= r2 ? r1 : r2) * 1024.0 / 0.35;
+        if (c < best)
+            best = c, pick = r1 <= r2 ? 4 : 5;
+    }
+#ifdef REPDL_DEBUG_HOOKS
+    if (g_force_tile > 0)
+        pick = g_force_tile;
+#endif
+    switch (pick)
+    {
+    case 1:
+        return launch_dma<4, 2, 2, 4, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+    case 2:
+        return launch_dma<2, 2, 2, 2, 8, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+    case 3:
+        return launch_dma<2, 2, 2, 2, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+    case 4:
+        return launch_dma<1, 1, 4, 1, 16, 7, 5>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+    case 5:
+        return launch_dma<1, 1, 1, 4, 16, 7, 5>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+    default:
+        return REPDL_E_UNSUPPORTED;
+    }
 }
 
 template <bool TA, bool TB, int FM, int FN, int WGM, int WGN>
@@ -1113,6 +1296,33 @@ int launch_mfma(const float *A, const float *B, float *C, const float *bias, int
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 } // namespace
 
+#ifdef REPDL_DEBUG_HOOKS
+REPDL_API int repdl_debug_mm_tile(int t)
+{
+    g_force_tile = t;
+    return 0;
+}
+#endif
+
+int repdl_mm_batched(const float *A, const float *B, float *C, const float *row_bias, int64_t M, int64_t N, int64_t K,
+                     int transA, int transB, int64_t nbatch, int64_t strideA, int64_t strideB, int64_t strideC,
+                     hipStream_t stream)
+{
+    if (!repdl_mfma_exact() || M < 1 || N < 1 || K < 1 || nbatch < 1)
+        return REPDL_E_UNSUPPORTED;
+#ifdef REPDL_DEBUG_HOOKS
+    if (g_force_tile == 99)
+        return REPDL_E_UNSUPPORTED;
+#endif
+    const int64_t lda = transA ? M : K, ldb = transB ? K : N;
+    const int avec = aligned16(A) && lda % 4 == 0 && strideA % 4 == 0;
+    const int bvec = aligned16(B) && ldb % 4 == 0 && strideB % 4 == 0;
+    if (!avec || !bvec)
+        return REPDL_E_UNSUPPORTED;
+    return mm_dma_dispatch(A, B, C, nullptr, row_bias, M, N, K, transA, transB, avec, bvec, nbatch,
+                           MmBatch{strideA, strideB, strideC}, stream);
+}
+
 REPDL_API int repdl_hip_mm(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K,
                            int transA, int transB, void *stream)
 {
@@ -1133,64 +1343,14 @@ REPDL_API int repdl_hip_mm_bias(const float *A, const float *B, const float *bia
     hipStream_t s = repdl_stream(stream);
     if (repdl_mfma_exact())
     {
-        // Whole-tile shapes with aligned operands: mm_dma_kernel.  Its configurations, with the share
-        // of the chip's matrix rate (145 TFLOP/s on the 128x128 tile with many tiles per CU) each was
-        // measured at, by tiles per CU r (a CU holds up to three workgroups of either tile at once):
-        //   128x128, 8 waves of 64x32, k-tile 16:   r = 1 0.76, 2 0.92, 3 0.97, more 0.99
-        //   64x64, 4 waves of 32x32, k-tile 32/16:  r = 1 0.60, 2 0.76, 3..5 0.83, 6..11 0.89, more 0.94
-        //   64x16 or 16x64, 4 waves of 16x16, k-tile 64, five buffers: 0.35 (one 16x16 block per SIMD is
-        //     a chain of dependent instructions; for C with fewer 64x64 tiles than CUs)
-        // (8192^3 NT: 145 / 138 TFLOP/s on the first two; 3072^2 x 4096: 108 / 129; 2048^3: 110 / 121;
-        // 1536^2 x 4096: 75 / 96; 1024^3: - / 87; 64 x 4096 x 4096: 28 on 64x64, 51 on 64x16.)
+        // operand rows on 16-byte boundaries: the kernel that moves them straight into LDS
         if (avec && bvec)
         {
-            auto rounds = [&](int64_t tm, int64_t tn) { return repdl_cdiv((M / tm) * (N / tn), 256); };
-            double best = 1e300;
-            int pick = 0;
-            if (dma_applies<4, 2, 2, 4, 4>(M, N, K, transA, transB, avec, bvec))
-            {
-                const int64_t r = rounds(128, 128);
-                const double c = (double)r * 16384.0 / (r >= 4 ? 0.99 : r == 3 ? 0.97 : r == 2 ? 0.92 : 0.76);
-                if (c < best)
-                    best = c, pick = 1;
-            }
-            if (dma_applies<2, 2, 2, 2, 4>(M, N, K, transA, transB, avec, bvec))
-            {
-                const int64_t r = rounds(64, 64);
-                const double c = (double)r * 4096.0 / (r >= 12 ? 0.94 : r >= 6 ? 0.89 : r >= 3 ? 0.83 : r == 2 ? 0.76 : 0.60);
-                // the deeper k-tile pays when a CU has one workgroup; the shallower one lets six share a CU
-                if (c < best)
-                    best = c, pick = (r == 1 && dma_applies<2, 2, 2, 2, 8>(M, N, K, transA, transB, avec, bvec)) ? 2 : 3;
-            }
-            if (dma_applies<1, 1, 4, 1, 16>(M, N, K, transA, transB, avec, bvec))
-            {
-                const double c = (double)rounds(64, 16) * 1024.0 / 0.35;
-                if (c < best)
-                    best = c, pick = 4;
-            }
-            else if (dma_applies<1, 1, 1, 4, 16>(M, N, K, transA, transB, avec, bvec))
-            {
-                const double c = (double)rounds(16, 64) * 1024.0 / 0.35;
-                if (c < best)
-                    best = c, pick = 5;
-            }
-            switch (pick)
-            {
-            case 1:
-                return launch_dma<4, 2, 2, 4, 4, 1, 3>(A, B, C, bias, M, N, K, transA, transB, s);
-            case 2:
-                return launch_dma<2, 2, 2, 2, 8, 1, 3>(A, B, C, bias, M, N, K, transA, transB, s);
-            case 3:
-                return launch_dma<2, 2, 2, 2, 4, 1, 3>(A, B, C, bias, M, N, K, transA, transB, s);
-            case 4:
-                return launch_dma<1, 1, 4, 1, 16, 7, 5>(A, B, C, bias, M, N, K, transA, transB, s);
-            case 5:
-                return launch_dma<1, 1, 1, 4, 16, 7, 5>(A, B, C, bias, M, N, K, transA, transB, s);
-            default:
-                break;
-            }
+            const int rc = mm_dma_dispatch(A, B, C, bias, nullptr, M, N, K, transA, transB, avec, bvec, 1, MmBatch{0, 0, 0}, s);
+            if (rc != REPDL_E_UNSUPPORTED)
+                return rc;
         }
-        // Every other shape: the kernels that stage operands through registers.  A CU runs its tiles one after the other (256x256: one workgroup fills it) or
+        // Other operands: the kernels that stage them through registers.  A CU runs its tiles one after the other (256x256: one workgroup fills it) or
         // side by side (smaller tiles), so a configuration costs (most tiles on any CU) x tile area
         // / rate, with the rates measured per configuration and tiles per CU, relative to the
         // 256x256 tile (135 TFLOP/s chip-wide): 128x128 0.785 alone on its CU, 0.92 with two, 0.955

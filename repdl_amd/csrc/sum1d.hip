@@ -981,6 +981,8 @@ __global__ __launch_bounds__(64) void sum1d_plan_kernel(const double *__restrict
 
 #ifdef REPDL_DEBUG_HOOKS
 __device__ unsigned long long g_dbg[8]; // wave-level counts: nodes, blocks failed, groups failed, chunk replays
+#endif
+#if defined(REPDL_DEBUG_HOOKS) && defined(REPDL_DEBUG_COUNTS) // (the counting itself slows the walks many times over)
 #define DBG_COUNT(i) do { if ((threadIdx.x & 63) == 0) atomicAdd(&g_dbg[i], 1ull); } while (0)
 #else
 #define DBG_COUNT(i) do { } while (0)
@@ -1382,12 +1384,12 @@ static int g_debug_rounds = -1;
 #endif
 static int spec_rounds(int64_t rows, int64_t n)
 {
-    if (rows != 1 || n < ((int64_t)1 << 22))
-        return 0;
 #ifdef REPDL_DEBUG_HOOKS
     if (g_debug_rounds >= 0)
         return g_debug_rounds;
 #endif
+    if (rows != 1 || n < ((int64_t)1 << 22))
+        return 0;
     return n < ((int64_t)1 << 24) ? 4 : (n < ((int64_t)1 << 26) ? 8 : MAX_ROUNDS);
 }
 

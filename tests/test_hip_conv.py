@@ -44,6 +44,11 @@ FWD = [
     (2, 32, 33, 40, 64, 1, 1, 1, 1, 0, 0, 1),      # 1320 pixels: 10.3 tiles
     (1, 16, 32, 32, 128, 1, 1, 1, 1, 0, 0, 1),     # two row tiles forward, 16 channels: one step of the stream
     (3, 64, 30, 45, 64, 1, 1, 1, 1, 0, 0, 1),      # 1350 pixels, the last tile half full
+    # 1x1 at stride 1 without padding, pixels in fours, channels in fours: a batch of matrix products per image
+    (2, 96, 20, 20, 72, 1, 1, 1, 1, 0, 0, 1),      # 400 pixels, 72 rows forward (96 in grad-input): tile edges both ways
+    (3, 128, 33, 40, 192, 1, 1, 1, 1, 0, 0, 1),    # chains of 128 (forward) and 192 (grad-input) terms
+    (1, 68, 6, 6, 20, 1, 1, 1, 1, 0, 0, 1),        # one small image: a k-tile tail of one quad, 20 rows
+    (5, 24, 8, 12, 36, 1, 1, 1, 1, 0, 0, 1),       # chains shorter than a k-tile
 ]
 
 

@@ -23,12 +23,14 @@ def test_layouts_and_edges(shape, tA, tB):
     assert torch.equal(got, oracle.mm(a, b, bool(tA), bool(tB)))
 
 
-# Whole-tile shapes with aligned operands take the kernels that move operands from global memory
-# straight into LDS; one shape per tile configuration (128x128; 64x64 with the shallow and the
-# deep k-tile; 64x16; 16x64), each in all four layouts.
+# Operands whose rows start on 16-byte boundaries take the kernel that moves them from global memory
+# straight into LDS.  Whole-tile shapes for each of its tile configurations (128x128; 64x64 with the
+# shallow and the deep k-tile; 64x16; 16x64), then shapes that hang over the tile edges, K that
+# leaves a tail behind the last whole k-tile, K shorter than one k-tile, and the smallest extents.
 WHOLE_TILE_SHAPES = [(4096, 4096, 48), (2048, 2048, 80), (512, 512, 96), (512, 512, 48), (64, 1024, 128), (48, 1024, 192),
-                     (256, 192, 128), (128, 128, 2048)]
-
+                     (256, 192, 128), (128, 128, 2048),
+                     (260, 132, 1000), (100, 36, 52), (4, 4, 4), (68, 20, 24), (1028, 2052, 36), (2500, 1300, 76), (8, 4100, 12),
+                     (132, 260, 1001), (64, 64, 71), (512, 512, 2)]
 
 @pytest.mark.parametrize("tA,tB", [(0, 0), (1, 0), (0, 1), (1, 1)])
 @pytest.mark.parametrize("shape", WHOLE_TILE_SHAPES, ids=str)
@@ -55,6 +57,17 @@ def test_whole_tile_shapes(shape, tA, tB):
     want += bias
     got = ops.mm_bias(a.cuda(), b.cuda(), bias.cuda(), bool(tA), bool(tB)).cpu()
     assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+
+
+def test_edge_of_the_largest_tile():
+    """Enough tiles that the 128x128 configuration is chosen, with a last tile-row of four rows."""
+    from repdl_amd import ops
+
+    M, N, K = 8196, 8192, 20
+    a = gen.scaled_normal(5, M, K, lo=-6, hi=6)
+    b = gen.normal_like(6, K, N)
+    got = ops.mm(a.cuda(), b.cuda()).cpu()
+    assert torch.equal(got.view(torch.int32), oracle.mm(a, b).view(torch.int32))
 
 
 @pytest.mark.parametrize("tA,tB", [(0, 1), (0, 0), (1, 0), (1, 1)])
