@@ -47,32 +47,37 @@ HBM_PEAK_GBS = 8000.0
 TRAFFIC_JSON = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 
 # Which kernels make up a call of each leg (substrings of the kernel names rocprofv3 reports), for
-# --write-traffic.  The first entry is the leg's anchor: it runs exactly once per call, so the
-# number of calls in a profiled run is its dispatch count.
+# --write-traffic.  The LAST entry is the kernel that ends a call.  Several legs may share kernels
+# (the sequential sums do): "grid" then names the launch size, in threads, of the leg's first kernel
+# at the bench's workload.  "split": the bench runs that many workloads through these kernels one
+# after the other, an equal number of calls each; they get a traffic entry each, in that order.
+_S1 = ["sum1d_blocksum_kernel", "sum1d_prefix_kernel", "sum1d_tuple_kernel", "sum1d_super_kernel", "sum1d_plan_kernel",
+       "sum1d_cand_walk_kernel", "sum1d_compose_kernel", "sum1d_compose2_kernel", "sum1d_resolve_kernel", "sum1d_walk_kernel"]
 LEG_KERNELS = {
-    "mm": ["mm_dma_kernel<false, true, 4, 2, 2, 4"],
-    "mm_fma": ["mm_kernel<false, true"],
-    "sum2d_dim1": ["rowchain_kernel"],
-    "sum2d_dim0": ["coltile_kernel"],
-    "sum1d": ["sum1d_super_kernel", "sum1d_blocksum_kernel", "sum1d_prefix_kernel", "sum1d_tuple_kernel", "sum1d_plan_kernel",
-              "sum1d_cand_walk_kernel", "sum1d_compose_kernel", "sum1d_compose2_kernel", "sum1d_resolve_kernel", "sum1d_walk_kernel"],
-    "exp": ["unary_kernel<0>"],
-    "log": ["unary_kernel<1>"],
-    "sqrt": ["unary_kernel<2>"],
-    "div_scalar": ["unary_kernel<3>"],
-    "div": ["div_kernel"],
-    "softmax": ["rows_onchip_kernel"],
-    "adam_step": ["adam_kernel"],
+    "mm": {"kernels": ["mm_dma_kernel<false, true, 4, 2, 2, 4, 4"]},
+    "mm_fma": {"kernels": ["mm_kernel<false, true"]},
+    "mm1024": {"kernels": ["mm_dma_kernel<false, false, 2, 2, 2, 2, 8"]},
+    "sum2d_dim1": {"kernels": ["rowchain_kernel<32, 128, true, false>"]},
+    "sum2d_dim0": {"kernels": ["coltile_kernel<16, true, 2>"]},
+    "sum4d_dim023": {"kernels": _S1, "grid": 49 * 256 * 64},
+    "sum1d": {"kernels": _S1, "grid": 65536 * 256, "split": ["sum1d", "sum1d_drift"]},
+    "exp": {"kernels": ["unary_kernel<0>"]},
+    "log": {"kernels": ["unary_kernel<1>"]},
+    "sqrt": {"kernels": ["unary_kernel<2>"]},
+    "div_scalar": {"kernels": ["unary_kernel<3>"]},
+    "div": {"kernels": ["div_kernel"]},
+    "softmax": {"kernels": ["rows_onchip_kernel<8, 32, true>"]},
+    "cross_entropy": {"kernels": ["rows_onchip_kernel<8, 32, false>"]},
+    "conv3x3_fwd": {"kernels": ["conv_patch_prep_kernel", "conv_patch_kernel<0>"]},
+    "conv3x3_dgrad": {"kernels": ["conv_patch_prep_kernel", "conv_patch_kernel<1>"]},
+    "conv3x3_wgrad": {"kernels": ["conv_wgrad_mfma_kernel<14, true, 2>"]},
+    "conv1x1_fwd": {"kernels": ["mm_dma_kernel<false, false, 2, 2, 2, 2, 4"]},
+    "conv1x1_dgrad": {"kernels": ["conv_point_prep_kernel", "conv_point_kernel<1>"]},
+    "conv1x1_wgrad": {"kernels": ["conv_wgrad_mfma_kernel<14, true, 8>"]},
+    "adam_step": {"kernels": ["adam_kernel"]},
 }
 
 
-def sha(t) -> str:
-    return hashlib.sha256(t.detach().cpu().contiguous().numpy().tobytes()).hexdigest()
-
-
-# ----------------------------------------------------------------------------------------------
-# rocprofv3 summaries (no GPU needed)
-# ----------------------------------------------------------------------------------------------
 def _short(name: str) -> str:
     return name.replace("(anonymous namespace)::", "").replace("void ", "")
 
@@ -112,31 +117,53 @@ def summarise_counters(dirnames) -> None:
             print("%-100s %-30s %7d %18.1f" % (k[:100], c, len(v), sum(v) / len(v)))
 
 
+def _leg_calls(dirname: str, counter: str, spec):
+    """The counter summed over each call of a leg: the leg's dispatches in launch order, cut after
+    every dispatch of the leg's last kernel; only calls whose first kernel has the leg's launch size
+    (the largest seen, if the leg names none)."""
+    subs, end = spec["kernels"], spec["kernels"][-1]
+    rows = [r for r in csv.DictReader(open(_find(dirname, "*counter_collection.csv")))
+            if r["Counter_Name"] == counter and any(x in _short(r["Kernel_Name"]) for x in subs)]
+    rows.sort(key=lambda r: int(r["Dispatch_Id"]))
+    calls, cur = [], []
+    for r in rows:
+        cur.append(r)
+        if end in _short(r["Kernel_Name"]):
+            calls.append(cur)
+            cur = []
+    if not calls:
+        return []
+    first_grid = lambda c: max(int(r["Grid_Size"]) for r in c if subs[0] in _short(r["Kernel_Name"])) if any(subs[0] in _short(r["Kernel_Name"]) for r in c) else 0
+    grid = spec.get("grid") or max(first_grid(c) for c in calls)
+    return [sum(float(r["Counter_Value"]) for r in c) for c in calls if first_grid(c) == grid]
+
+
+def _median(v):
+    v = sorted(v)
+    return v[len(v) // 2]
+
+
 def write_traffic(fetch_dir: str, write_dir: str) -> None:
     """FETCH_SIZE / WRITE_SIZE count in device-specific units: both are scaled by what the same counter
-    reads for the --copy-probe kernel, which reads exactly 1 GiB and writes exactly 1 GiB per dispatch."""
-    fetch, write = _counter_means(fetch_dir), _counter_means(write_dir)
-
-    def mean_of(agg, sub, counter):
-        hits = [(k, v) for (k, c), v in agg.items() if c == counter and sub in k]
-        return hits
-
-    probe = "trunc"
-    pf, pw = mean_of(fetch, probe, "FETCH_SIZE"), mean_of(write, probe, "WRITE_SIZE")
+    reads for the --copy-probe kernel, which reads exactly 1 GiB and writes exactly 1 GiB per dispatch.
+    Per leg: the median over its calls (a call of a leg that shares a set-up kernel with the leg before
+    it can pick up that leg's last set-up launches)."""
+    probe = {"kernels": ["trunc"]}
+    pf, pw = _leg_calls(fetch_dir, "FETCH_SIZE", probe), _leg_calls(write_dir, "WRITE_SIZE", probe)
     if not pf or not pw:
         raise SystemExit("the copy-probe kernel is missing from the counter runs (run bench.py with --copy-probe)")
-    f_unit = float(1 << 30) / (sum(pf[0][1]) / len(pf[0][1]))
-    w_unit = float(1 << 30) / (sum(pw[0][1]) / len(pw[0][1]))
+    f_unit, w_unit = float(1 << 30) / _median(pf), float(1 << 30) / _median(pw)
     legs, detail = {}, {}
-    for leg, subs in LEG_KERNELS.items():
-        anchor_f, anchor_w = mean_of(fetch, subs[0], "FETCH_SIZE"), mean_of(write, subs[0], "WRITE_SIZE")
-        if not anchor_f or not anchor_w:
+    for leg, spec in LEG_KERNELS.items():
+        rd, wr = _leg_calls(fetch_dir, "FETCH_SIZE", spec), _leg_calls(write_dir, "WRITE_SIZE", spec)
+        if not rd or not wr:
             continue
-        calls_f, calls_w = sum(len(v) for _, v in anchor_f), sum(len(v) for _, v in anchor_w)
-        rd = sum(sum(v) for sub in subs for _, v in mean_of(fetch, sub, "FETCH_SIZE")) * f_unit / calls_f
-        wr = sum(sum(v) for sub in subs for _, v in mean_of(write, sub, "WRITE_SIZE")) * w_unit / calls_w
-        legs[leg] = round(rd + wr)
-        detail[leg] = {"read_bytes_per_call": round(rd), "written_bytes_per_call": round(wr), "calls_profiled": calls_f}
+        names = spec.get("split", [leg])
+        for i, name in enumerate(names):
+            part = lambda v: v[len(v) * i // len(names):len(v) * (i + 1) // len(names)]
+            r, w = _median(part(rd)) * f_unit, _median(part(wr)) * w_unit
+            legs[name] = round(r + w)
+            detail[name] = {"read_bytes_per_call": round(r), "written_bytes_per_call": round(w), "calls_profiled": len(part(rd))}
     out = {"source": "rocprofv3 --pmc FETCH_SIZE / --pmc WRITE_SIZE over `bench.py --copy-probe`, one run per counter",
            "calibration": {"fetch_bytes_per_count": f_unit, "write_bytes_per_count": w_unit,
                            "probe": "torch.trunc(x, out=y) on 2^28 floats: 1 GiB read, 1 GiB written per dispatch"},
@@ -394,7 +421,7 @@ def main() -> int:
             dt, y_cpu = cpu_time(lambda: (refmods[0].mm(a_h, b_h, False, False) if refmods else oracle.mm(a_h, b_h, False, False)))
             par = {"equal": sha(hold["y"]) == sha(y_cpu), "sha256_gpu": sha(hold["y"])}
             cpu = {"value": round(2.0 * 1024 ** 3 / dt / 1e9, 3), "unit": "GFLOP/s", "cores": cores, "kind": kind, "sample": "the full product"}
-            also.append(leg_entry("mm", "1024x1024x1024 NN, N(0,1) entries (configs[0])", "mfma", 2.0 * 1024 ** 3, f, args.steps * 4, args.warmup, par, cpu))
+            also.append(leg_entry("mm", "1024x1024x1024 NN, N(0,1) entries (configs[0])", "mfma", 2.0 * 1024 ** 3, f, args.steps * 4, args.warmup, par, cpu, "mm1024"))
             del a_d, b_d
 
         if want("sum2d"):
@@ -440,7 +467,7 @@ def main() -> int:
             par = {"equal": sha(hold["y"]) == sha(y_cpu), "sha256_gpu": sha(hold["y"])}
             cpu = {"value": round(t_h.numel() * 4 / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": kind, "sample": "the full tensor"}
             also.append(leg_entry("sum4d_dim023", "channel sums of [64,64,56,56] N(0,1) (conv grad-bias shape)", "hbm", 4.0 * t_h.numel(), f,
-                                  args.steps, args.warmup, par, cpu))
+                                  args.steps, args.warmup, par, cpu, "sum4d_dim023"))
             del t_d, t_h, hold
 
         if want("sum1d"):
@@ -460,7 +487,7 @@ def main() -> int:
             f()
             y_cpu = oracle.sum1d(v_h)
             par = {"equal": sha(hold["y"]) == sha(y_cpu), "gpu": float(hold["y"]), "cpu": float(y_cpu)}
-            also.append(leg_entry("sum1d", "sequential sum of 2^28 uniform[0,1) (drifting)", "hbm", 4.0 * n, f, args.steps, args.warmup, par, None))
+            also.append(leg_entry("sum1d", "sequential sum of 2^28 uniform[0,1) (drifting)", "hbm", 4.0 * n, f, args.steps, args.warmup, par, None, "sum1d_drift"))
             del v_d, v_h, hold
 
         ew = [k for k in ("exp", "log", "sqrt", "div") if want(k)]
@@ -526,7 +553,7 @@ def main() -> int:
                 dt, _ = cpu_time(rfn)
                 cpu = {"value": round(nbytes / M * ms / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": kind, "sample": "first %d rows" % ms}
                 also.append(leg_entry(name, "%s of 65536x1000 logits N(0,16)" % name, "hbm", nbytes, f, args.steps, args.warmup, par, cpu,
-                                      "softmax" if name == "softmax" else None))
+                                      name))
                 del y_cpu
             del z_d, z_h
 
@@ -562,8 +589,9 @@ def main() -> int:
                     dt, _ = cpu_time(rfn)
                     cpu = {"value": round(cflop * nb / N / dt / 1e9, 2), "unit": "GFLOP/s", "cores": cores, "kind": kind,
                            "sample": "the first %d of %d images (for grad-kernel: chains %d times shorter)" % (nb, N, N // nb)}
+                    tleg = "conv%dx%d_%s" % (Kk, Kk, {"conv2d": "fwd", "conv2d_grad_input": "dgrad", "conv2d_grad_kernel": "wgrad"}[name])
                     also.append(leg_entry(name, "batch %d, %dx%d conv %d->%d at %dx%d" % (N, Kk, Kk, IC, OC, H, W), "mfma", cflop, f, args.steps,
-                                          args.warmup, par, cpu))
+                                          args.warmup, par, cpu, tleg))
                     del y_cpu
                 del x_d, w_d, go_d
 

@@ -1230,6 +1230,14 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
         return launch_dma<1, 1, 4, 1, 16, 7, 5>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 5:
         return launch_dma<1, 1, 1, 4, 16, 7, 5>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+#ifdef REPDL_DEBUG_HOOKS
+    case 6:
+        return launch_dma<8, 4, 2, 4, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+    case 7:
+        return launch_dma<4, 4, 2, 2, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+    case 8:
+        return launch_dma<4, 2, 2, 4, 8, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+#endif
     default:
         return REPDL_E_UNSUPPORTED;
     }
