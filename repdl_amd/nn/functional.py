@@ -169,6 +169,12 @@ class _BatchNorm(torch.autograd.Function):
         return gx, gmean, gvar, gweight, gbias, None
 
 
+# The reference evaluates the running-statistics updates in training (batchnorm.py:92-93) and drops
+# the results, so its buffers keep their initial values.  False reproduces that; True stores the two
+# expressions it evaluates (running mean as PyTorch's, running variance from the biased batch variance).
+STORE_RUNNING_STATS = False
+
+
 def batch_norm(input: torch.Tensor, running_mean: Optional[torch.Tensor], running_var: Optional[torch.Tensor],
                weight: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
                batch_statistics: bool = False, momentum: float = 0.1, eps: float = 1e-5) -> torch.Tensor:
@@ -184,9 +190,7 @@ def batch_norm(input: torch.Tensor, running_mean: Optional[torch.Tensor], runnin
             mean = func.mean2d_dim0(input)
             centred = input - func.expand_as(mean, input)
             var = func.mean2d_dim0(centred * centred)
-        if running_mean is not None and running_var is not None:
-            # The reference evaluates these two expressions (batchnorm.py:92-93) but
-            # drops the results; here they are stored, which is what the buffers are for.
+        if STORE_RUNNING_STATS and running_mean is not None and running_var is not None:
             with torch.no_grad():
                 running_mean.copy_(momentum * mean.detach() + (1.0 - momentum) * running_mean)
                 running_var.copy_(momentum * var.detach() + (1.0 - momentum) * running_var)

@@ -85,7 +85,7 @@ def test_cross_entropy_matches_torch():
             repdl_amd.nn.functional.cross_entropy(x2, t, reduction="sum")
 
 
-def test_batchnorm_close_to_torch():
+def test_batchnorm_close_to_torch(monkeypatch):
     with oracle_for_cpu_tensors():
         for bn_t, x in ((torch.nn.BatchNorm2d(5), gen.normal_like(31, 4, 5, 6, 7)),
                         (torch.nn.BatchNorm1d(6), gen.normal_like(32, 9, 6))):
@@ -94,7 +94,13 @@ def test_batchnorm_close_to_torch():
                 bn_t.bias.copy_(gen.normal_like(34, bn_t.num_features))
             bn_r = repdl_amd.from_torch_module(bn_t)
             x1, x2 = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+            # as the reference (batchnorm.py:92-93): the updates are evaluated and dropped
+            before = bn_r.running_mean.clone(), bn_r.running_var.clone()
+            bn_r(x.clone())
+            assert torch.equal(bn_r.running_mean, before[0]) and torch.equal(bn_r.running_var, before[1])
+            monkeypatch.setattr(repdl_amd.nn.functional, "STORE_RUNNING_STATS", True)
             y_t, y_r = bn_t(x1), bn_r(x2)
+            monkeypatch.setattr(repdl_amd.nn.functional, "STORE_RUNNING_STATS", False)
             assert torch.allclose(y_r, y_t, atol=2e-5)
             go = gen.normal_like(35, *x.shape)
             y_t.backward(go)
