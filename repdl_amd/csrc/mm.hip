@@ -1177,10 +1177,14 @@ int launch_dma(const float *A, const float *B, float *C, const float *cbias, con
 // of the first two tiles at once):
 //   128x128, 8 waves of 64x32, k-tile 16:   r = 1 0.77, 2 0.85, 3 0.88, more 0.97
 //   64x64, 4 waves of 32x32, k-tile 32/16:  r = 1 0.60, 2 0.76, 3 0.86, 4..7 0.88, more 0.92
-//   64x16 or 16x64, 4 waves of 16x16, k-tile 64, five buffers: 0.35 (one 16x16 block per SIMD is a
-//     chain of dependent instructions; for C with fewer 64x64 tiles than CUs)
+//   32x32, 4 waves of one 16x16 block, k-tile 64, read-ahead 7 quads, five buffers: 0.39 at r = 1, 0.46 beyond;
+//   64x32, 8 such waves: 0.53 -- for C with fewer 64x64 tiles than CUs: one or two blocks per SIMD, each
+//     a chain of dependent instructions, and what bounds them is L2: the smaller the tile, the more
+//     often an operand row is fetched (a 32x32 tile asks for 64 rows per 1024 outputs; 64x16 tiles,
+//     80 rows, were slower: 42 against 38 us on 64 x 4096 x 4096)
 // (8192^3 NT: 145 / 138 TFLOP/s on the first two; 3072^2 x 4096: 96 / 133; 2048^2 x 4096: 112 / 128;
-// 1408^2 x 4096: 57 / 105; 1024^3: - / 87; 64 x 4096 x 4096: 28 on 64x64, 51 on 64x16.)  A tile that
+// 1408^2 x 4096: 57 / 105; 1024^3: - / 87; 64 x 4096 x 4096: 28 on 64x64, 57 on 32x32; 128 x 4096 x 4096:
+// 67 on 32x32, 77 on 64x32; 256 x 1024 x 8192: 61 on 32x32.)  A tile that
 // hangs over an edge costs what a whole one does.
 #ifdef REPDL_DEBUG_HOOKS
 int g_force_tile = 0; // 1..5: that configuration whatever the shape
@@ -1206,13 +1210,18 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
         if (c < best)
             best = c, pick = r == 1 ? 2 : 3;
     }
-    if (dma_applies<1, 1, 4, 1, 16>(M, N, K, transA, transB, avec, bvec, nbatch))
+    if (dma_applies<1, 1, 2, 2, 16>(M, N, K, transA, transB, avec, bvec, nbatch))
     {
-        // 64x16 or 16x64: whichever makes fewer tiles
-        const int64_t r1 = rounds(64, 16), r2 = rounds(16, 64);
-        const double c = (double)(r1 <= r2 ? r1 : r2) * 1024.0 / 0.35;
+        const int64_t r = rounds(32, 32);
+        const double c = (double)r * 1024.0 / (r >= 2 ? 0.46 : 0.39);
         if (c < best)
-            best = c, pick = r1 <= r2 ? 4 : 5;
+            best = c, pick = 4;
+    }
+    if (dma_applies<1, 1, 4, 2, 16>(M, N, K, transA, transB, avec, bvec, nbatch))
+    {
+        const double c = (double)rounds(64, 32) * 2048.0 / 0.53;
+        if (c < best)
+            best = c, pick = 5;
     }
 #ifdef REPDL_DEBUG_HOOKS
     if (g_force_tile > 0)
@@ -1227,17 +1236,9 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
     case 3:
         return launch_dma<2, 2, 2, 2, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 4:
-        return launch_dma<1, 1, 4, 1, 16, 7, 5>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+        return launch_dma<1, 1, 2, 2, 16, 7, 5>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 5:
-        return launch_dma<1, 1, 1, 4, 16, 7, 5>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
-#ifdef REPDL_DEBUG_HOOKS
-    case 6:
-        return launch_dma<8, 4, 2, 4, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
-    case 7:
-        return launch_dma<4, 4, 2, 2, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
-    case 8:
-        return launch_dma<4, 2, 2, 4, 8, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
-#endif
+        return launch_dma<1, 1, 4, 2, 16, 7, 5>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     default:
         return REPDL_E_UNSUPPORTED;
     }

@@ -25,12 +25,12 @@ def test_layouts_and_edges(shape, tA, tB):
 
 # Operands whose rows start on 16-byte boundaries take the kernel that moves them from global memory
 # straight into LDS.  Whole-tile shapes for each of its tile configurations (128x128; 64x64 with the
-# shallow and the deep k-tile; 64x16; 16x64), then shapes that hang over the tile edges, K that
+# shallow and the deep k-tile; 32x32; 64x32), then shapes that hang over the tile edges, K that
 # leaves a tail behind the last whole k-tile, K shorter than one k-tile, and the smallest extents.
 WHOLE_TILE_SHAPES = [(4096, 4096, 48), (2048, 2048, 80), (512, 512, 96), (512, 512, 48), (64, 1024, 128), (48, 1024, 192),
                      (256, 192, 128), (128, 128, 2048),
                      (260, 132, 1000), (100, 36, 52), (4, 4, 4), (68, 20, 24), (1028, 2052, 36), (2500, 1300, 76), (8, 4100, 12),
-                     (132, 260, 1001), (64, 64, 71), (512, 512, 2)]
+                     (132, 260, 1001), (64, 64, 71), (512, 512, 2), (128, 4096, 72), (132, 4100, 40)]
 
 @pytest.mark.parametrize("tA,tB", [(0, 0), (1, 0), (0, 1), (1, 1)])
 @pytest.mark.parametrize("shape", WHOLE_TILE_SHAPES, ids=str)
