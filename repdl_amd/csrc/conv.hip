@@ -2084,6 +2084,355 @@ int launch(const float *gathered, const float *kernel, float *out, const ConvDim
 } // namespace patch
 
 // ---------------------------------------------------------------------------
+// The same layers (3x3, stride 1) with both operands moved from global memory straight into LDS
+// (global_load_lds_dwordx4, see mm.hip) and v_mfma_f32_16x16x4_f32.
+//
+// A workgroup owns 64 rows x TN consecutive pixels of one image (2 x WGN waves of 32 x 32; rows past
+// the last channel repeat it and are not stored).  Per
+// chunk of four source channels (36 k = nine quads of the matrix instruction):
+//   * the kernel operand A[64][36], k contiguous (the kernel itself for forward, a transposed copy
+//     for grad-input), lands as [quad][row][4] -- one bank per lane for the instruction's reads;
+//   * the source patch lands as [channel][patch row][pitch] with pitch = source width + 4: DMA lane
+//     s brings 16 bytes (four columns of one source row) to words 4s .. 4s+3, lanes whose row lies
+//     outside the image or whose columns lie past the row's end are switched off, and their words
+//     keep the zeros written once before the first chunk.  So the four cells after each row are
+//     the zeros right of the image, and -- one row further on -- the zeros left of it; rows above
+//     and below the image are rows of zeros.  Tap (c, kh, kw) of pixel (y, x) is the patch word
+//     c * plane + (y - y0 + dy(kh)) * pitch + x + dx(kw), a per-lane constant for each (quad, lane
+//     group): 18 address registers, every operand read a ds_read_b32 with an immediate.
+// Three LDS buffers, operands read two quads ahead, one barrier per chunk, no vector arithmetic in
+// the loop: the schedule of mm_dma_kernel.  Zeros stand where the reference skips a tap, with the
+// same epilogue as above (NaN results, and zero results when the guard asks, recomputed with the
+// literal chain).
+// ---------------------------------------------------------------------------
+namespace tapdma
+{
+// words per patch row: the source row and four zero cells (rows padded so that the four lane groups
+// of an operand read fall on different banks were measured too: no difference)
+__host__ __device__ inline int patch_pitch(int SW) { return SW + 4; }
+constexpr int CCH = 4, NQ = 9, D = 2, R = D + 1, NB = 3;
+constexpr int QSA = 4 * 64;        // words per quad of the kernel operand
+constexpr int OPA = NQ * QSA;      // words per chunk
+constexpr int BLEAD = 4;           // zero words before the first patch row (the cells left of row 0)
+constexpr int BWORDS = 2048;       // patch words per chunk, at most
+constexpr int BSTR = BLEAD + BWORDS + 12; // words between patch buffers (a multiple of 4)
+constexpr int NIB = BWORDS / 4 / 64;     // DMA instructions of a patch, at most
+
+__device__ __forceinline__ void dma16(const void *base, uint32_t voff, uint32_t lds_byte)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(base), "s"(lds_byte)
+                 : "memory", "m0");
+}
+
+template <int MODE, int WGN>
+__global__ __launch_bounds__(128 * WGN) void conv_tapdma_kernel(const float *__restrict__ Src, // gathered tensor [N][C][SH][SW]
+                                                                const float *__restrict__ Wt,  // the kernel (epilogue)
+                                                                const float *__restrict__ PA,  // kernel operand [M][C * 9]
+                                                                float *__restrict__ Out, ConvDims d, const unsigned *__restrict__ parts_a,
+                                                                int count_a, const unsigned *__restrict__ parts_b, int count_b,
+                                                                int use_guard, int PR)
+{
+    constexpr bool FLIP = MODE == MODE_DGRAD;
+    constexpr int NW = 2 * WGN, NTH = 64 * NW, TN = 32 * WGN;
+    constexpr int CA = (NQ + NW - 1) / NW, CB = (NIB + NW - 1) / NW;
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    extern __shared__ __attribute__((aligned(16))) float smem[]; // [NB][OPA] then [NB][BSTR]
+    __shared__ float bias_s[64];
+    __shared__ unsigned gmin_s[NW][2];
+    float *const As = smem, *const Bs = smem + NB * OPA;
+    // where the dynamic LDS starts (the arrays above lie before it): DMA destinations are LDS byte addresses
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)smem;
+    const int tid = threadIdx.x, lane = tid & 63, l16 = lane & 15, g = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave & 1, wn = wave >> 1;
+    const int C = MODE == MODE_FWD ? d.IC : d.OC, M = MODE == MODE_FWD ? d.OC : d.IC;
+    const int SH = MODE == MODE_FWD ? d.H : d.OH, SW = MODE == MODE_FWD ? d.W : d.OW; // source plane
+    const int PH = MODE == MODE_FWD ? d.OH : d.H, PW = MODE == MODE_FWD ? d.OW : d.W; // output plane
+    const int P = PH * PW, K = C * 9;
+    const int dymin = MODE == MODE_FWD ? -d.pH : d.pH - 2, dxmin = MODE == MODE_FWD ? -d.pW : d.pW - 2;
+    const int n = blockIdx.z, m0 = blockIdx.y * 64, p0 = blockIdx.x * TN;
+    const int y0 = p0 / PW;
+    const int pitch = patch_pitch(SW), gpr = pitch / 4, plane = PR * pitch;
+    const int nslot = CCH * PR * gpr, nib = (nslot + 63) / 64;
+    const int nkt = C / CCH;
+
+    // the guard's parts, requested now and reduced after the main loop
+    unsigned ga = GUARD_NONE, gb = GUARD_NONE;
+    if (use_guard)
+    {
+        for (int i = tid; i < count_a; i += NTH)
+            ga = guard_min(ga, parts_a[i]);
+        for (int i = tid; i < count_b; i += NTH)
+            gb = guard_min(gb, parts_b[i]);
+    }
+    const bool has_bias = MODE == MODE_FWD && d.bias != nullptr;
+    if (has_bias && tid < 64)
+        bias_s[tid] = m0 + tid < M ? d.bias[m0 + tid] : 0.0f;
+    // the patch buffers start as zeros; the DMA only ever writes cells that hold image data
+    for (int i = tid; i < NB * BSTR / 4; i += NTH)
+        reinterpret_cast<v4f *>(Bs)[i] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    // DMA lanes.  Kernel operand: instruction e = quad e, lane = row.  Patch: slot s = (c * PR + i) * gpr + gi.
+    uint32_t va[CA], vb[CB];
+    bool okb[CB];
+    const int arow = m0 + lane < M ? lane : M - 1 - m0; // rows past the last: the last one again, never stored
+#pragma unroll
+    for (int t = 0; t < CA; t++)
+        va[t] = (uint32_t)((arow * K + 4 * (wave + NW * t)) * 4);
+#pragma unroll
+    for (int t = 0; t < CB; t++)
+    {
+        const int sl = 64 * (wave + NW * t) + lane;
+        const int c = sl / (PR * gpr), rem = sl - c * (PR * gpr), i = rem / gpr, gi = rem - i * gpr;
+        const int ys = y0 + dymin + i;
+        okb[t] = sl < nslot && ys >= 0 && ys < SH && 4 * gi < SW;
+        vb[t] = okb[t] ? (uint32_t)(((c * SH + ys) * SW + 4 * gi) * 4) : 0u;
+    }
+    const char *a_base = reinterpret_cast<const char *>(PA + (int64_t)m0 * K);
+    const char *b_base = reinterpret_cast<const char *>(Src + (int64_t)n * C * SH * SW);
+    const int64_t b_step = (int64_t)CCH * SH * SW * 4;
+    auto issue = [&](int buf) {
+#pragma unroll
+        for (int t = 0; t < CA; t++)
+            if (wave + NW * t < NQ)
+                dma16(a_base, va[t], lds0 + (uint32_t)((buf * OPA + (wave + NW * t) * QSA) * 4));
+#pragma unroll
+        for (int t = 0; t < CB; t++)
+            if (wave + NW * t < nib)
+            {
+                if (okb[t])
+                    dma16(b_base, vb[t], lds0 + (uint32_t)((NB * OPA + buf * BSTR + BLEAD + 256 * (wave + NW * t)) * 4));
+            }
+        a_base += CCH * 9 * 4;
+        b_base += b_step;
+    };
+
+    // operand read addresses
+    const float *ra = As + (wm * 32 + l16) * 4 + g;
+    const float *rbp[2][NQ];
+    int pix[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+    {
+        pix[j] = p0 + wn * 32 + 16 * j + l16;
+        const int pc = pix[j] < P ? pix[j] : P - 1;
+        const int y = pc / PW, x = pc - y * PW;
+        const int base = BLEAD + (y - y0) * pitch + x + dxmin;
+#pragma unroll
+        for (int q = 0; q < NQ; q++)
+        {
+            const int k = 4 * q + g, c = k / 9, kh = (k % 9) / 3, kw = k % 3;
+            rbp[j][q] = Bs + base + c * plane + (FLIP ? 2 - kh : kh) * pitch + (FLIP ? 2 - kw : kw);
+        }
+    }
+
+    v4f acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+            acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+    float xa[R][2], xb[R][2];
+    auto read_q = [&](int buf, int q, float(&a)[2], float(&b)[2]) {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+            a[i] = ra[buf * OPA + q * QSA + 64 * i];
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+            b[j] = rbp[j][q][buf * BSTR];
+    };
+    auto mfma_q = [&](float(&a)[2], float(&b)[2]) {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], b[j], acc[i][j], 0, 0, 0);
+    };
+
+    __syncthreads(); // the zeros are in place before any DMA
+#pragma unroll
+    for (int u = 0; u < NB - 1; u++)
+        if (u < nkt)
+            issue(u);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < D; q++)
+        read_q(0, q, xa[q], xb[q]);
+    for (int kt = 0; kt < nkt; kt += NB)
+    {
+#pragma unroll
+        for (int u = 0; u < NB; u++)
+        {
+            if (kt + u >= nkt)
+                break;
+            const bool more1 = kt + u + 1 < nkt, more_dma = kt + u + NB - 1 < nkt;
+#pragma unroll
+            for (int q = 0; q < NQ; q++)
+            {
+                if (q == NQ - D)
+                {
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    __builtin_amdgcn_s_barrier();
+                    asm volatile("" ::: "memory");
+                    if (more_dma)
+                        issue((u + NB - 1) % NB);
+                }
+                const int qq = q + D;
+                if (qq < NQ)
+                    read_q(u, qq, xa[qq % R], xb[qq % R]);
+                else if (more1)
+                    read_q((u + 1) % NB, qq - NQ, xa[qq % R], xb[qq % R]);
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_q(xa[q % R], xb[q % R]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+
+    // the guard: minimum over the workgroup of each operand's parts
+    bool tiny = false;
+    if (use_guard)
+    {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1)
+        {
+            ga = guard_min(ga, (unsigned)__shfl_xor((int)ga, o));
+            gb = guard_min(gb, (unsigned)__shfl_xor((int)gb, o));
+        }
+        if (lane == 0)
+        {
+            gmin_s[wave][0] = ga;
+            gmin_s[wave][1] = gb;
+        }
+        __syncthreads();
+        ga = gmin_s[0][0];
+        gb = gmin_s[0][1];
+#pragma unroll
+        for (int w = 1; w < NW; w++)
+        {
+            ga = guard_min(ga, gmin_s[w][0]);
+            gb = guard_min(gb, gmin_s[w][1]);
+        }
+        tiny = (double)__uint_as_float(ga) * (double)__uint_as_float(gb) < 0x1p-101;
+    }
+
+    float *Oimg = Out + (int64_t)n * M * P;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+        {
+            const int m = m0 + wm * 32 + 16 * i + 4 * g + r;
+            if (m >= M)
+                continue;
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+            {
+                if (pix[j] >= P)
+                    continue;
+                float v = acc[i][j][r];
+                if (guard_suspect(v, tiny))
+                {
+                    const int ph = pix[j] / PW, pw = pix[j] - ph * PW;
+                    v = MODE == MODE_FWD ? conv2d_exact(Src, Wt, d, n, m, ph, pw) : conv2d_grad_input_exact(Src, Wt, d, n, m, ph, pw);
+                }
+                if (has_bias)
+                    v = v + bias_s[m - m0];
+                Oimg[(int64_t)m * P + pix[j]] = v;
+            }
+        }
+}
+
+// The small jobs of a call in one launch: blocks [0, ca) scan the gathered tensor for the guard,
+// the next cb the kernel, the rest (grad-input only) write the kernel operand with k contiguous:
+//   A[m][k = (oc, kh, kw)] = W[oc][m][kh][kw]
+__global__ __launch_bounds__(256) void conv_tapdma_prep_kernel(const float *__restrict__ G, int64_t gcount, int ca,
+                                                               const float *__restrict__ W, int64_t wcount, int cb,
+                                                               unsigned *__restrict__ parts_a, unsigned *__restrict__ parts_b,
+                                                               float *__restrict__ PA, int IC, int OC)
+{
+    const int b = blockIdx.x;
+    if (b < ca)
+    {
+        guard_scan_block(G, gcount, b, ca, parts_a);
+        return;
+    }
+    if (b < ca + cb)
+    {
+        guard_scan_block(W, wcount, b - ca, cb, parts_b);
+        return;
+    }
+    const int64_t idx = (int64_t)(b - ca - cb) * 256 + threadIdx.x;
+    if (idx >= wcount)
+        return;
+    const int K = OC * 9;
+    const int m = (int)(idx / K), k = (int)(idx - (int64_t)m * K);
+    const int oc = k / 9, rem = k - oc * 9;
+    PA[idx] = W[((int64_t)oc * IC + m) * 9 + rem];
+}
+
+// rows of the patch of TN consecutive pixels: the image rows they span, and two more
+inline int patch_rows(int TN, int PW) { return (TN + PW - 2) / PW + 1 + 2; }
+
+template <int MODE>
+bool applies(const ConvDims &d, const float *gathered, const float *kernel, int TN)
+{
+    const int C = MODE == MODE_FWD ? d.IC : d.OC, M = MODE == MODE_FWD ? d.OC : d.IC;
+    const int SH = MODE == MODE_FWD ? d.H : d.OH, SW = MODE == MODE_FWD ? d.W : d.OW;
+    const int PH = MODE == MODE_FWD ? d.OH : d.H, PW = MODE == MODE_FWD ? d.OW : d.W;
+    if (!(d.groups == 1 && d.KH == 3 && d.KW == 3 && d.sH == 1 && d.sW == 1 && d.pH <= 2 && d.pW <= 2 && M >= 1 && (M + 63) / 64 <= 65535 &&
+          C % CCH == 0 && C >= CCH && PH >= 1 && PW >= 1 && SH >= 1 && SW >= 4 && SW % 4 == 0 && d.N <= 65535))
+        return false;
+    if ((reinterpret_cast<uintptr_t>(kernel) & 15) != 0 || (reinterpret_cast<uintptr_t>(gathered) & 15) != 0)
+        return false;
+    return (int64_t)patch_rows(TN, PW) * patch_pitch(SW) * CCH <= BWORDS && (int64_t)C * SH * SW * 4 < (1LL << 31) &&
+           (int64_t)64 * C * 9 * 4 < (1LL << 31) && (int64_t)PH * PW < (1LL << 30);
+}
+
+template <int MODE, int WGN>
+int launch(const float *gathered, const float *kernel, float *out, const ConvDims &d, hipStream_t s)
+{
+    constexpr int TN = 32 * WGN;
+    const int C = MODE == MODE_FWD ? d.IC : d.OC, M = MODE == MODE_FWD ? d.OC : d.IC;
+    const int P = MODE == MODE_FWD ? d.OH * d.OW : d.H * d.W, PW = MODE == MODE_FWD ? d.OW : d.W;
+    const int64_t gcount = (int64_t)d.N * C * (MODE == MODE_FWD ? (int64_t)d.H * d.W : (int64_t)d.OH * d.OW);
+    const int64_t wcount = (int64_t)d.OC * d.IC * 9;
+    // the reference skips taps at every border of a 3x3 kernel unless forward runs without padding
+    const bool skips = MODE == MODE_DGRAD || d.pH > 0 || d.pW > 0;
+    const size_t pa_bytes = MODE == MODE_DGRAD ? ((size_t)wcount * sizeof(float) + 255) / 256 * 256 : 0;
+    char *ws = nullptr;
+    const hipError_t e0 = hipMallocAsync(reinterpret_cast<void **>(&ws), GUARD_BYTES + pa_bytes, s);
+    if (e0 != hipSuccess)
+        return (int)e0;
+    unsigned *guard = reinterpret_cast<unsigned *>(ws);
+    float *PA = reinterpret_cast<float *>(ws + GUARD_BYTES);
+    const int ca = skips ? guard_blocks(gcount) : 0, cb = skips ? guard_blocks(wcount) : 0;
+    const int wb = MODE == MODE_DGRAD ? (int)repdl_cdiv(wcount, 256) : 0;
+    if (ca + cb + wb > 0)
+        hipLaunchKernelGGL(conv_tapdma_prep_kernel, dim3((unsigned)(ca + cb + wb)), dim3(256), 0, s, gathered, gcount, ca, kernel, wcount,
+                           cb, guard_parts(guard, 0), guard_parts(guard, 1), PA, d.IC, d.OC);
+    constexpr size_t shmem = (size_t)NB * (OPA + BSTR) * sizeof(float);
+    auto kern = &conv_tapdma_kernel<MODE, WGN>;
+    if (shmem > 48 * 1024)
+    {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        if (e != hipSuccess)
+        {
+            (void)hipFreeAsync(ws, s);
+            return (int)e;
+        }
+    }
+    const dim3 grid((unsigned)repdl_cdiv(P, TN), (unsigned)repdl_cdiv(M, 64), (unsigned)d.N);
+    hipLaunchKernelGGL(kern, grid, dim3(128 * WGN), shmem, s, gathered, kernel, MODE == MODE_DGRAD ? PA : kernel, out, d,
+                       guard_parts(guard, 0), ca, guard_parts(guard, 1), cb, skips ? 1 : 0, patch_rows(TN, PW));
+    const int rc = repdl_launch_status();
+    const hipError_t e = hipFreeAsync(ws, s);
+    return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
+}
+} // namespace tapdma
+
+// ---------------------------------------------------------------------------
 // 1x1 kernels at stride 1 without padding: forward and grad-input are plain products per image,
 //     Out[m][pixel] = sum_c A[m][c] * Src[c][pixel],
 // and Src is already what the matrix instruction wants: lanes 0-31 of an operand register take 32
@@ -2235,6 +2584,10 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
     const bool mfma = repdl_mfma_exact();
     if (mfma && patch::applies<MODE>(d, kernel))
         return patch::launch<MODE>(gathered, kernel, out, d, s);
+    // other widths in fours (28x28: 128 -> 128 forward 0.208 -> 0.167 ms; at 56x56 the kernel above is the
+    // faster one, 0.156 against 0.162 ms)
+    if (mfma && tapdma::applies<MODE>(d, gathered, kernel, 64))
+        return tapdma::launch<MODE, 2>(gathered, kernel, out, d, s);
     // (chains of 64 terms or fewer: the streaming kernel, which has no prologue to fill -- batch 64,
     // 56x56, 64 channels in, 256 out: 0.087 against 0.098 ms)
     const bool short_chain = K <= 64 && point::applies<MODE>(d);

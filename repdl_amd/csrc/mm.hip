@@ -874,6 +874,8 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__re
     typedef float v4f __attribute__((ext_vector_type(4)));
     extern __shared__ __attribute__((aligned(16))) float smem[]; // [NB][OPA] then [NB][OPB]
 
+    // where the dynamic LDS starts: DMA destinations are LDS byte addresses
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)smem;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WGM, wn = wave / WGM;
@@ -914,7 +916,7 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__re
             const int64_t r = (w & ~3) + 3 < am ? (w & ~3) : am - 4;
             va[t] = (uint32_t)(((int64_t)(4 * q + (w & 3)) * lda + r) * 4);
         }
-        la[t] = __builtin_amdgcn_readfirstlane(64 * e * 16);
+        la[t] = __builtin_amdgcn_readfirstlane(lds0 + 64 * e * 16);
     }
 #pragma unroll
     for (int t = 0; t < CB; t++)
@@ -930,7 +932,7 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__re
             const int64_t r = (w & ~3) + 3 < bn ? (w & ~3) : bn - 4;
             vb[t] = (uint32_t)(((int64_t)(4 * q + (w & 3)) * ldb + r) * 4);
         }
-        lb[t] = __builtin_amdgcn_readfirstlane(NB * OPA * 4 + 64 * e * 16);
+        lb[t] = __builtin_amdgcn_readfirstlane(lds0 + NB * OPA * 4 + 64 * e * 16);
     }
     const char *a_base = reinterpret_cast<const char *>(A_KC ? A + m0 * lda : A + m0);
     const char *b_base = reinterpret_cast<const char *>(B_KC ? B + n0 * ldb : B + n0);

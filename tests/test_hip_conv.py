@@ -44,6 +44,12 @@ FWD = [
     (2, 32, 33, 40, 64, 1, 1, 1, 1, 0, 0, 1),      # 1320 pixels: 10.3 tiles
     (1, 16, 32, 32, 128, 1, 1, 1, 1, 0, 0, 1),     # two row tiles forward, 16 channels: one step of the stream
     (3, 64, 30, 45, 64, 1, 1, 1, 1, 0, 0, 1),      # 1350 pixels, the last tile half full
+    # 3x3 at stride 1, source width in fours, channels in fours: both operands straight into LDS
+    (2, 32, 20, 24, 64, 3, 3, 1, 1, 1, 1, 1),      # (also above) 480 pixels: 7.5 tiles of 64
+    (3, 8, 12, 28, 40, 3, 3, 1, 1, 1, 1, 1),       # 40 rows of a 64-row tile forward, 8 in grad-input
+    (2, 16, 9, 112, 72, 3, 3, 1, 1, 0, 2, 1),      # wide rows (a tile inside one row), no padding above, two columns left
+    (1, 4, 8, 8, 4, 3, 3, 1, 1, 2, 2, 1),          # one chunk, padding 2, eight patch rows for a tile
+    (2, 132, 10, 12, 68, 3, 3, 1, 1, 1, 0, 1),     # 33 chunks (three buffers: 11 turns), ragged rows both ways
     # 1x1 at stride 1 without padding, pixels in fours, channels in fours: a batch of matrix products per image
     (2, 96, 20, 20, 72, 1, 1, 1, 1, 0, 0, 1),      # 400 pixels, 72 rows forward (96 in grad-input): tile edges both ways
     (3, 128, 33, 40, 192, 1, 1, 1, 1, 0, 0, 1),    # chains of 128 (forward) and 192 (grad-input) terms
