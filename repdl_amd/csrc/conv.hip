@@ -2107,24 +2107,29 @@ int launch(const float *gathered, const float *kernel, float *out, const ConvDim
 // ---------------------------------------------------------------------------
 namespace tapdma
 {
-// words per patch row: the source row and four zero cells (rows padded so that the four lane groups
-// of an operand read fall on different banks were measured too: no difference)
-__host__ __device__ inline int patch_pitch(int SW) { return SW + 4; }
+// words per patch row: the source row and the zero cells after it -- four where the DMA moves 16
+// bytes per lane (source width in fours), two where it moves 4 (any width).  (Rows padded so that
+// the four lane groups of an operand read fall on different banks were measured too: no difference.)
+__host__ __device__ inline int patch_pitch(int SW, int vec) { return SW + (vec == 4 ? 4 : 2); }
 constexpr int CCH = 4, NQ = 9, D = 2, R = D + 1, NB = 3;
 constexpr int QSA = 4 * 64;        // words per quad of the kernel operand
 constexpr int OPA = NQ * QSA;      // words per chunk
 constexpr int BLEAD = 4;           // zero words before the first patch row (the cells left of row 0)
 constexpr int BWORDS = 2048;       // patch words per chunk, at most
 constexpr int BSTR = BLEAD + BWORDS + 12; // words between patch buffers (a multiple of 4)
-constexpr int NIB = BWORDS / 4 / 64;     // DMA instructions of a patch, at most
 
 __device__ __forceinline__ void dma16(const void *base, uint32_t voff, uint32_t lds_byte)
 {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(base), "s"(lds_byte)
                  : "memory", "m0");
 }
+__device__ __forceinline__ void dma4(const void *base, uint32_t voff, uint32_t lds_byte)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(voff), "s"(base), "s"(lds_byte)
+                 : "memory", "m0");
+}
 
-template <int MODE, int WGN>
+template <int MODE, int WGN, int VEC>
 __global__ __launch_bounds__(128 * WGN) void conv_tapdma_kernel(const float *__restrict__ Src, // gathered tensor [N][C][SH][SW]
                                                                 const float *__restrict__ Wt,  // the kernel (epilogue)
                                                                 const float *__restrict__ PA,  // kernel operand [M][C * 9]
@@ -2134,6 +2139,7 @@ __global__ __launch_bounds__(128 * WGN) void conv_tapdma_kernel(const float *__r
 {
     constexpr bool FLIP = MODE == MODE_DGRAD;
     constexpr int NW = 2 * WGN, NTH = 64 * NW, TN = 32 * WGN;
+    constexpr int NIB = BWORDS / VEC / 64; // DMA instructions of a patch, at most
     constexpr int CA = (NQ + NW - 1) / NW, CB = (NIB + NW - 1) / NW;
     typedef float v4f __attribute__((ext_vector_type(4)));
     extern __shared__ __attribute__((aligned(16))) float smem[]; // [NB][OPA] then [NB][BSTR]
@@ -2152,7 +2158,7 @@ __global__ __launch_bounds__(128 * WGN) void conv_tapdma_kernel(const float *__r
     const int dymin = MODE == MODE_FWD ? -d.pH : d.pH - 2, dxmin = MODE == MODE_FWD ? -d.pW : d.pW - 2;
     const int n = blockIdx.z, m0 = blockIdx.y * 64, p0 = blockIdx.x * TN;
     const int y0 = p0 / PW;
-    const int pitch = patch_pitch(SW), gpr = pitch / 4, plane = PR * pitch;
+    const int pitch = patch_pitch(SW, VEC), gpr = pitch / VEC, plane = PR * pitch; // gpr: DMA lanes per patch row
     const int nslot = CCH * PR * gpr, nib = (nslot + 63) / 64;
     const int nkt = C / CCH;
 
@@ -2185,8 +2191,8 @@ __global__ __launch_bounds__(128 * WGN) void conv_tapdma_kernel(const float *__r
         const int sl = 64 * (wave + NW * t) + lane;
         const int c = sl / (PR * gpr), rem = sl - c * (PR * gpr), i = rem / gpr, gi = rem - i * gpr;
         const int ys = y0 + dymin + i;
-        okb[t] = sl < nslot && ys >= 0 && ys < SH && 4 * gi < SW;
-        vb[t] = okb[t] ? (uint32_t)(((c * SH + ys) * SW + 4 * gi) * 4) : 0u;
+        okb[t] = sl < nslot && ys >= 0 && ys < SH && VEC * gi < SW;
+        vb[t] = okb[t] ? (uint32_t)(((c * SH + ys) * SW + VEC * gi) * 4) : 0u;
     }
     const char *a_base = reinterpret_cast<const char *>(PA + (int64_t)m0 * K);
     const char *b_base = reinterpret_cast<const char *>(Src + (int64_t)n * C * SH * SW);
@@ -2201,7 +2207,12 @@ __global__ __launch_bounds__(128 * WGN) void conv_tapdma_kernel(const float *__r
             if (wave + NW * t < nib)
             {
                 if (okb[t])
-                    dma16(b_base, vb[t], lds0 + (uint32_t)((NB * OPA + buf * BSTR + BLEAD + 256 * (wave + NW * t)) * 4));
+                {
+                    if (VEC == 4)
+                        dma16(b_base, vb[t], lds0 + (uint32_t)((NB * OPA + buf * BSTR + BLEAD + 256 * (wave + NW * t)) * 4));
+                    else
+                        dma4(b_base, vb[t], lds0 + (uint32_t)((NB * OPA + buf * BSTR + BLEAD + 64 * (wave + NW * t)) * 4));
+                }
             }
         a_base += CCH * 9 * 4;
         b_base += b_step;
@@ -2376,21 +2387,23 @@ __global__ __launch_bounds__(256) void conv_tapdma_prep_kernel(const float *__re
 inline int patch_rows(int TN, int PW) { return (TN + PW - 2) / PW + 1 + 2; }
 
 template <int MODE>
-bool applies(const ConvDims &d, const float *gathered, const float *kernel, int TN)
+bool applies(const ConvDims &d, const float *gathered, const float *kernel, int TN, int vec)
 {
     const int C = MODE == MODE_FWD ? d.IC : d.OC, M = MODE == MODE_FWD ? d.OC : d.IC;
     const int SH = MODE == MODE_FWD ? d.H : d.OH, SW = MODE == MODE_FWD ? d.W : d.OW;
     const int PH = MODE == MODE_FWD ? d.OH : d.H, PW = MODE == MODE_FWD ? d.OW : d.W;
     if (!(d.groups == 1 && d.KH == 3 && d.KW == 3 && d.sH == 1 && d.sW == 1 && d.pH <= 2 && d.pW <= 2 && M >= 1 && (M + 63) / 64 <= 65535 &&
-          C % CCH == 0 && C >= CCH && PH >= 1 && PW >= 1 && SH >= 1 && SW >= 4 && SW % 4 == 0 && d.N <= 65535))
+          C % CCH == 0 && C >= CCH && PH >= 1 && PW >= 1 && SH >= 1 && SW >= 1 && d.N <= 65535))
         return false;
-    if ((reinterpret_cast<uintptr_t>(kernel) & 15) != 0 || (reinterpret_cast<uintptr_t>(gathered) & 15) != 0)
+    if ((reinterpret_cast<uintptr_t>(kernel) & 15) != 0)
         return false;
-    return (int64_t)patch_rows(TN, PW) * patch_pitch(SW) * CCH <= BWORDS && (int64_t)C * SH * SW * 4 < (1LL << 31) &&
+    if (vec == 4 && (SW % 4 != 0 || (reinterpret_cast<uintptr_t>(gathered) & 15) != 0))
+        return false;
+    return (int64_t)patch_rows(TN, PW) * patch_pitch(SW, vec) * CCH <= BWORDS && (int64_t)C * SH * SW * 4 < (1LL << 31) &&
            (int64_t)64 * C * 9 * 4 < (1LL << 31) && (int64_t)PH * PW < (1LL << 30);
 }
 
-template <int MODE, int WGN>
+template <int MODE, int WGN, int VEC>
 int launch(const float *gathered, const float *kernel, float *out, const ConvDims &d, hipStream_t s)
 {
     constexpr int TN = 32 * WGN;
@@ -2413,7 +2426,7 @@ int launch(const float *gathered, const float *kernel, float *out, const ConvDim
         hipLaunchKernelGGL(conv_tapdma_prep_kernel, dim3((unsigned)(ca + cb + wb)), dim3(256), 0, s, gathered, gcount, ca, kernel, wcount,
                            cb, guard_parts(guard, 0), guard_parts(guard, 1), PA, d.IC, d.OC);
     constexpr size_t shmem = (size_t)NB * (OPA + BSTR) * sizeof(float);
-    auto kern = &conv_tapdma_kernel<MODE, WGN>;
+    auto kern = &conv_tapdma_kernel<MODE, WGN, VEC>;
     if (shmem > 48 * 1024)
     {
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
@@ -2586,8 +2599,11 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
         return patch::launch<MODE>(gathered, kernel, out, d, s);
     // other widths in fours (28x28: 128 -> 128 forward 0.208 -> 0.167 ms; at 56x56 the kernel above is the
     // faster one, 0.156 against 0.162 ms)
-    if (mfma && tapdma::applies<MODE>(d, gathered, kernel, 64))
-        return tapdma::launch<MODE, 2>(gathered, kernel, out, d, s);
+    if (mfma && tapdma::applies<MODE>(d, gathered, kernel, 64, 4))
+        return tapdma::launch<MODE, 2, 4>(gathered, kernel, out, d, s);
+    // any other width, 4 bytes per DMA lane
+    if (mfma && tapdma::applies<MODE>(d, gathered, kernel, 64, 1))
+        return tapdma::launch<MODE, 2, 1>(gathered, kernel, out, d, s);
     // (chains of 64 terms or fewer: the streaming kernel, which has no prologue to fill -- batch 64,
     // 56x56, 64 channels in, 256 out: 0.087 against 0.098 ms)
     const bool short_chain = K <= 64 && point::applies<MODE>(d);
@@ -2841,6 +2857,7 @@ __global__ __launch_bounds__(256) void conv_mm_out_kernel(const float *__restric
 // is the faster one, 0.29 against 0.34 ms for 256 -> 256 3x3.)
 inline bool conv_prefers_mm(const ConvDims &d, int64_t M, int64_t K, int64_t P)
 {
+
     return d.groups == 1 && P <= 100 && K >= 512 && M >= 128 && (int64_t)d.N * P >= 2048 && (int64_t)d.N * P * K < (1LL << 31) &&
            (int64_t)d.N * P * M < (1LL << 31) && M * K < (1LL << 31) && repdl_mfma_exact();
 }
@@ -2919,7 +2936,10 @@ REPDL_API int repdl_hip_conv2d_bias(const float *input, const float *kernel, con
     REPDL_REQUIRE(fits_i32(OH * sH + KH + pH) && fits_i32(OW * sW + KW + pW));
     ConvDims d{(int)N, (int)IC, (int)H, (int)W, (int)OC, (int)KH, (int)KW, (int)OH,
                (int)OW, (int)sH, (int)sW, (int)pH, (int)pW, (int)groups, bias};
-    if (conv_prefers_mm(d, OC, IC * KH * KW, OH * OW))
+    // (3x3 kernels at stride 1 have a kernel of their own that is faster than the product also on small
+    // images: 512 -> 512 at 7x7, batch 64, 0.26 -> 0.19 ms; at 10x10 0.48 -> 0.34)
+    const bool tap = repdl_mfma_exact() && tapdma::applies<MODE_FWD>(d, input, kernel, 64, 1);
+    if (!tap && conv_prefers_mm(d, OC, IC * KH * KW, OH * OW))
         return launch_conv_mm<MODE_FWD>(input, kernel, output, d, stream);
     return launch_conv_gemm<MODE_FWD>(input, kernel, output, d, stream);
 }
@@ -2941,7 +2961,8 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
     REPDL_REQUIRE(fits_i32(H + pH + KH) && fits_i32(W + pW + KW) && fits_i32(IC * KH * KW * 4));
     ConvDims d{(int)N, (int)IC, (int)H, (int)W, (int)OC, (int)KH, (int)KW, (int)OH,
                (int)OW, (int)sH, (int)sW, (int)pH, (int)pW, 1};
-    if (OC * OH * OW > 0 && conv_prefers_mm(d, IC, OC * KH * KW, H * W))
+    const bool tap = repdl_mfma_exact() && OC * OH * OW > 0 && tapdma::applies<MODE_DGRAD>(d, grad_output, kernel, 64, 1);
+    if (!tap && OC * OH * OW > 0 && conv_prefers_mm(d, IC, OC * KH * KW, H * W))
         return launch_conv_mm<MODE_DGRAD>(grad_output, kernel, grad_input, d, stream);
     return launch_conv_gemm<MODE_DGRAD>(grad_output, kernel, grad_input, d, stream);
 }

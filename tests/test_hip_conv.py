@@ -50,6 +50,11 @@ FWD = [
     (2, 16, 9, 112, 72, 3, 3, 1, 1, 0, 2, 1),      # wide rows (a tile inside one row), no padding above, two columns left
     (1, 4, 8, 8, 4, 3, 3, 1, 1, 2, 2, 1),          # one chunk, padding 2, eight patch rows for a tile
     (2, 132, 10, 12, 68, 3, 3, 1, 1, 1, 0, 1),     # 33 chunks (three buffers: 11 turns), ragged rows both ways
+    # the same with 4 bytes per DMA lane: any width
+    (3, 64, 14, 14, 64, 3, 3, 1, 1, 1, 1, 1),
+    (2, 16, 11, 30, 24, 3, 3, 1, 1, 2, 1, 1),      # rows of 30, padding 2 above and below, 24 rows
+    (5, 128, 7, 7, 128, 3, 3, 1, 1, 1, 1, 1),      # an image smaller than a tile
+    (2, 8, 6, 61, 20, 3, 3, 1, 1, 0, 0, 1),        # no padding: 4x59 output, nothing skipped forward
     # 1x1 at stride 1 without padding, pixels in fours, channels in fours: a batch of matrix products per image
     (2, 96, 20, 20, 72, 1, 1, 1, 1, 0, 0, 1),      # 400 pixels, 72 rows forward (96 in grad-input): tile edges both ways
     (3, 128, 33, 40, 192, 1, 1, 1, 1, 0, 0, 1),    # chains of 128 (forward) and 192 (grad-input) terms
