@@ -78,6 +78,13 @@ LEG_KERNELS = {
 }
 
 
+def sha(t) -> str:
+    return hashlib.sha256(t.detach().cpu().contiguous().numpy().tobytes()).hexdigest()
+
+
+# ----------------------------------------------------------------------------------------------
+# rocprofv3 summaries (no GPU needed)
+# ----------------------------------------------------------------------------------------------
 def _short(name: str) -> str:
     return name.replace("(anonymous namespace)::", "").replace("void ", "")
 
