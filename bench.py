@@ -243,6 +243,25 @@ def cpu_time(fn, reps=1):
     return best, r
 
 
+# Legs that a sequential chain keeps off the throughput roofline: the order of the additions (or of the
+# multiply-adds) of one output is fixed, so a launch cannot be shorter than its longest chain at the
+# latency of a dependent instruction (about 10 clocks for v_add_f32 in a lone wave, 35 for a dependent
+# v_mfma_f32_16x16x4_f32 = 8.75 per k), whatever the bandwidth.
+CHAIN_LIMITS = {
+    "sum2d_dim0": "chain latency: 65536 dependent additions per column at ~10 clocks = 0.28 ms",
+    "sum4d_dim023": "chain latency: 64 chains of 200704 additions (0.85 ms if every addition were made one after the other; the "
+                    "interval maps of the parallel evaluation skip about half of them)",
+    "sum1d": "one chain of 2^28 additions (1.1 s at 10 clocks each): evaluated exactly in parallel by interval maps over candidate "
+             "states, three passes over the input and about nine rounds of speculative walks",
+    "sum1d_drift": "one chain of 2^28 additions: as above, fewer rounds because the sum's magnitude only grows",
+    "conv3x3_wgrad": "chain latency: every output is a chain of 200704 multiply-adds; 50176 dependent 16x16x4 matrix instructions "
+                     "at 35 clocks = 0.75-0.80 ms (measured with everything but the chain switched off: 0.80 ms)",
+    "conv1x1_wgrad": "chain latency: as the 3x3 layer, 200704-term chains on 64 blocks of 16x16 outputs (floor 0.80 ms)",
+    "softmax": "vector ALU: the correctly rounded exp (about 30 instructions per element) and the division, plus a 1000-term chain per row",
+    "cross_entropy": "vector ALU: the correctly rounded exp (about 30 instructions per element), plus a 1000-term chain per row",
+}
+
+
 def leg_entry(name, workload, bound, work, fn, steps, warmup, parity, cpu, traffic_leg=None, default_size=True):
     """One "also" entry: `work` is the algorithmic bytes (bound "hbm") or flop (bound "mfma") of one call."""
     wall, ev_mean, ev_min = time_gpu(fn, steps, warmup, SETTLE_MS)
@@ -256,6 +275,9 @@ def leg_entry(name, workload, bound, work, fn, steps, warmup, parity, cpu, traff
     roof = {"bound": bound, "achieved": round(rate, 3), "peak": peak, "unit": unit, "frac": round(rate / peak, 4), "traffic": traffic}
     if traffic is None:
         roof["traffic_note"] = why
+    limit = CHAIN_LIMITS.get(traffic_leg)
+    if limit is not None and default_size:
+        roof["limited_by"] = limit  # what keeps this leg off the roofline named in "bound"
     out = {"op": name, "workload": workload, "value": round(value, 2), "unit": vunit, "ms_per_step": round(ev_mean, 4),
            "ms_min": round(ev_min, 4), "roofline": roof}
     if parity is not None:
