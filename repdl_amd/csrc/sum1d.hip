@@ -285,15 +285,19 @@ __device__ __forceinline__ double quantise(float x, const Quantum &g)
     return g.q == 0.0 ? (double)x : rint((double)x * g.inv_q) * g.q;
 }
 
-// prev == nullptr: exact sums; else: sums of the elements rounded to the grid of the state
-// prev[block] predicted by the previous pass.
+// prev == nullptr: exact sums, and the sums of the magnitudes in babs; else: sums of the elements
+// rounded to the grid of the state prev[block] predicted by the previous pass -- unless that pass
+// found the refinement pointless for this row (refine[row] == 0: nothing is read, bsum stays).
 __global__ __launch_bounds__(256) void sum1d_blocksum_kernel(const float *__restrict__ x, Chains c,
                                                              const double *__restrict__ prev,
-                                                             double *__restrict__ bsum, int vec)
+                                                             double *__restrict__ bsum, double *__restrict__ babs,
+                                                             const int *__restrict__ refine, int vec)
 {
-    __shared__ double part[4];
+    __shared__ double part[2][4];
     const int tid = threadIdx.x;
     const int64_t row = blockIdx.y;
+    if (prev != nullptr && refine[row] == 0)
+        return;
     x += row * c.row_stride;
     bsum += row * c.nblk;
     float v[16];
@@ -302,28 +306,56 @@ __global__ __launch_bounds__(256) void sum1d_blocksum_kernel(const float *__rest
     g.q = g.inv_q = 0.0;
     if (prev != nullptr)
         g = quantum_of(prev[row * c.nblk + blockIdx.x]);
-    double d = 0.0;
+    double d = 0.0, a = 0.0;
 #pragma unroll
     for (int q = 0; q < 16; q++)
+    {
         d += quantise(v[q], g);
+        a += (double)__builtin_fabsf(v[q]);
+    }
     d = wave_sum(d);
+    if (prev == nullptr)
+        a = wave_sum(a);
     if ((tid & 63) == 0)
-        part[tid >> 6] = d;
+    {
+        part[0][tid >> 6] = d;
+        part[1][tid >> 6] = a;
+    }
     __syncthreads();
     if (tid == 0)
-        bsum[blockIdx.x] = (part[0] + part[1]) + (part[2] + part[3]);
+    {
+        bsum[blockIdx.x] = (part[0][0] + part[0][1]) + (part[0][2] + part[0][3]);
+        if (prev == nullptr)
+            babs[row * c.nblk + blockIdx.x] = (part[1][0] + part[1][1]) + (part[1][2] + part[1][3]);
+    }
 }
 
 // ---- step 2: exclusive prefix of the block sums (one workgroup per row) --------------------
 // Tiles of 8192 sums: a thread owns eight consecutive ones, the workgroup scans the thread totals.
+// First pass (babs given): also decides whether the refinement pass is worth its read of the input,
+// refine[row] = 1 if some block enters at a state whose grid is within 2^5 of the block's mean
+// magnitude -- where elements lose bits that matter, or vanish, the chain drifts away from the exact
+// sum systematically (a sum of 2^28 values in [0,1) stalls at 2^24) and only the refined prediction
+// follows it; where the grid is far finer than the elements the rounding errors have no direction
+// and the rounds re-centre the windows anyway.  Either answer gives the same result: the prediction
+// only places the candidate windows.  Second pass (babs null): nothing to do if refine[row] == 0.
 __global__ __launch_bounds__(1024) void sum1d_prefix_kernel(const double *__restrict__ bsum,
-                                                            double *__restrict__ prefix, int64_t nblk)
+                                                            double *__restrict__ prefix, int64_t nblk,
+                                                            const double *__restrict__ babs, int *__restrict__ refine, int64_t n)
 {
     constexpr int PER = 8;
     __shared__ double wsum[2][16];
+    __shared__ int want_s;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (babs == nullptr && refine[blockIdx.x] == 0)
+        return;
     bsum += (int64_t)blockIdx.x * nblk; // one workgroup per row
     prefix += (int64_t)blockIdx.x * nblk;
+    if (babs != nullptr)
+        babs += (int64_t)blockIdx.x * nblk;
+    if (tid == 0)
+        want_s = 0;
+    bool want = false;
     double carry = 0.0;
     int par = 0;
     for (int64_t base = 0; base < nblk; base += PER * 1024)
@@ -361,11 +393,26 @@ __global__ __launch_bounds__(1024) void sum1d_prefix_kernel(const double *__rest
         for (int d = 0; d < PER; d++)
         {
             if (i0 + d < nblk)
+            {
                 prefix[i0 + d] = run;
+                if (babs != nullptr)
+                {
+                    const int64_t left = n - (i0 + d) * BLK; // elements of this block (the last one may be short)
+                    want = want || quantum_of(run).q * 32.0 * (double)(left < BLK ? left : BLK) >= babs[i0 + d];
+                }
+            }
             run += v[d];
         }
         carry += total;
         par ^= 1;
+    }
+    if (babs != nullptr)
+    {
+        if (want)
+            want_s = 1; // (same value from every writer)
+        __syncthreads();
+        if (tid == 0)
+            refine[blockIdx.x] = want_s;
     }
 }
 
@@ -1381,6 +1428,7 @@ int repdl_sum1d_serial(const float *in, float *out, int64_t n, int average, void
 // already run side by side.
 #ifdef REPDL_DEBUG_HOOKS
 static int g_debug_rounds = -1;
+static int g_debug_norefine = 0;
 #endif
 static int spec_rounds(int64_t rows, int64_t n)
 {
@@ -1397,7 +1445,7 @@ namespace
 {
 struct Layout
 {
-    size_t bsum, prefix, T3, TN, T2, TG, T1, ctl, work, sc, nbase[2], tab[2], worklist, SE, SA, SOK, sbase, HE, HA, HOK, hbase, hc, total;
+    size_t bsum, babs, refine, prefix, T3, TN, T2, TG, T1, ctl, work, sc, nbase[2], tab[2], worklist, SE, SA, SOK, sbase, HE, HA, HOK, hbase, hc, total;
 };
 
 Layout layout(int64_t rows, int64_t n)
@@ -1412,6 +1460,8 @@ Layout layout(int64_t rows, int64_t n)
         return here;
     };
     l.bsum = take(r * nblk * sizeof(double));
+    l.babs = take(r * nblk * sizeof(double));
+    l.refine = take(r * sizeof(int));
     l.prefix = take(r * nblk * sizeof(double));
     l.T3 = take(r * nsup * sizeof(Tup));
     l.TN = take(r * nnode * sizeof(Tup));
@@ -1480,11 +1530,22 @@ int repdl_sum_chains(const float *in, float *out, int64_t rows, int64_t nseg, in
     // 16-byte loads: every row and segment starts on a 16-byte boundary
     const int vec = aligned16(in) && (rows == 1 || row_stride % 4 == 0) && (nseg == 1 || seg_stride % 4 == 0);
     const dim3 g2((unsigned)nblk, (unsigned)rows);
-    hipLaunchKernelGGL(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(nullptr), bsum, vec);
-    hipLaunchKernelGGL(sum1d_prefix_kernel, dim3((unsigned)rows), dim3(1024), 0, s, bsum, prefix, nblk);
+    double *babs = reinterpret_cast<double *>(w + l.babs);
+    int *refine = reinterpret_cast<int *>(w + l.refine);
+    hipLaunchKernelGGL(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(nullptr), bsum, babs,
+                       static_cast<const int *>(refine), vec);
+    hipLaunchKernelGGL(sum1d_prefix_kernel, dim3((unsigned)rows), dim3(1024), 0, s, bsum, prefix, nblk,
+                       static_cast<const double *>(babs), refine, n);
     // one refinement of the prediction (see quantum_of)
-    hipLaunchKernelGGL(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(prefix), bsum, vec);
-    hipLaunchKernelGGL(sum1d_prefix_kernel, dim3((unsigned)rows), dim3(1024), 0, s, bsum, prefix, nblk);
+#ifdef REPDL_DEBUG_HOOKS
+    if (!g_debug_norefine)
+#endif
+    {
+    hipLaunchKernelGGL(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(prefix), bsum, babs,
+                       static_cast<const int *>(refine), vec);
+    hipLaunchKernelGGL(sum1d_prefix_kernel, dim3((unsigned)rows), dim3(1024), 0, s, bsum, prefix, nblk,
+                       static_cast<const double *>(nullptr), refine, n);
+    }
     hipLaunchKernelGGL(sum1d_tuple_kernel, g2, dim3(256), 0, s, in, c, prefix, T1, TG, T2, vec);
     hipLaunchKernelGGL(sum1d_super_kernel, dim3((unsigned)repdl_cdiv(nsup, 4), (unsigned)rows), dim3(256), 0, s, T2, TN, T3, ctl,
                        work, nblk, nnode, nsup);
@@ -1622,6 +1683,7 @@ REPDL_API int repdl_hip_sum1d_static(const float *in, float *out, int64_t n, int
 #ifdef REPDL_DEBUG_HOOKS
 // Development only (not built into the library): force the number of rounds, read a row's front.
 REPDL_API void repdl_debug_sum1d_rounds(int r) { g_debug_rounds = r; }
+REPDL_API void repdl_debug_sum1d_norefine(int v) { g_debug_norefine = v; }
 REPDL_API int repdl_debug_sum1d_front(const void *workspace, int64_t n)
 {
     const Layout l = layout(1, n);
