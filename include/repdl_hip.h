@@ -100,9 +100,8 @@ int repdl_hip_mm_bias(const float *A, const float *B, const float *bias, float *
  * allocator (hipMallocAsync / hipFreeAsync on `stream`): 17 KiB whenever the geometry
  * makes the reference skip taps (padding, strides of grad-input, kernels wider than one
  * tap in grad-input); on the matrix path also a copy of the kernel in the order the matrix
- * instruction reads it (3x3 kernels at stride 1: for some widths only in grad-input, and 1x1
- * kernels with chains of at most 64 terms; a 1x1 kernel at stride 1 without padding otherwise
- * takes none at all), or for the
+ * instruction reads it (3x3 kernels at stride 1 in grad-input, and 1x1 kernels with chains of
+ * at most 64 terms; 3x3 forward and the other 1x1 kernels at stride 1 take nothing else), or for the
  * remaining shapes a zero-padded copy of the gathered operand
  * of conv2d / conv2d_grad_input with two small offset tables (or, for images of at most
  * 100 pixels with many channels, its im2col: output elements x IC*KH*KW floats), and for conv2d_grad_kernel

@@ -1762,348 +1762,32 @@ inline bool wgrad_prefers_gemm(int64_t OC, int64_t NC, int64_t K)
 }
 
 // ---------------------------------------------------------------------------
-// Forward and grad-input of 3x3 kernels at stride 1 from an INPUT PATCH in LDS.
+// Forward and grad-input of 3x3 kernels at stride 1 from an INPUT PATCH in LDS, both operands moved
+// from global memory straight into LDS (global_load_lds, see mm.hip), v_mfma_f32_16x16x4_f32.
 //
-// The implicit GEMM above fetches the gathered operand tap by tap: nine global loads and nine
-// LDS stores per input value, from a zero-padded copy of the whole tensor that a separate pass
-// writes first.  Here a workgroup owns 64 rows (channels out) x 128 consecutive pixels of one
-// image and brings the patch of the source those pixels touch -- the rows above and below and
-// the columns left and right included, zeros where the image ends (buffer loads return zero
-// for offsets marked out of range) -- into LDS once per chunk of CCH source channels.  The
-// nine shifted operands of a channel are then the same LDS words read at nine constant offsets:
-//     B[k = (c, kh, kw)][pixel (y, x)] = patch[c][(y - y0) + dyi(kh)][x + dxi(kw)]
-// with dyi(kh) = kh, dxi(kw) = kw for forward and 2 - kh, 2 - kw for grad-input, k running in the
-// reference's order (c, kh, kw).  A wave computes 64 rows x 64 pixels with v_mfma_f32_32x32x2_f32
-// (2 x 2 blocks): lanes 0-31 of an operand register hold the even k of a pair, lanes 32-63 the
-// odd one, whose patch offset differs by one of three constants (next tap in the row, first tap
-// of the next row, first tap of the next channel); three lane address registers, one per constant,
-// make every operand read a ds_read_b32 with an immediate offset, so that a k-pair is one LDS
-// read, two loads of the kernel operand (below) and two matrix instructions, and no vector
-// arithmetic at all (vector instructions and matrix instructions do not overlap on a SIMD).  Padded zeros stand where
-// the reference skips a tap, as in the implicit GEMM, with the same epilogue (NaN results, and
-// zero results when the guard asks, recomputed with the literal chain).  The guard's minima are
-// reduced by every workgroup from the per-block parts of the scan launch: the loads are issued
-// before the main loop and used after it.
-// ---------------------------------------------------------------------------
-namespace patch
-{
-constexpr int CCH = 4;            // source channels per chunk
-constexpr int KC = CCH * 9;       // k-steps per chunk
-constexpr int PITCH = 64;         // LDS words per patch row (image width + 2 <= 64)
-constexpr int ROWS = 7;           // patch rows: 128 consecutive pixels of rows >= 32 wide span 5, + 2
-constexpr int PLANE = ROWS * PITCH;
-constexpr int BSZ = CCH * PLANE;  // words of a patch
-constexpr int BSLOTS = BSZ / 256; // patch words per thread
-
-template <bool FLIP>
-__host__ __device__ constexpr int koff(int k)
-{
-    const int c = k / 9, kh = (k % 9) / 3, kw = k % 3;
-    return c * PLANE + (FLIP ? 2 - kh : kh) * PITCH + (FLIP ? 2 - kw : kw);
-}
-// which of the three lane address registers serves the pair (k, k + 1), k even
-__host__ __device__ constexpr int pair_kind(int k) { return (k % 9 == 8) ? 2 : ((k % 3 == 2) ? 1 : 0); }
-template <bool FLIP>
-__host__ __device__ constexpr int pair_delta(int kind)
-{
-    return kind == 0 ? koff<FLIP>(1) - koff<FLIP>(0) : (kind == 1 ? koff<FLIP>(3) - koff<FLIP>(2) : koff<FLIP>(9) - koff<FLIP>(8));
-}
-
-// The kernel operand comes from a copy in the matrix instruction's own register layout, written
-// by the prep launch: word ((((mt * nch + ch) * (KC / 2) + kp) * 2 + i) * 64 + lane) holds
-// A[mt * 64 + 32 * i + lane % 32][ch * KC + 2 * kp + lane / 32], so that an operand register is
-// one coalesced 256-byte load (all workgroups read the same 9 KiB per chunk: it stays in the
-// vector cache), requested AHEAD pairs before its use.  No LDS, no transposition, no barrier for it.
-// (Measured on the 64 -> 64 layer at 56x56, batch 64, whole call: seven waves per SIMD and three
-// pairs ahead 0.170 ms; 7 / 6: 0.172; 6 / 6: 0.171; 5 / 6: 0.177; 6 / 9: 0.190; 8 / 3: 0.194.)
-constexpr int AHEAD = 3;
-
-template <int MODE>
-__global__ __launch_bounds__(256, 7) void conv_patch_kernel(const float *__restrict__ Src, // gathered tensor [N][C][SH][SW]
-                                                            const float *__restrict__ Wt,  // the kernel (epilogue)
-                                                            const float *__restrict__ PA,  // kernel operand, register layout
-                                                            float *__restrict__ Out, ConvDims d, const unsigned *__restrict__ parts_a,
-                                                            int count_a, const unsigned *__restrict__ parts_b, int count_b, int use_guard)
-{
-    constexpr bool FLIP = MODE == MODE_DGRAD;
-    __shared__ __attribute__((aligned(16))) float Bs[2][BSZ];
-    __shared__ float bias_s[64];
-    __shared__ unsigned gmin_s[4][2];
-    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, half = lane >> 5;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int C = MODE == MODE_FWD ? d.IC : d.OC, M = MODE == MODE_FWD ? d.OC : d.IC;
-    const int SH = MODE == MODE_FWD ? d.H : d.OH, SW = MODE == MODE_FWD ? d.W : d.OW;   // source plane
-    const int PH = MODE == MODE_FWD ? d.OH : d.H, PW = MODE == MODE_FWD ? d.OW : d.W;   // output plane
-    const int P = PH * PW;
-    const int dymin = MODE == MODE_FWD ? -d.pH : d.pH - 2, dxmin = MODE == MODE_FWD ? -d.pW : d.pW - 2;
-    const int n = blockIdx.z, m0 = blockIdx.y * 64, p0 = blockIdx.x * 128;
-    const int y0 = p0 / PW;
-    const int nch = C / CCH;
-
-    // the guard's parts, requested now and reduced after the main loop
-    unsigned ga = GUARD_NONE, gb = GUARD_NONE;
-    if (use_guard)
-    {
-        for (int i = tid; i < count_a; i += 256)
-            ga = guard_min(ga, parts_a[i]);
-        for (int i = tid; i < count_b; i += 256)
-            gb = guard_min(gb, parts_b[i]);
-    }
-
-    // patch slots of this thread: byte offsets into the image (out of range where the image ends)
-    const __amdgpu_buffer_rsrc_t rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(Src + (int64_t)n * C * SH * SW), 0, C * SH * SW * 4, 0x00020000);
-    int b_voff[BSLOTS];
-    {
-        const int plast = p0 + 127 < P ? p0 + 127 : P - 1;
-        const int nrows = plast / PW - y0 + 3;
-#pragma unroll
-        for (int j = 0; j < BSLOTS; j++)
-        {
-            const int sl = tid + 256 * j;
-            const int c = sl / PLANE, i = (sl % PLANE) / PITCH, col = sl % PITCH;
-            const int ys = y0 + dymin + i, xs = dxmin + col;
-            const bool ok = i < nrows && col < PW + 2 && ys >= 0 && ys < SH && xs >= 0 && xs < SW;
-            b_voff[j] = ok ? ((c * SH + ys) * SW + xs) * 4 : (int)0x80000000;
-        }
-    }
-    // the kernel operand of this row tile: chunk ch starts at byte ch * KC * 64 * 4
-    const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<float *>(PA + (int64_t)blockIdx.y * nch * (KC * 64)), 0, nch * KC * 64 * 4, 0x00020000);
-    const int a_voff = lane * 4;
-
-    float fb[BSLOTS];
-    auto load_patch = [&](int ch) {
-        const int soff = ch * CCH * SH * SW * 4;
-#pragma unroll
-        for (int j = 0; j < BSLOTS; j++)
-            fb[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, b_voff[j], soff, 0));
-    };
-
-    // lane addresses (words into a patch buffer): the patch position of this lane's pixel, for each of
-    // the three pair kinds
-    const int pix = p0 + wave * 32 + l32;
-    int b_lane[3];
-    {
-        const int pc = pix < P ? pix : P - 1;
-        const int y = pc / PW, x = pc - y * PW;
-        const int base = (y - y0) * PITCH + x;
-#pragma unroll
-        for (int kd = 0; kd < 3; kd++)
-            b_lane[kd] = base + (half ? pair_delta<FLIP>(kd) : 0);
-    }
-
-    f16v acc[2];
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++)
-            acc[i][r] = 0.0f;
-
-    const bool has_bias = MODE == MODE_FWD && d.bias != nullptr;
-    load_patch(0);
-    if (has_bias && tid < 64)
-        bias_s[tid] = d.bias[m0 + tid];
-#pragma unroll
-    for (int j = 0; j < BSLOTS; j++)
-        Bs[0][tid + 256 * j] = fb[j];
-    // the ring of kernel-operand registers: pair q of the stream (chunk q / 18, pair q % 18) sits in ar[q % AHEAD]
-    float ar[AHEAD][2];
-    auto request_a = [&](int slot, int ch, int kp) {
-        // (the immediate of a buffer load reaches 4095 bytes: the chunk's 9216 bytes in three parts)
-        const int part = kp / 6;
-        const int soff = (ch * KC * 64 + part * 6 * 128) * 4;
-        ar[slot][0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(arsrc, a_voff + ((kp - part * 6) * 128 + 0) * 4, soff, 0));
-        ar[slot][1] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(arsrc, a_voff + ((kp - part * 6) * 128 + 64) * 4, soff, 0));
-    };
-#pragma unroll
-    for (int q = 0; q < AHEAD; q++)
-        request_a(q, 0, q);
-    __syncthreads();
-
-    auto chunk = [&](int ch, auto curc) {
-        constexpr int cur = decltype(curc)::value;
-        if (ch + 1 < nch)
-            load_patch(ch + 1);
-        const float *bs = &Bs[cur][0];
-#pragma unroll
-        for (int kp = 0; kp < KC / 2; kp++)
-        {
-            const int k = 2 * kp;
-            const int kd = pair_kind(k);
-            const int slot = kp % AHEAD; // (KC / 2 is a multiple of AHEAD: the ring position depends on kp alone)
-            const float a0 = ar[slot][0], a1 = ar[slot][1];
-            const float b0 = bs[b_lane[kd] + koff<FLIP>(k)];
-            acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0], 0, 0, 0);
-            acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1], 0, 0, 0);
-            // the pair AHEAD further on takes this one's registers
-            if (kp + AHEAD < KC / 2)
-                request_a(slot, ch, kp + AHEAD);
-            else if (ch + 1 < nch)
-                request_a(slot, ch + 1, kp + AHEAD - KC / 2);
-        }
-        if (ch + 1 < nch)
-        {
-#pragma unroll
-            for (int j = 0; j < BSLOTS; j++)
-                Bs[cur ^ 1][tid + 256 * j] = fb[j]; // (last read before the barrier that ended the previous chunk)
-        }
-        __syncthreads();
-    };
-    static_assert((KC / 2) % AHEAD == 0, "the ring position of a pair must not depend on the chunk");
-    for (int ch = 0; ch < nch; ch += 2)
-    {
-        chunk(ch, std::integral_constant<int, 0>());
-        if (ch + 1 < nch)
-            chunk(ch + 1, std::integral_constant<int, 1>());
-    }
-
-    // the guard: minimum over the workgroup of each operand's parts
-    bool tiny = false;
-    if (use_guard)
-    {
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1)
-        {
-            ga = guard_min(ga, (unsigned)__shfl_xor((int)ga, o));
-            gb = guard_min(gb, (unsigned)__shfl_xor((int)gb, o));
-        }
-        if (lane == 0)
-        {
-            gmin_s[wave][0] = ga;
-            gmin_s[wave][1] = gb;
-        }
-        __syncthreads();
-        ga = guard_min(guard_min(gmin_s[0][0], gmin_s[1][0]), guard_min(gmin_s[2][0], gmin_s[3][0]));
-        gb = guard_min(guard_min(gmin_s[0][1], gmin_s[1][1]), guard_min(gmin_s[2][1], gmin_s[3][1]));
-        tiny = (double)__uint_as_float(ga) * (double)__uint_as_float(gb) < 0x1p-101;
-    }
-
-    float *Oimg = Out + (int64_t)n * M * P;
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++)
-        {
-            const int m = m0 + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3);
-            if (pix >= P)
-                continue;
-            float v = acc[i][r];
-            if (guard_suspect(v, tiny))
-            {
-                const int ph = pix / PW, pw = pix - ph * PW;
-                v = MODE == MODE_FWD ? conv2d_exact(Src, Wt, d, n, m, ph, pw) : conv2d_grad_input_exact(Src, Wt, d, n, m, ph, pw);
-            }
-            if (has_bias)
-                v = v + bias_s[m - m0];
-            Oimg[(int64_t)m * P + pix] = v;
-        }
-}
-
-// The small jobs of a call in one launch: blocks [0, ca) scan the gathered tensor for the guard,
-// the next cb the kernel, the rest write the kernel operand in register layout (see above):
-//   forward     A[m][k] = W[m][k],               k = (ic, kh, kw)
-//   grad-input  A[m][k] = W[oc][m][kh][kw],      k = (oc, kh, kw)
-__global__ __launch_bounds__(256) void conv_patch_prep_kernel(const float *__restrict__ G, int64_t gcount, int ca,
-                                                              const float *__restrict__ W, int64_t wcount, int cb,
-                                                              unsigned *__restrict__ parts_a, unsigned *__restrict__ parts_b,
-                                                              float *__restrict__ PA, int mode, int IC, int K)
-{
-    const int b = blockIdx.x;
-    if (b < ca)
-    {
-        guard_scan_block(G, gcount, b, ca, parts_a);
-        return;
-    }
-    if (b < ca + cb)
-    {
-        guard_scan_block(W, wcount, b - ca, cb, parts_b);
-        return;
-    }
-    const int64_t idx = (int64_t)(b - ca - cb) * 256 + threadIdx.x;
-    if (idx >= wcount)
-        return;
-    const int lane = (int)(idx & 63), i = (int)((idx >> 6) & 1);
-    const int64_t t = idx >> 7;                 // = (mt * nch + ch) * (KC / 2) + kp
-    const int kp = (int)(t % (KC / 2));
-    const int64_t t2 = t / (KC / 2);
-    const int nch = K / KC;
-    const int ch = (int)(t2 % nch), mt = (int)(t2 / nch);
-    const int m = mt * 64 + 32 * i + (lane & 31), k = ch * KC + 2 * kp + (lane >> 5);
-    float v;
-    if (mode == MODE_FWD)
-        v = W[(int64_t)m * K + k];
-    else
-    {
-        const int oc = k / 9, rem = k - oc * 9;
-        v = W[((int64_t)oc * IC + m) * 9 + rem];
-    }
-    PA[idx] = v;
-}
-
-template <int MODE>
-bool applies(const ConvDims &d, const float *kernel)
-{
-    const int C = MODE == MODE_FWD ? d.IC : d.OC, M = MODE == MODE_FWD ? d.OC : d.IC;
-    const int SH = MODE == MODE_FWD ? d.H : d.OH, SW = MODE == MODE_FWD ? d.W : d.OW;
-    const int PH = MODE == MODE_FWD ? d.OH : d.H, PW = MODE == MODE_FWD ? d.OW : d.W;
-    return d.groups == 1 && d.KH == 3 && d.KW == 3 && d.sH == 1 && d.sW == 1 && d.pH <= 2 && d.pW <= 2 && M % 64 == 0 && M / 64 <= 65535 &&
-           C % CCH == 0 && C >= CCH && PW >= 32 && PW + 2 <= PITCH && PH >= 1 && SH >= 1 && SW >= 1 && d.N <= 65535 &&
-           (int64_t)C * SH * SW * 4 < (1LL << 31) && (int64_t)M * C * 9 * 4 < (1LL << 31) && (int64_t)PH * PW < (1LL << 30) &&
-           (reinterpret_cast<uintptr_t>(kernel) & 15) == 0;
-}
-
-template <int MODE>
-int launch(const float *gathered, const float *kernel, float *out, const ConvDims &d, hipStream_t s)
-{
-    const int C = MODE == MODE_FWD ? d.IC : d.OC, M = MODE == MODE_FWD ? d.OC : d.IC;
-    const int P = MODE == MODE_FWD ? d.OH * d.OW : d.H * d.W;
-    const int K = C * 9;
-    const int64_t gcount = (int64_t)d.N * C * (MODE == MODE_FWD ? (int64_t)d.H * d.W : (int64_t)d.OH * d.OW);
-    const int64_t wcount = (int64_t)d.OC * d.IC * 9;
-    // the reference skips taps at every border of a 3x3 kernel unless forward runs without padding
-    const bool skips = MODE == MODE_DGRAD || d.pH > 0 || d.pW > 0;
-    const size_t pa_bytes = ((size_t)wcount * sizeof(float) + 255) / 256 * 256;
-    char *ws = nullptr;
-    const hipError_t e0 = hipMallocAsync(reinterpret_cast<void **>(&ws), GUARD_BYTES + pa_bytes, s);
-    if (e0 != hipSuccess)
-        return (int)e0;
-    unsigned *guard = reinterpret_cast<unsigned *>(ws);
-    float *PA = reinterpret_cast<float *>(ws + GUARD_BYTES);
-    const int ca = skips ? guard_blocks(gcount) : 0, cb = skips ? guard_blocks(wcount) : 0;
-    const int wb = (int)repdl_cdiv(wcount, 256);
-    hipLaunchKernelGGL(conv_patch_prep_kernel, dim3((unsigned)(ca + cb + wb)), dim3(256), 0, s, gathered, gcount, ca, kernel, wcount, cb,
-                       guard_parts(guard, 0), guard_parts(guard, 1), PA, MODE, d.IC, K);
-    const dim3 grid((unsigned)repdl_cdiv(P, 128), (unsigned)(M / 64), (unsigned)d.N);
-    hipLaunchKernelGGL((conv_patch_kernel<MODE>), grid, dim3(256), 0, s, gathered, kernel, PA, out, d, guard_parts(guard, 0), ca,
-                       guard_parts(guard, 1), cb, skips ? 1 : 0);
-    const int rc = repdl_launch_status();
-    const hipError_t e = hipFreeAsync(ws, s);
-    return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
-}
-} // namespace patch
-
-// ---------------------------------------------------------------------------
-// The same layers (3x3, stride 1) with both operands moved from global memory straight into LDS
-// (global_load_lds_dwordx4, see mm.hip) and v_mfma_f32_16x16x4_f32.
-//
-// A workgroup owns 64 rows x TN consecutive pixels of one image (2 x WGN waves of 32 x 32; rows past
-// the last channel repeat it and are not stored).  Per
-// chunk of four source channels (36 k = nine quads of the matrix instruction):
+// The implicit GEMM above fetches the gathered operand tap by tap: nine global loads and nine LDS
+// stores per input value, from a zero-padded copy of the whole tensor that a separate pass writes
+// first.  Here a workgroup owns 64 rows x TN consecutive pixels of one image (2 x WGN waves of
+// 32 x 32; rows past the last channel repeat it and are not stored) and brings the patch of the
+// source those pixels touch into LDS once per chunk of four source channels (36 k = nine quads of
+// the matrix instruction, k running in the reference's order (c, kh, kw)):
 //   * the kernel operand A[64][36], k contiguous (the kernel itself for forward, a transposed copy
-//     for grad-input), lands as [quad][row][4] -- one bank per lane for the instruction's reads;
+//     for grad-input), lands as [quad][row][4];
 //   * the source patch lands as [channel][patch row][pitch] with pitch = source width + 4: DMA lane
 //     s brings 16 bytes (four columns of one source row) to words 4s .. 4s+3, lanes whose row lies
 //     outside the image or whose columns lie past the row's end are switched off, and their words
 //     keep the zeros written once before the first chunk.  So the four cells after each row are
 //     the zeros right of the image, and -- one row further on -- the zeros left of it; rows above
-//     and below the image are rows of zeros.  Tap (c, kh, kw) of pixel (y, x) is the patch word
-//     c * plane + (y - y0 + dy(kh)) * pitch + x + dx(kw), a per-lane constant for each (quad, lane
-//     group): 18 address registers, every operand read a ds_read_b32 with an immediate.
+//     and below the image are rows of zeros.  (Widths that are not multiples of 4, or a tensor off
+//     16-byte boundaries: 4 bytes per DMA lane, pitch = width + 2.)  Tap (c, kh, kw) of pixel (y, x)
+//     is the patch word c * plane + (y - y0 + dy(kh)) * pitch + x + dx(kw), dy(kh) = kh, dx(kw) = kw
+//     for forward and 2 - kh, 2 - kw for grad-input: a per-lane constant for each (quad, lane group),
+//     18 address registers, every operand read a ds_read_b32 with an immediate.
 // Three LDS buffers, operands read two quads ahead, one barrier per chunk, no vector arithmetic in
-// the loop: the schedule of mm_dma_kernel.  Zeros stand where the reference skips a tap, with the
-// same epilogue as above (NaN results, and zero results when the guard asks, recomputed with the
-// literal chain).
+// the loop: the schedule of mm_dma_kernel.  Padded zeros stand where the reference skips a tap, as
+// in the implicit GEMM, with the same epilogue (NaN results, and zero results when the guard asks,
+// recomputed with the literal chain).  The guard's minima are reduced by every workgroup from the
+// per-block parts of the scan launch.
 // ---------------------------------------------------------------------------
 namespace tapdma
 {
@@ -2595,10 +2279,8 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
     const int ovec = aligned16(out) && (P % 4 == 0);
     hipStream_t s = repdl_stream(stream);
     const bool mfma = repdl_mfma_exact();
-    if (mfma && patch::applies<MODE>(d, kernel))
-        return patch::launch<MODE>(gathered, kernel, out, d, s);
-    // other widths in fours (28x28: 128 -> 128 forward 0.208 -> 0.167 ms; at 56x56 the kernel above is the
-    // faster one, 0.156 against 0.162 ms)
+    // 3x3 at stride 1: the input-patch kernel (batch 64: 64 -> 64 at 56x56 0.213 -> 0.149 ms, 128 -> 128 at
+    // 28x28 0.208 -> 0.143, 256 -> 256 at 14x14 0.28 -> 0.18)
     if (mfma && tapdma::applies<MODE>(d, gathered, kernel, 64, 4))
         return tapdma::launch<MODE, 2, 4>(gathered, kernel, out, d, s);
     // any other width, 4 bytes per DMA lane
