@@ -127,7 +127,7 @@ def summarise_counters(dirnames) -> None:
 def _leg_calls(dirname: str, counter: str, spec):
     """The counter summed over each call of a leg: the leg's dispatches in launch order, cut after
     every dispatch of the leg's last kernel; only calls whose first kernel has the leg's launch size
-    (the largest seen, if the leg names none)."""
+    (the one seen most often, if the leg names none: the bench's own workload makes most of the calls)."""
     subs, end = spec["kernels"], spec["kernels"][-1]
     rows = [r for r in csv.DictReader(open(_find(dirname, "*counter_collection.csv")))
             if r["Counter_Name"] == counter and any(x in _short(r["Kernel_Name"]) for x in subs)]
@@ -141,7 +141,8 @@ def _leg_calls(dirname: str, counter: str, spec):
     if not calls:
         return []
     first_grid = lambda c: max(int(r["Grid_Size"]) for r in c if subs[0] in _short(r["Kernel_Name"])) if any(subs[0] in _short(r["Kernel_Name"]) for r in c) else 0
-    grid = spec.get("grid") or max(first_grid(c) for c in calls)
+    grids = [first_grid(c) for c in calls]
+    grid = spec.get("grid") or max(set(grids), key=grids.count)
     return [sum(float(r["Counter_Value"]) for r in c) for c in calls if first_grid(c) == grid]
 
 
