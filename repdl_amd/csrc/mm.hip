@@ -1175,21 +1175,27 @@ int launch_dma(const float *A, const float *B, float *C, const float *cbias, con
 
 // The tile for a batch of products, and its launch; REPDL_E_UNSUPPORTED if mm_dma_kernel cannot
 // take the operands.  Shares of the chip's matrix rate (145 TFLOP/s on the 128x128 tile with many
-// tiles per CU) by tiles per CU r, measured on whole-tile shapes (a CU holds up to three workgroups
-// of the first two tiles at once):
-//   128x128, 8 waves of 64x32, k-tile 16:   r = 1 0.77, 2 0.85, 3 0.88, more 0.97
-//   64x64, 4 waves of 32x32, k-tile 32/16:  r = 1 0.60, 2 0.76, 3 0.86, 4..7 0.88, more 0.92
+// tiles per CU) by tiles per CU r, measured on whole-tile shapes with K = 2048 (a CU holds two or
+// three workgroups of the first two tiles at once):
+//   128x128, 8 waves of 64x32, k-tile 16:  r = 1 0.82, 2 0.94, 3 0.88, 4 0.95, 5 0.83, 6 0.95, 7 0.89,
+//     more 0.97 (an odd count leaves a last round of one workgroup per CU);
+//   64x64: r = 1 0.65, 2 0.82, 3 0.875, 4..7 0.89, more 0.92, on
+//     r = 1: 8 waves of 16x32, k-tile 32, four buffers (1024^2 x 2048: 94-95 TFLOP/s in every layout,
+//            against 81-83 with four waves of 32x32 or with three buffers; chains of 1024 terms
+//            and fewer are over before the fourth buffer pays: three buffers);
+//     r = 2, 3: 8 waves of 16x32, three buffers (2048 x 1024 x 2048: 119 against 113; 1536 x 2048 x 2048: 127 / 125);
+//     r >= 4: 4 waves of 32x32, k-tile 16, six workgroups to a CU (2048^2 x 2048: 128 against 121);
 //   32x32, 4 waves of one 16x16 block, k-tile 64, read-ahead 7 quads, five buffers: 0.39 at r = 1, 0.46 beyond;
 //   64x32, 8 such waves: 0.53 -- for C with fewer 64x64 tiles than CUs: one or two blocks per SIMD, each
 //     a chain of dependent instructions, and what bounds them is L2: the smaller the tile, the more
 //     often an operand row is fetched (a 32x32 tile asks for 64 rows per 1024 outputs; 64x16 tiles,
 //     80 rows, were slower: 42 against 38 us on 64 x 4096 x 4096)
-// (8192^3 NT: 145 / 138 TFLOP/s on the first two; 3072^2 x 4096: 96 / 133; 2048^2 x 4096: 112 / 128;
-// 1408^2 x 4096: 57 / 105; 1024^3: - / 87; 64 x 4096 x 4096: 28 on 64x64, 57 on 32x32; 128 x 4096 x 4096:
-// 67 on 32x32, 77 on 64x32; 256 x 1024 x 8192: 61 on 32x32.)  A tile that
-// hangs over an edge costs what a whole one does.
+// (8192^3 NT: 145 / 138 TFLOP/s on the first two; 3072 x 4096 x 2048: 106-139 by layout / 132-136;
+// 4096 x 2048 x 2048: 136 / 132; 5120 x 4096 x 2048: 121 / 134; 2048^2 x 2048: 118 / 128; 1408^2 x 4096: 57 / 108;
+// 64 x 4096 x 4096: 28 on 64x64, 57 on 32x32; 128 x 4096 x 4096: 67 on 32x32, 77 on 64x32;
+// 256 x 1024 x 8192: 61 on 32x32.)  A tile that hangs over an edge costs what a whole one does.
 #ifdef REPDL_DEBUG_HOOKS
-int g_force_tile = 0; // 1..5: that configuration whatever the shape
+int g_force_tile = 0; // 1..6: that configuration whatever the shape
 #endif
 int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias, const float *rbias, int64_t M, int64_t N,
                     int64_t K, int transA, int transB, int avec, int bvec, int64_t nbatch, MmBatch batch, hipStream_t s)
@@ -1200,17 +1206,19 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
     if (dma_applies<4, 2, 2, 4, 4>(M, N, K, transA, transB, avec, bvec, nbatch))
     {
         const int64_t r = rounds(128, 128);
-        const double c = (double)r * 16384.0 / (r >= 4 ? 0.97 : r == 3 ? 0.88 : r == 2 ? 0.85 : 0.77);
+        static const double e128[8] = {0.82, 0.94, 0.88, 0.95, 0.83, 0.95, 0.89, 0.97};
+        const double c = (double)r * 16384.0 / e128[r < 8 ? r - 1 : 7];
         if (c < best)
             best = c, pick = 1;
     }
-    if (dma_applies<2, 2, 2, 2, 8>(M, N, K, transA, transB, avec, bvec, nbatch))
+    if (dma_applies<1, 2, 4, 2, 8>(M, N, K, transA, transB, avec, bvec, nbatch))
     {
         const int64_t r = rounds(64, 64);
-        const double c = (double)r * 4096.0 / (r >= 8 ? 0.92 : r >= 4 ? 0.88 : r == 3 ? 0.86 : r == 2 ? 0.76 : 0.60);
-        // the deeper k-tile pays when a CU has one workgroup; the shallower one lets six share a CU
+        const double c = (double)r * 4096.0 / (r >= 8 ? 0.92 : r >= 4 ? 0.89 : r == 3 ? 0.875 : r == 2 ? 0.82 : 0.65);
+        // one workgroup per CU: eight waves and, on chains long enough to fill them, four buffers;
+        // two or three: eight waves; more: four waves on the shallower k-tile, six workgroups to a CU
         if (c < best)
-            best = c, pick = r == 1 ? 2 : 3;
+            best = c, pick = r >= 4 ? 3 : r == 1 && K > 1024 ? 2 : 6;
     }
     if (dma_applies<1, 1, 2, 2, 16>(M, N, K, transA, transB, avec, bvec, nbatch))
     {
@@ -1241,7 +1249,9 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
             return launch_dma_t<true, false, 4, 4, 2, 2, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
         return launch_dma<4, 2, 2, 4, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 2:
-        return launch_dma<2, 2, 2, 2, 8, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+        return launch_dma<1, 2, 4, 2, 8, 1, 4>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+    case 6:
+        return launch_dma<1, 2, 4, 2, 8, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 3:
         return launch_dma<2, 2, 2, 2, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 4:
