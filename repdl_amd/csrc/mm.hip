@@ -836,6 +836,10 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_fast_kernel(const float
 // from global memory: the same chain step as the matrix instruction's.  So nothing is padded and
 // no accumulator that is -0 is touched.
 //
+// DW > 0: the workgroup has DW more waves that issue all the DMA and do nothing else; they meet the
+// computing waves at the same barriers (one before the loop, one per whole k-tile) and leave after
+// the last one, when every load has landed.
+//
 // Batch: blockIdx.y selects one of several products with the same shapes, operand b at X + b * stride
 // (stride 0: shared by all).  `cbias` is added per column, `rbias` per row (one rounded addition after
 // the chain, whichever is given; at most one is).
@@ -851,8 +855,8 @@ struct MmBatch
     int64_t a, b, c; // elements between consecutive products' operands and results
 };
 
-template <bool TA, bool TB, int FM, int FN, int WGM, int WGN, int NQ, int D, int NB>
-__global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__restrict__ A, const float *__restrict__ B,
+template <bool TA, bool TB, int FM, int FN, int WGM, int WGN, int NQ, int D, int NB, int DW>
+__global__ __launch_bounds__(64 * (WGM * WGN + DW)) void mm_dma_kernel(const float *__restrict__ A, const float *__restrict__ B,
                                                                float *__restrict__ C, const float *__restrict__ cbias,
                                                                const float *__restrict__ rbias, int64_t M, int64_t N,
                                                                int64_t K, int64_t gx, int64_t gy, int64_t ntiles8, MmBatch batch)
@@ -867,8 +871,9 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__re
     static_assert(NB >= 3, "a buffer being read, one landed or landing, one being filled");
     static_assert((TM * NQ) % 64 == 0 && (TN * NQ) % 64 == 0, "a DMA instruction fills 64 slots");
     constexpr int NIA = TM * NQ / 64, NIB = TN * NQ / 64; // DMA instructions per k-tile
-    constexpr int CA = (NIA + NW - 1) / NW, CB = (NIB + NW - 1) / NW;
-    static_assert(NB == 3 || (NIA % NW == 0 && NIB % NW == 0), "every wave must issue the same number of loads per tile");
+    constexpr int NI = DW > 0 ? DW : NW;                  // waves that issue them: DW waves that do nothing else, or all
+    constexpr int CA = (NIA + NI - 1) / NI, CB = (NIB + NI - 1) / NI;
+    static_assert(NB == 3 || (NIA % NI == 0 && NIB % NI == 0), "every wave must issue the same number of loads per tile");
     constexpr int INFLIGHT = (NB - 3) * (CA + CB); // loads of later tiles that may still be under way at a barrier
     static_assert(INFLIGHT < 64, "vmcnt is a 6-bit counter");
     typedef float v4f __attribute__((ext_vector_type(4)));
@@ -880,6 +885,8 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__re
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WGM, wn = wave / WGM;
     const int l16 = lane & 15, g = lane >> 4;
+    const bool mover = DW > 0 && wave >= NW;              // a wave that only moves operands
+    const int wi = DW > 0 ? (mover ? wave - NW : 0) : wave; // index among the issuing waves
 
     int64_t tile = blockIdx.x;
     if (tile < ntiles8)
@@ -905,7 +912,7 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__re
 #pragma unroll
     for (int t = 0; t < CA; t++)
     {
-        const int e = wave + NW * t, s = 64 * e + lane, q = s / TM, w = s % TM;
+        const int e = wi + NI * t, s = 64 * e + lane, q = s / TM, w = s % TM;
         if (A_KC)
         {
             const int64_t r = w < am ? w : am - 1;
@@ -921,7 +928,7 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__re
 #pragma unroll
     for (int t = 0; t < CB; t++)
     {
-        const int e = wave + NW * t, s = 64 * e + lane, q = s / TN, w = s % TN;
+        const int e = wi + NI * t, s = 64 * e + lane, q = s / TN, w = s % TN;
         if (B_KC)
         {
             const int64_t r = w < bn ? w : bn - 1;
@@ -946,25 +953,54 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__re
     auto issue = [&](int buf, bool tail) {
 #pragma unroll
         for (int t = 0; t < CA; t++)
-            if (NIA % NW == 0 || wave + NW * t < NIA)
+            if (NIA % NI == 0 || wi + NI * t < NIA)
             {
                 if (!tail)
                     dma16(a_base, va[t], la[t] + buf * OPA * 4);
-                else if ((64 * (wave + NW * t) + lane) / TM < tq)
+                else if ((64 * (wi + NI * t) + lane) / TM < tq)
                     dma16(a_base, va[t], la[t] + buf * OPA * 4);
             }
 #pragma unroll
         for (int t = 0; t < CB; t++)
-            if (NIB % NW == 0 || wave + NW * t < NIB)
+            if (NIB % NI == 0 || wi + NI * t < NIB)
             {
                 if (!tail)
                     dma16(b_base, vb[t], lb[t] + buf * OPB * 4);
-                else if ((64 * (wave + NW * t) + lane) / TN < tq)
+                else if ((64 * (wi + NI * t) + lane) / TN < tq)
                     dma16(b_base, vb[t], lb[t] + buf * OPB * 4);
             }
         a_base += a_step;
         b_base += b_step;
     };
+
+    if (mover)
+    {
+        // the same barriers as the computing waves, one per k-tile: wait for the own share of the
+        // next tile, meet, refill the buffer whose reads ended a tile ago
+        if (ntile > 0)
+        {
+#pragma unroll
+            for (int u = 0; u < NB - 1; u++)
+                if (u < ntile)
+                    issue(u, u == nkt);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+        }
+        int buf = NB - 1;
+        for (int64_t kt = 0; kt < nkt; kt++)
+        {
+            if (INFLIGHT > 0 && kt + NB - 2 < nkt)
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(INFLIGHT) : "memory");
+            else
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            if (kt + NB - 1 < ntile)
+                issue(buf, kt + NB - 1 == nkt);
+            buf = buf + 1 == NB ? 0 : buf + 1;
+        }
+        return;
+    }
 
     v4f acc[FM][FN];
 #pragma unroll
@@ -997,7 +1033,7 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__re
     {
 #pragma unroll
         for (int u = 0; u < NB - 1; u++)
-            if (u < ntile)
+            if (DW == 0 && u < ntile)
                 issue(u, u == nkt);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
@@ -1020,13 +1056,15 @@ __global__ __launch_bounds__(64 * WGM *WGN) void mm_dma_kernel(const float *__re
                 {
                     // the next tile (this wave's share) has landed; after the barrier everyone's has,
                     // and every read of the tile before this one has long been consumed
-                    if (INFLIGHT > 0 && kt + u + NB - 2 < nkt)
+                    if (DW > 0)
+                        ;
+                    else if (INFLIGHT > 0 && kt + u + NB - 2 < nkt)
                         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(INFLIGHT) : "memory");
                     else
                         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                     __builtin_amdgcn_s_barrier();
                     asm volatile("" ::: "memory");
-                    if (more_dma)
+                    if (DW == 0 && more_dma)
                         issue((u + NB - 1) % NB, kt + u + NB - 1 == nkt);
                 }
                 const int qq = q + D;
@@ -1138,7 +1176,7 @@ bool dma_applies(int64_t M, int64_t N, int64_t K, int transA, int transB, int av
     return ea * 4 < (1LL << 32) && eb * 4 < (1LL << 32) && repdl_cdiv(M, TM) * repdl_cdiv(N, TN) <= REPDL_I32_MAX;
 }
 
-template <bool TA, bool TB, int FM, int FN, int WGM, int WGN, int NQ, int D, int NB>
+template <bool TA, bool TB, int FM, int FN, int WGM, int WGN, int NQ, int D, int NB, int DW = 0>
 int launch_dma_t(const float *A, const float *B, float *C, const float *cbias, const float *rbias, int64_t M, int64_t N,
                  int64_t K, int64_t nbatch, MmBatch batch, hipStream_t s)
 {
@@ -1147,7 +1185,7 @@ int launch_dma_t(const float *A, const float *B, float *C, const float *cbias, c
     static_assert(shmem <= 160 * 1024, "LDS of one CU");
     const int64_t gx = repdl_cdiv(N, TN), gy = repdl_cdiv(M, TM);
     const int64_t ntiles8 = (gx * gy) & ~(int64_t)7;
-    auto kern = &mm_dma_kernel<TA, TB, FM, FN, WGM, WGN, NQ, D, NB>;
+    auto kern = &mm_dma_kernel<TA, TB, FM, FN, WGM, WGN, NQ, D, NB, DW>;
     if (shmem > 48 * 1024)
     {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1155,47 +1193,47 @@ int launch_dma_t(const float *A, const float *B, float *C, const float *cbias, c
         if (e != hipSuccess)
             return (int)e;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)(gx * gy), (unsigned)nbatch), dim3(64 * WGM * WGN), shmem, s, A, B, C, cbias, rbias, M,
+    hipLaunchKernelGGL(kern, dim3((unsigned)(gx * gy), (unsigned)nbatch), dim3(64 * (WGM * WGN + DW)), shmem, s, A, B, C, cbias, rbias, M,
                        N, K, gx, gy, ntiles8, batch);
     return repdl_launch_status();
 }
 
-template <int FM, int FN, int WGM, int WGN, int NQ, int D, int NB>
+template <int FM, int FN, int WGM, int WGN, int NQ, int D, int NB, int DW = 0>
 int launch_dma(const float *A, const float *B, float *C, const float *cbias, const float *rbias, int64_t M, int64_t N, int64_t K,
                int transA, int transB, int64_t nbatch, MmBatch batch, hipStream_t s)
 {
     if (!transA && !transB)
-        return launch_dma_t<false, false, FM, FN, WGM, WGN, NQ, D, NB>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
+        return launch_dma_t<false, false, FM, FN, WGM, WGN, NQ, D, NB, DW>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
     if (transA && !transB)
-        return launch_dma_t<true, false, FM, FN, WGM, WGN, NQ, D, NB>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
+        return launch_dma_t<true, false, FM, FN, WGM, WGN, NQ, D, NB, DW>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
     if (!transA && transB)
-        return launch_dma_t<false, true, FM, FN, WGM, WGN, NQ, D, NB>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
-    return launch_dma_t<true, true, FM, FN, WGM, WGN, NQ, D, NB>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
+        return launch_dma_t<false, true, FM, FN, WGM, WGN, NQ, D, NB, DW>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
+    return launch_dma_t<true, true, FM, FN, WGM, WGN, NQ, D, NB, DW>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
 }
 
 // The tile for a batch of products, and its launch; REPDL_E_UNSUPPORTED if mm_dma_kernel cannot
 // take the operands.  Shares of the chip's matrix rate (145 TFLOP/s on the 128x128 tile with many
 // tiles per CU) by tiles per CU r, measured on whole-tile shapes with K = 2048 (a CU holds two or
-// three workgroups of the first two tiles at once):
-//   128x128, 8 waves of 64x32, k-tile 16:  r = 1 0.82, 2 0.94, 3 0.88, 4 0.95, 5 0.83, 6 0.95, 7 0.89,
-//     more 0.97 (an odd count leaves a last round of one workgroup per CU);
-//   64x64: r = 1 0.65, 2 0.82, 3 0.875, 4..7 0.89, more 0.92, on
-//     r = 1: 8 waves of 16x32, k-tile 32, four buffers (1024^2 x 2048: 94-95 TFLOP/s in every layout,
-//            against 81-83 with four waves of 32x32 or with three buffers; chains of 1024 terms
-//            and fewer are over before the fourth buffer pays: three buffers);
-//     r = 2, 3: 8 waves of 16x32, three buffers (2048 x 1024 x 2048: 119 against 113; 1536 x 2048 x 2048: 127 / 125);
+// three workgroups of the first two tiles at once).  "+4" = four more waves that only issue the DMA:
+// it pays while a CU holds one workgroup (a lone wave per SIMD issues a DMA instruction about every
+// 60 clocks, two matrix instructions' worth of its chain), and costs 10 % on 8192^3.
+//   128x128, 8 waves of 64x32, k-tile 16:  r = 1 0.88 (+4: 2048^3 119 -> 128 TFLOP/s), 2 0.94, 3 0.88, 4 0.95,
+//     5 0.83, 6 0.95, 7 0.89, more 0.97 (an odd count leaves a last round of one workgroup per CU);
+//   64x64: r = 1 0.73, 2 0.84, 3 0.875, 4..7 0.89, more 0.92, on
+//     r = 1, 2: 8 waves of 16x32, k-tile 32, four buffers, +4 (1024^2 x 2048: 106 TFLOP/s, against 95 without
+//            the four, 81-83 with four waves of 32x32 or with three buffers; 2048 x 1024 x 2048: 122); chains of
+//            1024 terms and fewer are over before the fourth buffer pays: three buffers, +4 only at r = 1;
+//     r = 3: 8 waves of 16x32, three buffers (1536 x 2048 x 2048: 127 against 125);
 //     r >= 4: 4 waves of 32x32, k-tile 16, six workgroups to a CU (2048^2 x 2048: 128 against 121);
-//   32x32, 4 waves of one 16x16 block, k-tile 64, read-ahead 7 quads, five buffers: 0.39 at r = 1, 0.46 beyond;
-//   64x32, 8 such waves: 0.53 -- for C with fewer 64x64 tiles than CUs: one or two blocks per SIMD, each
-//     a chain of dependent instructions, and what bounds them is L2: the smaller the tile, the more
-//     often an operand row is fetched (a 32x32 tile asks for 64 rows per 1024 outputs; 64x16 tiles,
-//     80 rows, were slower: 42 against 38 us on 64 x 4096 x 4096)
+//   32x32, 4 waves of one 16x16 block, k-tile 64, read-ahead 7 quads, five buffers, +4: 0.445 at r = 1, 0.52 beyond;
+//   64x32, 8 such waves, +4: 0.60 -- for C with fewer 64x64 tiles than CUs: one or two blocks per SIMD, each
+//     a chain of dependent instructions (64 x 4096 x 4096: 58 -> 66 TFLOP/s with the four, 128 x 4096 x 4096:
+//     80 -> 91, 256 x 1024 x 8192: 62 -> 72; more buffers changed nothing; 64x16 tiles were slower)
 // (8192^3 NT: 145 / 138 TFLOP/s on the first two; 3072 x 4096 x 2048: 106-139 by layout / 132-136;
-// 4096 x 2048 x 2048: 136 / 132; 5120 x 4096 x 2048: 121 / 134; 2048^2 x 2048: 118 / 128; 1408^2 x 4096: 57 / 108;
-// 64 x 4096 x 4096: 28 on 64x64, 57 on 32x32; 128 x 4096 x 4096: 67 on 32x32, 77 on 64x32;
-// 256 x 1024 x 8192: 61 on 32x32.)  A tile that hangs over an edge costs what a whole one does.
+// 4096 x 2048 x 2048: 136 / 132; 5120 x 4096 x 2048: 121 / 134; 1408^2 x 4096: 57 / 108.)  A tile that hangs
+// over an edge costs what a whole one does.
 #ifdef REPDL_DEBUG_HOOKS
-int g_force_tile = 0; // 1..6: that configuration whatever the shape
+int g_force_tile = 0; // 1..7: that configuration whatever the shape
 #endif
 int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias, const float *rbias, int64_t M, int64_t N,
                     int64_t K, int transA, int transB, int avec, int bvec, int64_t nbatch, MmBatch batch, hipStream_t s)
@@ -1206,7 +1244,7 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
     if (dma_applies<4, 2, 2, 4, 4>(M, N, K, transA, transB, avec, bvec, nbatch))
     {
         const int64_t r = rounds(128, 128);
-        static const double e128[8] = {0.82, 0.94, 0.88, 0.95, 0.83, 0.95, 0.89, 0.97};
+        static const double e128[8] = {0.88, 0.94, 0.88, 0.95, 0.83, 0.95, 0.89, 0.97};
         const double c = (double)r * 16384.0 / e128[r < 8 ? r - 1 : 7];
         if (c < best)
             best = c, pick = 1;
@@ -1214,22 +1252,20 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
     if (dma_applies<1, 2, 4, 2, 8>(M, N, K, transA, transB, avec, bvec, nbatch))
     {
         const int64_t r = rounds(64, 64);
-        const double c = (double)r * 4096.0 / (r >= 8 ? 0.92 : r >= 4 ? 0.89 : r == 3 ? 0.875 : r == 2 ? 0.82 : 0.65);
-        // one workgroup per CU: eight waves and, on chains long enough to fill them, four buffers;
-        // two or three: eight waves; more: four waves on the shallower k-tile, six workgroups to a CU
+        const double c = (double)r * 4096.0 / (r >= 8 ? 0.92 : r >= 4 ? 0.89 : r == 3 ? 0.875 : r == 2 ? 0.84 : 0.73);
         if (c < best)
-            best = c, pick = r >= 4 ? 3 : r == 1 && K > 1024 ? 2 : 6;
+            best = c, pick = r >= 4 ? 3 : r == 3 ? 6 : K > 1024 ? 2 : r == 1 ? 7 : 6;
     }
     if (dma_applies<1, 1, 2, 2, 16>(M, N, K, transA, transB, avec, bvec, nbatch))
     {
         const int64_t r = rounds(32, 32);
-        const double c = (double)r * 1024.0 / (r >= 2 ? 0.46 : 0.39);
+        const double c = (double)r * 1024.0 / (r >= 2 ? 0.52 : 0.445);
         if (c < best)
             best = c, pick = 4;
     }
     if (dma_applies<1, 1, 4, 2, 16>(M, N, K, transA, transB, avec, bvec, nbatch))
     {
-        const double c = (double)rounds(64, 32) * 2048.0 / 0.53;
+        const double c = (double)rounds(64, 32) * 2048.0 / 0.60;
         if (c < best)
             best = c, pick = 5;
     }
@@ -1247,17 +1283,21 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
         // every other shape and layout the eight-wave form is the faster one by 4-6 %.
         if (transA && !transB && K >= 4 * (M > N ? M : N))
             return launch_dma_t<true, false, 4, 4, 2, 2, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
+        if (rounds(128, 128) == 1)
+            return launch_dma<4, 2, 2, 4, 4, 1, 3, 4>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
         return launch_dma<4, 2, 2, 4, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 2:
-        return launch_dma<1, 2, 4, 2, 8, 1, 4>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+        return launch_dma<1, 2, 4, 2, 8, 1, 4, 4>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 6:
         return launch_dma<1, 2, 4, 2, 8, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 3:
         return launch_dma<2, 2, 2, 2, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+    case 7:
+        return launch_dma<1, 2, 4, 2, 8, 1, 3, 4>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 4:
-        return launch_dma<1, 1, 2, 2, 16, 7, 5>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+        return launch_dma<1, 1, 2, 2, 16, 7, 5, 4>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 5:
-        return launch_dma<1, 1, 4, 2, 16, 7, 5>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+        return launch_dma<1, 1, 4, 2, 16, 7, 5, 4>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     default:
         return REPDL_E_UNSUPPORTED;
     }
