@@ -293,7 +293,7 @@ def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=10)  # 77 ms of headline launches: the first tens of ms after idle are not steady state
     ap.add_argument("--quick", action="store_true", help="headline only, no secondary operators, no full parity")
     ap.add_argument("--only", default="", help="comma list of secondary legs to run (mm1024,mm_fma,sum2d,sum2d_dim0,sum4d,sum1d,"
                                                "exp,log,sqrt,div,loss,conv,linear,adam,cnn)")

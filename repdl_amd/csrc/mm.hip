@@ -6,13 +6,12 @@
 // operands are staged are free; the order along K is not, so K is never split
 // across threads.
 //
-// Three families of kernels implement it.  The matrix-instruction kernels feed
-// v_mfma_f32_16x16x4_f32 (mm_dma_kernel: operand rows on 16-byte boundaries, moved from global
-// memory straight into LDS) or v_mfma_f32_32x32x2_f32 (mm_mfma_fast_kernel, mm_mfma_kernel: every
-// other operand, staged through registers), which on gfx950 evaluate exactly such a chain (four or two k per
-// instruction, ascending; checked on the device before first use, see mfma_check.hip).
-// mm_kernel is the same computation with one v_fma_f32 per term; it runs when that check
-// fails or the matrix path is switched off.
+// Two families of kernels implement it.  mm_dma_kernel feeds v_mfma_f32_16x16x4_f32 from operand
+// tiles moved from global memory straight into LDS; on gfx950 the instruction evaluates exactly such
+// a chain (four k per instruction, ascending; checked on the device before first use, see
+// mfma_check.hip).  mm_kernel is the same computation with one v_fma_f32 per term; it runs when
+// that check fails, when the matrix path is switched off, or when an operand tile spans more than
+// 32 bits of byte offsets.
 //
 // mm_kernel layout: a workgroup of 256 threads computes a 128x128 tile of C; each thread
 // an 8x8 micro-tile held in registers (rows ty*4+{0..3} and 64+ty*4+{0..3},
@@ -243,566 +242,6 @@ __global__ __launch_bounds__(NT) void mm_kernel(const float *__restrict__ A,
     }
 }
 
-// ---------------------------------------------------------------------------
-// Matrix-core kernel.  A workgroup of WGM x WGN waves computes a (32 FM WGM) x
-// (32 FN WGN) tile of C; each wave FM x FN blocks of 32x32, one
-// v_mfma_f32_32x32x2_f32 per block and pair of k.  The instruction takes from lane l
-// the A element of row l%32 and the B element of column l%32, both at k = l/32, and
-// adds the k = 0 product to the accumulator first.  Operand tiles sit in LDS k-major
-// exactly as in mm_kernel, so an operand register is one ds_read_b32: lanes 0..31
-// read 32 consecutive rows at k, lanes 32..63 the same rows at k+1.
-//
-// K tail: positions k >= K are filled with -0.0f in the A tile and +0.0f in the B
-// tile.  Their product is -0, and x + (-0) = x for every x (both zeros, infinities
-// and NaN included), so a padded step leaves every accumulator bit for bit
-// unchanged.
-// ---------------------------------------------------------------------------
-typedef float f16v __attribute__((ext_vector_type(16)));
-
-template <int R, int NTH>
-struct TileFrag
-{
-    float4 v[R * BK / 4 / NTH];
-};
-
-// Same two memory layouts as load_tile above, for an R x BK tile and NTH threads; k >= K
-// (and rows beyond Rlim, whose products are never stored) read as `pad`.
-template <bool KC, int R, int NTH>
-__device__ __forceinline__ void load_tile_pad(const float *__restrict__ X, int64_t ld, int64_t Rlim, int64_t K,
-                                              int64_t r0, int64_t k0, bool vec_ok, int tid, float pad,
-                                              TileFrag<R, NTH> &f)
-{
-    constexpr int NV = R * BK / 4 / NTH;
-#pragma unroll
-    for (int i = 0; i < NV; i++)
-    {
-        const int idx = tid + NTH * i;
-        float4 v = make_float4(pad, pad, pad, pad);
-        if (KC)
-        {
-            const int64_t r = r0 + (idx >> 2), k = k0 + ((idx & 3) << 2);
-            if (r < Rlim)
-            {
-                const float *p = X + r * ld + k;
-                if (vec_ok && k + 3 < K)
-                    v = *reinterpret_cast<const float4 *>(p);
-                else
-                {
-                    if (k + 0 < K) v.x = p[0];
-                    if (k + 1 < K) v.y = p[1];
-                    if (k + 2 < K) v.z = p[2];
-                    if (k + 3 < K) v.w = p[3];
-                }
-            }
-        }
-        else
-        {
-            const int64_t k = k0 + idx / (R / 4), r = r0 + (idx % (R / 4)) * 4;
-            if (k < K)
-            {
-                const float *p = X + k * ld + r;
-                if (vec_ok && r + 3 < Rlim)
-                    v = *reinterpret_cast<const float4 *>(p);
-                else
-                {
-                    if (r + 0 < Rlim) v.x = p[0];
-                    if (r + 1 < Rlim) v.y = p[1];
-                    if (r + 2 < Rlim) v.z = p[2];
-                    if (r + 3 < Rlim) v.w = p[3];
-                }
-            }
-        }
-        f.v[i] = v;
-    }
-}
-
-template <bool KC, int R, int NTH>
-__device__ __forceinline__ void store_tile_pad(float *__restrict__ S, int tid, const TileFrag<R, NTH> &f)
-{
-    constexpr int NV = R * BK / 4 / NTH, LD = R + 4;
-#pragma unroll
-    for (int i = 0; i < NV; i++)
-    {
-        const int idx = tid + NTH * i;
-        if (KC)
-        {
-            const int r = idx >> 2, k = (idx & 3) << 2;
-            S[(k + 0) * LD + r] = f.v[i].x;
-            S[(k + 1) * LD + r] = f.v[i].y;
-            S[(k + 2) * LD + r] = f.v[i].z;
-            S[(k + 3) * LD + r] = f.v[i].w;
-        }
-        else
-        {
-            const int k = idx / (R / 4), r = (idx % (R / 4)) * 4;
-            *reinterpret_cast<float4 *>(&S[k * LD + r]) = f.v[i];
-        }
-    }
-}
-
-template <bool TA, bool TB, int FM, int FN, int WGM, int WGN>
-__global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_kernel(const float *__restrict__ A, const float *__restrict__ B,
-                                                                float *__restrict__ C, const float *__restrict__ bias,
-                                                                int64_t M, int64_t N, int64_t K, int avec, int bvec,
-                                                                int64_t gx, int64_t gy, int64_t ntiles8)
-{
-    constexpr int NTH = 64 * WGM * WGN;
-    constexpr int TM = 32 * FM * WGM, TN = 32 * FN * WGN;
-    constexpr int LDA_ = TM + 4, LDB_ = TN + 4;
-    constexpr bool A_KC = !TA, B_KC = TB;
-    extern __shared__ __attribute__((aligned(16))) float smem[];
-    float *const As = smem;                 // [2][BK * LDA_]
-    float *const Bs = smem + 2 * BK * LDA_; // [2][BK * LDB_]
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave % WGM, wn = wave / WGM;
-    const int l32 = lane & 31, half = lane >> 5;
-
-    // tile order: see mm_kernel
-    int64_t tile = blockIdx.x;
-    if (tile < ntiles8)
-        tile = (tile & 7) * (ntiles8 >> 3) + (tile >> 3);
-    const int64_t group_sz = (int64_t)GROUP_M * gx;
-    const int64_t group = tile / group_sz;
-    const int64_t first_row = group * GROUP_M;
-    const int64_t rows_here = (gy - first_row < GROUP_M) ? gy - first_row : GROUP_M;
-    const int64_t in_group = tile - group * group_sz;
-    const int64_t trow = first_row + in_group % rows_here, tcol = in_group / rows_here;
-    const int64_t m0 = trow * TM, n0 = tcol * TN;
-    const int64_t lda = TA ? M : K, ldb = TB ? K : N;
-
-    f16v acc[FM][FN];
-#pragma unroll
-    for (int i = 0; i < FM; i++)
-#pragma unroll
-        for (int j = 0; j < FN; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++)
-                acc[i][j][r] = 0.0f;
-
-    const int a_off = half * LDA_ + wm * 32 * FM + l32;
-    const int b_off = half * LDB_ + wn * 32 * FN + l32;
-    const int64_t nkt = (K + BK - 1) / BK;
-    TileFrag<TM, NTH> fa;
-    TileFrag<TN, NTH> fb;
-    if (nkt > 0)
-    {
-        load_tile_pad<A_KC, TM, NTH>(A, lda, M, K, m0, 0, avec, tid, -0.0f, fa);
-        load_tile_pad<B_KC, TN, NTH>(B, ldb, N, K, n0, 0, bvec, tid, 0.0f, fb);
-        store_tile_pad<A_KC, TM, NTH>(As, tid, fa);
-        store_tile_pad<B_KC, TN, NTH>(Bs, tid, fb);
-    }
-    __syncthreads();
-
-    for (int64_t kt = 0; kt < nkt; kt++)
-    {
-        const int cur = (int)(kt & 1);
-        const bool more = kt + 1 < nkt;
-        if (more)
-        {
-            load_tile_pad<A_KC, TM, NTH>(A, lda, M, K, m0, (kt + 1) * BK, avec, tid, -0.0f, fa);
-            load_tile_pad<B_KC, TN, NTH>(B, ldb, N, K, n0, (kt + 1) * BK, bvec, tid, 0.0f, fb);
-        }
-        // Every k-tile runs all BK / 2 instructions per block (the tail of K is padded, see
-        // above): one code path keeps the accumulators in place.  All operand registers of
-        // the tile are read before the first instruction is issued.
-        const float *as = As + cur * BK * LDA_ + a_off, *bs = Bs + cur * BK * LDB_ + b_off;
-        float a[BK / 2][FM], b[BK / 2][FN];
-#pragma unroll
-        for (int kp = 0; kp < BK / 2; kp++)
-        {
-#pragma unroll
-            for (int i = 0; i < FM; i++)
-                a[kp][i] = as[2 * kp * LDA_ + 32 * i];
-#pragma unroll
-            for (int j = 0; j < FN; j++)
-                b[kp][j] = bs[2 * kp * LDB_ + 32 * j];
-        }
-#pragma unroll
-        for (int kp = 0; kp < BK / 2; kp++)
-#pragma unroll
-            for (int i = 0; i < FM; i++)
-#pragma unroll
-                for (int j = 0; j < FN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kp][i], b[kp][j], acc[i][j], 0, 0, 0);
-        if (more)
-        {
-            store_tile_pad<A_KC, TM, NTH>(As + (cur ^ 1) * BK * LDA_, tid, fa);
-            store_tile_pad<B_KC, TN, NTH>(Bs + (cur ^ 1) * BK * LDB_, tid, fb);
-        }
-        __syncthreads();
-    }
-
-    // register r of a block is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
-#pragma unroll
-    for (int i = 0; i < FM; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++)
-        {
-            const int64_t m = m0 + wm * 32 * FM + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3);
-            if (m >= M)
-                continue;
-#pragma unroll
-            for (int j = 0; j < FN; j++)
-            {
-                const int64_t n = n0 + wn * 32 * FN + 32 * j + l32;
-                if (n < N)
-                    C[m * N + n] = bias != nullptr ? acc[i][j][r] + bias[n] : acc[i][j][r];
-            }
-        }
-}
-
-// The same kernel for the common case that needs no bounds checks: M, N multiples of the
-// tile, K a multiple of BK, 16-byte aligned operands.  While a matrix instruction runs, its
-// SIMD issues no vector ALU instruction of any wave (measured), so address arithmetic in the
-// loop costs matrix time one for one.  Here the loop has none: a global load is a uniform
-// base (advanced per k-tile on the scalar unit) plus a per-thread byte offset that never
-// changes; LDS addresses are per-thread constants plus the buffer offset plus immediates.
-template <bool TA, bool TB, int FM, int FN, int WGM, int WGN, bool EDGE>
-__global__ __launch_bounds__(64 * WGM *WGN) void mm_mfma_fast_kernel(const float *__restrict__ A,
-                                                                     const float *__restrict__ B,
-                                                                     float *__restrict__ C,
-                                                                     const float *__restrict__ bias, int64_t M,
-                                                                     int64_t N, int64_t K, int64_t gx, int64_t gy,
-                                                                     int64_t ntiles8)
-{
-    constexpr int NTH = 64 * WGM * WGN;
-    constexpr int TM = 32 * FM * WGM, TN = 32 * FN * WGN;
-    constexpr bool A_KC = !TA, B_KC = TB;
-    constexpr int LDA_ = TM + 4, LDB_ = TN + 4;
-    // Tiles of one wave per SIMD (64x64, 128x128) run the software-pipelined loop below: a lone
-    // wave has nobody to cover its LDS latency after a barrier (1024^3: 31 -> 25-29 us, 1536^2 x
-    // 4096: +7 %).  With two waves per SIMD (256x256) the plain loop is the faster one by 3-4 %.
-    constexpr bool PIPE = FM * FN <= 4;
-    constexpr int PIPE_STORE_AT = 4; // k-pair after which the next k-tile goes to LDS
-    constexpr int NVA = TM * BK / 4 / NTH, NVB = TN * BK / 4 / NTH;
-    typedef float v4f __attribute__((ext_vector_type(4)));
-    extern __shared__ __attribute__((aligned(16))) float smem[];
-    float *const As = smem;                 // [2][BK * LDA_]
-    float *const Bs = smem + 2 * BK * LDA_; // [2][BK * LDB_]
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave % WGM, wn = wave / WGM;
-    const int l32 = lane & 31, half = lane >> 5;
-
-    int64_t tile = blockIdx.x;
-    if (tile < ntiles8)
-        tile = (tile & 7) * (ntiles8 >> 3) + (tile >> 3);
-    const int64_t group_sz = (int64_t)GROUP_M * gx;
-    const int64_t group = tile / group_sz;
-    const int64_t first_row = group * GROUP_M;
-    const int64_t rows_here = (gy - first_row < GROUP_M) ? gy - first_row : GROUP_M;
-    const int64_t in_group = tile - group * group_sz;
-    const int64_t trow = first_row + in_group % rows_here, tcol = in_group / rows_here;
-    const int64_t m0 = trow * TM, n0 = tcol * TN;
-    const int64_t lda = TA ? M : K, ldb = TB ? K : N;
-
-    // per-thread constants: byte offset of each float4 slot inside the operand tile, and the
-    // LDS word it goes to
-    uint32_t a_voff[NVA], b_voff[NVB];
-    int a_st[NVA], b_st[NVB];
-#pragma unroll
-    for (int i = 0; i < NVA; i++)
-    {
-        const int idx = tid + NTH * i;
-        if (A_KC)
-        {
-            const int r = idx >> 2, k = (idx & 3) << 2;
-            a_voff[i] = (uint32_t)((int64_t)r * lda + k) * 4u;
-            a_st[i] = k * LDA_ + r;
-        }
-        else
-        {
-            const int k = idx / (TM / 4), r = (idx % (TM / 4)) * 4;
-            a_voff[i] = (uint32_t)((int64_t)k * lda + r) * 4u;
-            a_st[i] = k * LDA_ + r;
-        }
-    }
-#pragma unroll
-    for (int i = 0; i < NVB; i++)
-    {
-        const int idx = tid + NTH * i;
-        if (B_KC)
-        {
-            const int r = idx >> 2, k = (idx & 3) << 2;
-            b_voff[i] = (uint32_t)((int64_t)r * ldb + k) * 4u;
-            b_st[i] = k * LDB_ + r;
-        }
-        else
-        {
-            const int k = idx / (TN / 4), r = (idx % (TN / 4)) * 4;
-            b_voff[i] = (uint32_t)((int64_t)k * ldb + r) * 4u;
-            b_st[i] = k * LDB_ + r;
-        }
-    }
-    // uniform tile bases, advanced by one k-tile per iteration
-    const char *a_base = reinterpret_cast<const char *>(A_KC ? A + m0 * lda : A + m0);
-    const char *b_base = reinterpret_cast<const char *>(B_KC ? B + n0 * ldb : B + n0);
-    const int64_t a_step = (A_KC ? (int64_t)BK : (int64_t)BK * lda) * 4;
-    const int64_t b_step = (B_KC ? (int64_t)BK : (int64_t)BK * ldb) * 4;
-
-    f16v acc[FM][FN];
-#pragma unroll
-    for (int i = 0; i < FM; i++)
-#pragma unroll
-        for (int j = 0; j < FN; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++)
-                acc[i][j][r] = 0.0f;
-
-    v4f fa[NVA], fb[NVB];
-    auto load_tiles = [&]() {
-#pragma unroll
-        for (int i = 0; i < NVA; i++)
-            fa[i] = *reinterpret_cast<const v4f *>(a_base + a_voff[i]);
-#pragma unroll
-        for (int i = 0; i < NVB; i++)
-            fb[i] = *reinterpret_cast<const v4f *>(b_base + b_voff[i]);
-        a_base += a_step;
-        b_base += b_step;
-    };
-    // EDGE variant: any M, N, K with 16-byte aligned operands.  A workgroup whose tile lies wholly
-    // inside C loads whole k-tiles as above; tiles on the lower or right edge, and the last
-    // partial k-tile of every workgroup, take predicated loads (rows past the edge are never
-    // stored; k positions past K hold -0.0f in the A tile and +0.0f in the B tile, a bit-exact
-    // no-op, see mm_mfma_kernel).
-    const bool interior = !EDGE || (m0 + TM <= M && n0 + TN <= N);
-    auto load_tiles_guarded = [&](int64_t kt) {
-        if constexpr (EDGE)
-        {
-#pragma unroll
-            for (int i = 0; i < NVA; i++)
-            {
-                const int idx = tid + NTH * i;
-                const int64_t r = m0 + (A_KC ? (idx >> 2) : (idx % (TM / 4)) * 4);
-                const int64_t k = kt * BK + (A_KC ? ((idx & 3) << 2) : idx / (TM / 4));
-                v4f v = {-0.0f, -0.0f, -0.0f, -0.0f};
-                if (A_KC)
-                {
-                    if (r < M)
-                    {
-                        const float *p = A + r * lda + k;
-                        if (k + 3 < K)
-                            v = *reinterpret_cast<const v4f *>(p);
-                        else
-                        {
-                            if (k + 0 < K) v[0] = p[0];
-                            if (k + 1 < K) v[1] = p[1];
-                            if (k + 2 < K) v[2] = p[2];
-                            if (k + 3 < K) v[3] = p[3];
-                        }
-                    }
-                }
-                else if (k < K)
-                {
-                    const float *p = A + k * lda + r;
-                    if (r + 3 < M)
-                        v = *reinterpret_cast<const v4f *>(p);
-                    else
-                    {
-                        if (r + 0 < M) v[0] = p[0];
-                        if (r + 1 < M) v[1] = p[1];
-                        if (r + 2 < M) v[2] = p[2];
-                        if (r + 3 < M) v[3] = p[3];
-                    }
-                }
-                fa[i] = v;
-            }
-#pragma unroll
-            for (int i = 0; i < NVB; i++)
-            {
-                const int idx = tid + NTH * i;
-                const int64_t r = n0 + (B_KC ? (idx >> 2) : (idx % (TN / 4)) * 4);
-                const int64_t k = kt * BK + (B_KC ? ((idx & 3) << 2) : idx / (TN / 4));
-                v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
-                if (B_KC)
-                {
-                    if (r < N)
-                    {
-                        const float *p = B + r * ldb + k;
-                        if (k + 3 < K)
-                            v = *reinterpret_cast<const v4f *>(p);
-                        else
-                        {
-                            if (k + 0 < K) v[0] = p[0];
-                            if (k + 1 < K) v[1] = p[1];
-                            if (k + 2 < K) v[2] = p[2];
-                            if (k + 3 < K) v[3] = p[3];
-                        }
-                    }
-                }
-                else if (k < K)
-                {
-                    const float *p = B + k * ldb + r;
-                    if (r + 3 < N)
-                        v = *reinterpret_cast<const v4f *>(p);
-                    else
-                    {
-                        if (r + 0 < N) v[0] = p[0];
-                        if (r + 1 < N) v[1] = p[1];
-                        if (r + 2 < N) v[2] = p[2];
-                        if (r + 3 < N) v[3] = p[3];
-                    }
-                }
-                fb[i] = v;
-            }
-        }
-    };
-    // k-tile kt: whole and inside -> the cheap loads (which also step the bases), else predicated
-    const int64_t nkt_whole = K / BK;
-    auto load_any = [&](int64_t kt) {
-        if (!EDGE || (interior && kt < nkt_whole))
-            load_tiles();
-        else
-            load_tiles_guarded(kt);
-    };
-    auto store_tiles = [&](int buf) {
-        float *as = As + buf * BK * LDA_, *bs = Bs + buf * BK * LDB_;
-#pragma unroll
-        for (int i = 0; i < NVA; i++)
-        {
-            if (A_KC)
-            {
-                as[a_st[i] + 0 * LDA_] = fa[i][0];
-                as[a_st[i] + 1 * LDA_] = fa[i][1];
-                as[a_st[i] + 2 * LDA_] = fa[i][2];
-                as[a_st[i] + 3 * LDA_] = fa[i][3];
-            }
-            else
-                *reinterpret_cast<v4f *>(&as[a_st[i]]) = fa[i];
-        }
-#pragma unroll
-        for (int i = 0; i < NVB; i++)
-        {
-            if (B_KC)
-            {
-                bs[b_st[i] + 0 * LDB_] = fb[i][0];
-                bs[b_st[i] + 1 * LDB_] = fb[i][1];
-                bs[b_st[i] + 2 * LDB_] = fb[i][2];
-                bs[b_st[i] + 3 * LDB_] = fb[i][3];
-            }
-            else
-                *reinterpret_cast<v4f *>(&bs[b_st[i]]) = fb[i];
-        }
-    };
-    const int a_off = half * LDA_ + wm * 32 * FM + l32;
-    const int b_off = half * LDB_ + wn * 32 * FN + l32;
-    auto compute = [&](int buf) {
-        const float *as = As + buf * BK * LDA_ + a_off, *bs = Bs + buf * BK * LDB_ + b_off;
-        float a[BK / 2][FM], b[BK / 2][FN];
-#pragma unroll
-        for (int kp = 0; kp < BK / 2; kp++)
-        {
-#pragma unroll
-            for (int i = 0; i < FM; i++)
-                a[kp][i] = as[2 * kp * LDA_ + 32 * i];
-#pragma unroll
-            for (int j = 0; j < FN; j++)
-                b[kp][j] = bs[2 * kp * LDB_ + 32 * j];
-        }
-#pragma unroll
-        for (int kp = 0; kp < BK / 2; kp++)
-#pragma unroll
-            for (int i = 0; i < FM; i++)
-#pragma unroll
-                for (int j = 0; j < FN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kp][i], b[kp][j], acc[i][j], 0, 0, 0);
-    };
-
-    const int64_t nkt = EDGE ? (K + BK - 1) / BK : K / BK;
-    if (nkt > 0)
-    {
-        load_any(0);
-        store_tiles(0);
-    }
-    __syncthreads();
-    if constexpr (PIPE)
-    {
-        // Software pipeline over the k-pairs of a k-tile: the operands of pair kp + 1 are read
-        // while the matrix instructions of pair kp run, the next k-tile is stored to the other
-        // LDS buffer mid-way, and the barrier sits before the last pair, whose instructions cover
-        // the first operand reads of the next k-tile.  One barrier per k-tile is enough: every read
-        // of a buffer is issued before the barrier that precedes the next stores into it.
-        float pa[2][FM], pb[2][FN];
-        auto read_ops = [&](int buf, int kp, float(&a)[FM], float(&b)[FN]) {
-            const float *as = As + buf * BK * LDA_ + a_off, *bs = Bs + buf * BK * LDB_ + b_off;
-#pragma unroll
-            for (int i = 0; i < FM; i++)
-                a[i] = as[2 * kp * LDA_ + 32 * i];
-#pragma unroll
-            for (int j = 0; j < FN; j++)
-                b[j] = bs[2 * kp * LDB_ + 32 * j];
-        };
-        if (nkt > 0)
-            read_ops(0, 0, pa[0], pb[0]);
-        for (int64_t kt = 0; kt < nkt; kt++)
-        {
-            const int cur = (int)(kt & 1);
-            const bool more = kt + 1 < nkt;
-            if (more)
-                load_any(kt + 1);
-#pragma unroll
-            for (int kp = 0; kp < BK / 2; kp++)
-            {
-                if (kp + 1 < BK / 2)
-                    read_ops(cur, kp + 1, pa[(kp + 1) & 1], pb[(kp + 1) & 1]);
-                else if (more)
-                    read_ops(cur ^ 1, 0, pa[0], pb[0]);
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int i = 0; i < FM; i++)
-#pragma unroll
-                    for (int j = 0; j < FN; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[kp & 1][i], pb[kp & 1][j], acc[i][j], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-                if (kp == PIPE_STORE_AT && more)
-                    store_tiles(cur ^ 1);
-                if (kp == BK / 2 - 2)
-                    __syncthreads();
-            }
-        }
-    }
-    else
-    for (int64_t kt = 0; kt < nkt; kt++)
-    {
-        const int cur = (int)(kt & 1);
-        const bool more = kt + 1 < nkt;
-        if (more)
-            load_any(kt + 1);
-        compute(cur);
-        if (more)
-            store_tiles(cur ^ 1);
-        __syncthreads();
-    }
-
-    // bias: one rounded add per output after its chain; a lane owns FN columns
-    float bv[FN];
-#pragma unroll
-    for (int j = 0; j < FN; j++)
-    {
-        const int64_t nn = n0 + wn * 32 * FN + 32 * j + l32;
-        bv[j] = bias != nullptr && (!EDGE || nn < N) ? bias[nn] : 0.0f;
-    }
-#pragma unroll
-    for (int i = 0; i < FM; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++)
-        {
-            const int64_t m = m0 + wm * 32 * FM + 32 * i + 8 * (r >> 2) + 4 * half + (r & 3);
-            if (EDGE && m >= M)
-                continue;
-#pragma unroll
-            for (int j = 0; j < FN; j++)
-            {
-                const int64_t nn = n0 + wn * 32 * FN + 32 * j + l32;
-                if (!EDGE || nn < N)
-                    __builtin_nontemporal_store(bias != nullptr ? acc[i][j][r] + bv[j] : acc[i][j][r], &C[m * N + nn]);
-            }
-        }
-}
-
 // ---------------------------------------------------------------------------------------------
 // mm_dma_kernel: operands whose rows start on 16-byte boundaries, any M, N, K; a batch of products.
 //
@@ -850,12 +289,18 @@ __device__ __forceinline__ void dma16(const void *base, uint32_t voff, uint32_t 
                  : "memory", "m0");
 }
 
+__device__ __forceinline__ void dma4(const void *base, uint32_t voff, uint32_t lds_byte)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(voff), "s"(base), "s"(lds_byte)
+                 : "memory", "m0");
+}
+
 struct MmBatch
 {
     int64_t a, b, c; // elements between consecutive products' operands and results
 };
 
-template <bool TA, bool TB, int FM, int FN, int WGM, int WGN, int NQ, int D, int NB, int DW>
+template <bool TA, bool TB, int FM, int FN, int WGM, int WGN, int NQ, int D, int NB, int DW, int VEC>
 __global__ __launch_bounds__(64 * (WGM * WGN + DW)) void mm_dma_kernel(const float *__restrict__ A, const float *__restrict__ B,
                                                                float *__restrict__ C, const float *__restrict__ cbias,
                                                                const float *__restrict__ rbias, int64_t M, int64_t N,
@@ -869,8 +314,10 @@ __global__ __launch_bounds__(64 * (WGM * WGN + DW)) void mm_dma_kernel(const flo
     constexpr int R = D + 1;                      // register sets in the ring
     static_assert(NQ % R == 0 && D >= 1 && D < NQ, "ring must divide the k-tile");
     static_assert(NB >= 3, "a buffer being read, one landed or landing, one being filled");
+    static_assert(VEC == 4 || VEC == 1, "16-byte or 4-byte DMA lanes");
     static_assert((TM * NQ) % 64 == 0 && (TN * NQ) % 64 == 0, "a DMA instruction fills 64 slots");
-    constexpr int NIA = TM * NQ / 64, NIB = TN * NQ / 64; // DMA instructions per k-tile
+    constexpr int SPW = 4 / VEC;                                      // slots per 16 bytes of the LDS image
+    constexpr int NIA = TM * NQ * SPW / 64, NIB = TN * NQ * SPW / 64; // DMA instructions per k-tile
     constexpr int NI = DW > 0 ? DW : NW;                  // waves that issue them: DW waves that do nothing else, or all
     constexpr int CA = (NIA + NI - 1) / NI, CB = (NIB + NI - 1) / NI;
     static_assert(NB == 3 || (NIA % NI == 0 && NIB % NI == 0), "every wave must issue the same number of loads per tile");
@@ -903,8 +350,10 @@ __global__ __launch_bounds__(64 * (WGM * WGN + DW)) void mm_dma_kernel(const flo
     B += (int64_t)blockIdx.y * batch.b;
     C += (int64_t)blockIdx.y * batch.c;
 
-    // DMA instruction e of an operand with T rows: 64 consecutive 16-byte slots of the tile's LDS
-    // image, i.e. slots [64e, 64e+64) of NQ*T; slot s = quad (s / T), position w = s % T in the quad.
+    // DMA instruction e of an operand with T rows: 64 consecutive slots (16 bytes, or 4 when rows do not
+    // start on 16-byte boundaries) of the tile's LDS image.  In 16-byte slots: slot s = quad (s / T),
+    // position w = s % T in the quad -- a row's four k where k is contiguous, else four consecutive rows
+    // at k = w % 4.  A 4-byte slot x is word x % 4 of the 16-byte slot x / 4.
     // Rows past the operand's last are clamped to rows it has.
     uint32_t va[CA], vb[CB];
     uint32_t la[CA], lb[CB];
@@ -912,34 +361,44 @@ __global__ __launch_bounds__(64 * (WGM * WGN + DW)) void mm_dma_kernel(const flo
 #pragma unroll
     for (int t = 0; t < CA; t++)
     {
-        const int e = wi + NI * t, s = 64 * e + lane, q = s / TM, w = s % TM;
+        const int e = wi + NI * t, x = 64 * e + lane, s = x / SPW, sub = x % SPW, q = s / TM, w = s % TM;
         if (A_KC)
         {
             const int64_t r = w < am ? w : am - 1;
-            va[t] = (uint32_t)((r * lda + 4 * q) * 4);
+            va[t] = (uint32_t)((r * lda + 4 * q + sub) * 4);
         }
-        else
+        else if (VEC == 4)
         {
             const int64_t r = (w & ~3) + 3 < am ? (w & ~3) : am - 4;
             va[t] = (uint32_t)(((int64_t)(4 * q + (w & 3)) * lda + r) * 4);
         }
-        la[t] = __builtin_amdgcn_readfirstlane(lds0 + 64 * e * 16);
+        else
+        {
+            const int64_t r = (w & ~3) + sub < am ? (w & ~3) + sub : am - 1;
+            va[t] = (uint32_t)(((int64_t)(4 * q + (w & 3)) * lda + r) * 4);
+        }
+        la[t] = __builtin_amdgcn_readfirstlane(lds0 + 64 * e * 4 * VEC);
     }
 #pragma unroll
     for (int t = 0; t < CB; t++)
     {
-        const int e = wi + NI * t, s = 64 * e + lane, q = s / TN, w = s % TN;
+        const int e = wi + NI * t, x = 64 * e + lane, s = x / SPW, sub = x % SPW, q = s / TN, w = s % TN;
         if (B_KC)
         {
             const int64_t r = w < bn ? w : bn - 1;
-            vb[t] = (uint32_t)((r * ldb + 4 * q) * 4);
+            vb[t] = (uint32_t)((r * ldb + 4 * q + sub) * 4);
         }
-        else
+        else if (VEC == 4)
         {
             const int64_t r = (w & ~3) + 3 < bn ? (w & ~3) : bn - 4;
             vb[t] = (uint32_t)(((int64_t)(4 * q + (w & 3)) * ldb + r) * 4);
         }
-        lb[t] = __builtin_amdgcn_readfirstlane(lds0 + NB * OPA * 4 + 64 * e * 16);
+        else
+        {
+            const int64_t r = (w & ~3) + sub < bn ? (w & ~3) + sub : bn - 1;
+            vb[t] = (uint32_t)(((int64_t)(4 * q + (w & 3)) * ldb + r) * 4);
+        }
+        lb[t] = __builtin_amdgcn_readfirstlane(lds0 + NB * OPA * 4 + 64 * e * 4 * VEC);
     }
     const char *a_base = reinterpret_cast<const char *>(A_KC ? A + m0 * lda : A + m0);
     const char *b_base = reinterpret_cast<const char *>(B_KC ? B + n0 * ldb : B + n0);
@@ -950,24 +409,30 @@ __global__ __launch_bounds__(64 * (WGM * WGN + DW)) void mm_dma_kernel(const flo
     const int64_t nkt = K / (4 * NQ);
     const int tq = (int)((K / 4) % NQ);
     const int64_t ntile = nkt + (tq > 0 ? 1 : 0);
+    auto move = [&](const char *base, uint32_t voff, uint32_t lds_byte) {
+        if (VEC == 4)
+            dma16(base, voff, lds_byte);
+        else
+            dma4(base, voff, lds_byte);
+    };
     auto issue = [&](int buf, bool tail) {
 #pragma unroll
         for (int t = 0; t < CA; t++)
             if (NIA % NI == 0 || wi + NI * t < NIA)
             {
                 if (!tail)
-                    dma16(a_base, va[t], la[t] + buf * OPA * 4);
-                else if ((64 * (wi + NI * t) + lane) / TM < tq)
-                    dma16(a_base, va[t], la[t] + buf * OPA * 4);
+                    move(a_base, va[t], la[t] + buf * OPA * 4);
+                else if ((64 * (wi + NI * t) + lane) / (SPW * TM) < tq)
+                    move(a_base, va[t], la[t] + buf * OPA * 4);
             }
 #pragma unroll
         for (int t = 0; t < CB; t++)
             if (NIB % NI == 0 || wi + NI * t < NIB)
             {
                 if (!tail)
-                    dma16(b_base, vb[t], lb[t] + buf * OPB * 4);
-                else if ((64 * (wi + NI * t) + lane) / TN < tq)
-                    dma16(b_base, vb[t], lb[t] + buf * OPB * 4);
+                    move(b_base, vb[t], lb[t] + buf * OPB * 4);
+                else if ((64 * (wi + NI * t) + lane) / (SPW * TN) < tq)
+                    move(b_base, vb[t], lb[t] + buf * OPB * 4);
             }
         a_base += a_step;
         b_base += b_step;
@@ -1159,16 +624,16 @@ __global__ __launch_bounds__(64 * (WGM * WGN + DW)) void mm_dma_kernel(const flo
         }
 }
 
-// Whether mm_dma_kernel with this tile can take the product: operand rows on 16-byte boundaries,
-// at least four rows (columns) where rows are contiguous (the edge clamp steps back by four), lane
-// offsets inside an operand tile within 32 bits.
+// Whether mm_dma_kernel with this tile can take the product: lane offsets inside an operand tile
+// within 32 bits and, with 16-byte DMA lanes (vec4), at least four rows (columns) where rows are
+// contiguous (the edge clamp steps back by four).
 template <int FM, int FN, int WGM, int WGN, int NQ>
-bool dma_applies(int64_t M, int64_t N, int64_t K, int transA, int transB, int avec, int bvec, int64_t nbatch = 1)
+bool dma_applies(int64_t M, int64_t N, int64_t K, int transA, int transB, bool vec4, int64_t nbatch = 1)
 {
     constexpr int TM = 16 * FM * WGM, TN = 16 * FN * WGN, BKQ = 4 * NQ;
-    if (!avec || !bvec || M < 1 || N < 1 || K < 1 || nbatch < 1 || nbatch > 65535)
+    if (M < 1 || N < 1 || K < 1 || nbatch < 1 || nbatch > 65535)
         return false;
-    if ((transA && M < 4) || (!transB && N < 4))
+    if (vec4 && ((transA && M < 4) || (!transB && N < 4)))
         return false;
     const int64_t lda = transA ? M : K, ldb = transB ? K : N;
     const int64_t ea = transA ? (int64_t)BKQ * lda + TM : (int64_t)TM * lda + BKQ;
@@ -1176,7 +641,7 @@ bool dma_applies(int64_t M, int64_t N, int64_t K, int transA, int transB, int av
     return ea * 4 < (1LL << 32) && eb * 4 < (1LL << 32) && repdl_cdiv(M, TM) * repdl_cdiv(N, TN) <= REPDL_I32_MAX;
 }
 
-template <bool TA, bool TB, int FM, int FN, int WGM, int WGN, int NQ, int D, int NB, int DW = 0>
+template <bool TA, bool TB, int FM, int FN, int WGM, int WGN, int NQ, int D, int NB, int DW = 0, int VEC = 4>
 int launch_dma_t(const float *A, const float *B, float *C, const float *cbias, const float *rbias, int64_t M, int64_t N,
                  int64_t K, int64_t nbatch, MmBatch batch, hipStream_t s)
 {
@@ -1185,7 +650,7 @@ int launch_dma_t(const float *A, const float *B, float *C, const float *cbias, c
     static_assert(shmem <= 160 * 1024, "LDS of one CU");
     const int64_t gx = repdl_cdiv(N, TN), gy = repdl_cdiv(M, TM);
     const int64_t ntiles8 = (gx * gy) & ~(int64_t)7;
-    auto kern = &mm_dma_kernel<TA, TB, FM, FN, WGM, WGN, NQ, D, NB, DW>;
+    auto kern = &mm_dma_kernel<TA, TB, FM, FN, WGM, WGN, NQ, D, NB, DW, VEC>;
     if (shmem > 48 * 1024)
     {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1198,17 +663,17 @@ int launch_dma_t(const float *A, const float *B, float *C, const float *cbias, c
     return repdl_launch_status();
 }
 
-template <int FM, int FN, int WGM, int WGN, int NQ, int D, int NB, int DW = 0>
+template <int FM, int FN, int WGM, int WGN, int NQ, int D, int NB, int DW = 0, int VEC = 4>
 int launch_dma(const float *A, const float *B, float *C, const float *cbias, const float *rbias, int64_t M, int64_t N, int64_t K,
                int transA, int transB, int64_t nbatch, MmBatch batch, hipStream_t s)
 {
     if (!transA && !transB)
-        return launch_dma_t<false, false, FM, FN, WGM, WGN, NQ, D, NB, DW>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
+        return launch_dma_t<false, false, FM, FN, WGM, WGN, NQ, D, NB, DW, VEC>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
     if (transA && !transB)
-        return launch_dma_t<true, false, FM, FN, WGM, WGN, NQ, D, NB, DW>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
+        return launch_dma_t<true, false, FM, FN, WGM, WGN, NQ, D, NB, DW, VEC>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
     if (!transA && transB)
-        return launch_dma_t<false, true, FM, FN, WGM, WGN, NQ, D, NB, DW>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
-    return launch_dma_t<true, true, FM, FN, WGM, WGN, NQ, D, NB, DW>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
+        return launch_dma_t<false, true, FM, FN, WGM, WGN, NQ, D, NB, DW, VEC>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
+    return launch_dma_t<true, true, FM, FN, WGM, WGN, NQ, D, NB, DW, VEC>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
 }
 
 // The tile for a batch of products, and its launch; REPDL_E_UNSUPPORTED if mm_dma_kernel cannot
@@ -1217,8 +682,9 @@ int launch_dma(const float *A, const float *B, float *C, const float *cbias, con
 // three workgroups of the first two tiles at once).  "+4" = four more waves that only issue the DMA:
 // it pays while a CU holds one workgroup (a lone wave per SIMD issues a DMA instruction about every
 // 60 clocks, two matrix instructions' worth of its chain), and costs 10 % on 8192^3.
-//   128x128, 8 waves of 64x32, k-tile 16:  r = 1 0.88 (+4: 2048^3 119 -> 128 TFLOP/s), 2 0.94, 3 0.88, 4 0.95,
-//     5 0.83, 6 0.95, 7 0.89, more 0.97 (an odd count leaves a last round of one workgroup per CU);
+//   128x128, 8 waves of 64x32, k-tile 16:  r = 1 0.82 (0.88 with +4, 2048^3 119 -> 128 TFLOP/s: what four rounds
+//     of 64x64 tiles reach, which is what the cost picks there), 2 0.94, 3 0.88, 4 0.95, 5 0.83, 6 0.95, 7 0.89,
+//     more 0.97 (an odd count leaves a last round of one workgroup per CU);
 //   64x64: r = 1 0.73, 2 0.84, 3 0.875, 4..7 0.89, more 0.92, on
 //     r = 1, 2: 8 waves of 16x32, k-tile 32, four buffers, +4 (1024^2 x 2048: 106 TFLOP/s, against 95 without
 //            the four, 81-83 with four waves of 32x32 or with three buffers; 2048 x 1024 x 2048: 122); chains of
@@ -1232,6 +698,9 @@ int launch_dma(const float *A, const float *B, float *C, const float *cbias, con
 // (8192^3 NT: 145 / 138 TFLOP/s on the first two; 3072 x 4096 x 2048: 106-139 by layout / 132-136;
 // 4096 x 2048 x 2048: 136 / 132; 5120 x 4096 x 2048: 121 / 134; 1408^2 x 4096: 57 / 108.)  A tile that hangs
 // over an edge costs what a whole one does.
+// Operand rows off 16-byte boundaries: the same tiles with 4-byte DMA lanes, four times the DMA
+// instructions (8190^3 NT / NN / TN: 120 / 124 / 137 TFLOP/s, against 96 through registers); the
+// one-workgroup-per-CU forms then take eight moving waves.
 #ifdef REPDL_DEBUG_HOOKS
 int g_force_tile = 0; // 1..7: that configuration whatever the shape
 #endif
@@ -1239,31 +708,32 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
                     int64_t K, int transA, int transB, int avec, int bvec, int64_t nbatch, MmBatch batch, hipStream_t s)
 {
     auto rounds = [&](int64_t tm, int64_t tn) { return repdl_cdiv(repdl_cdiv(M, tm) * repdl_cdiv(N, tn) * nbatch, 256); };
+    const bool vec4 = avec && bvec; // else rows off 16-byte boundaries: 4-byte DMA lanes, four times the DMA instructions
     double best = 1e300;
     int pick = 0;
-    if (dma_applies<4, 2, 2, 4, 4>(M, N, K, transA, transB, avec, bvec, nbatch))
+    if (dma_applies<4, 2, 2, 4, 4>(M, N, K, transA, transB, vec4, nbatch))
     {
         const int64_t r = rounds(128, 128);
-        static const double e128[8] = {0.88, 0.94, 0.88, 0.95, 0.83, 0.95, 0.89, 0.97};
+        static const double e128[8] = {0.82, 0.94, 0.88, 0.95, 0.83, 0.95, 0.89, 0.97};
         const double c = (double)r * 16384.0 / e128[r < 8 ? r - 1 : 7];
         if (c < best)
             best = c, pick = 1;
     }
-    if (dma_applies<1, 2, 4, 2, 8>(M, N, K, transA, transB, avec, bvec, nbatch))
+    if (dma_applies<1, 2, 4, 2, 8>(M, N, K, transA, transB, vec4, nbatch))
     {
         const int64_t r = rounds(64, 64);
         const double c = (double)r * 4096.0 / (r >= 8 ? 0.92 : r >= 4 ? 0.89 : r == 3 ? 0.875 : r == 2 ? 0.84 : 0.73);
         if (c < best)
             best = c, pick = r >= 4 ? 3 : r == 3 ? 6 : K > 1024 ? 2 : r == 1 ? 7 : 6;
     }
-    if (dma_applies<1, 1, 2, 2, 16>(M, N, K, transA, transB, avec, bvec, nbatch))
+    if (dma_applies<1, 1, 2, 2, 16>(M, N, K, transA, transB, vec4, nbatch))
     {
         const int64_t r = rounds(32, 32);
         const double c = (double)r * 1024.0 / (r >= 2 ? 0.52 : 0.445);
         if (c < best)
             best = c, pick = 4;
     }
-    if (dma_applies<1, 1, 4, 2, 16>(M, N, K, transA, transB, avec, bvec, nbatch))
+    if (dma_applies<1, 1, 4, 2, 16>(M, N, K, transA, transB, vec4, nbatch))
     {
         const double c = (double)rounds(64, 32) * 2048.0 / 0.60;
         if (c < best)
@@ -1273,6 +743,27 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
     if (g_force_tile > 0)
         pick = g_force_tile;
 #endif
+    if (!vec4)
+        switch (pick)
+        {
+        case 1:
+            return launch_dma<4, 2, 2, 4, 4, 1, 3, 0, 1>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+        case 2:
+        case 6:
+        case 7:
+            // one 64x64 tile per CU: eight waves that only move (1001^2 x 2049: 54 TFLOP/s on the
+            // four-wave form, 87 with four movers, 96 with eight)
+            if (rounds(64, 64) == 1)
+                return launch_dma<1, 2, 4, 2, 8, 1, 4, 8, 1>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+            return launch_dma<1, 2, 4, 2, 8, 1, 3, 0, 1>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+        case 3:
+            return launch_dma<2, 2, 2, 2, 4, 1, 3, 0, 1>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+        case 4:
+        case 5:
+            return launch_dma<1, 1, 2, 2, 16, 7, 5, 8, 1>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+        default:
+            return REPDL_E_UNSUPPORTED;
+        }
     switch (pick)
     {
     case 1:
@@ -1283,8 +774,6 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
         // every other shape and layout the eight-wave form is the faster one by 4-6 %.
         if (transA && !transB && K >= 4 * (M > N ? M : N))
             return launch_dma_t<true, false, 4, 4, 2, 2, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
-        if (rounds(128, 128) == 1)
-            return launch_dma<4, 2, 2, 4, 4, 1, 3, 4>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
         return launch_dma<4, 2, 2, 4, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 2:
         return launch_dma<1, 2, 4, 2, 8, 1, 4, 4>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
@@ -1301,64 +790,6 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
     default:
         return REPDL_E_UNSUPPORTED;
     }
-}
-
-template <bool TA, bool TB, int FM, int FN, int WGM, int WGN>
-int launch_mfma_t(const float *A, const float *B, float *C, const float *bias, int64_t M, int64_t N, int64_t K, int avec,
-                  int bvec, hipStream_t s)
-{
-    constexpr int TM = 32 * FM * WGM, TN = 32 * FN * WGN;
-    constexpr size_t shmem = (size_t)2 * BK * (TM + 4 + TN + 4) * sizeof(float);
-    const int64_t gx = repdl_cdiv(N, TN), gy = repdl_cdiv(M, TM);
-    if (gx * gy > REPDL_I32_MAX)
-        return REPDL_E_ARG;
-    const int64_t ntiles8 = (gx * gy) & ~(int64_t)7;
-    const int64_t lda = TA ? M : K, ldb = TB ? K : N;
-    // aligned operands whose in-tile byte offsets fit 32 bits: the kernel without address arithmetic
-    // in the loop -- its plain form for whole-tile shapes, its EDGE form (edge tiles and the K tail
-    // predicated) for the rest
-    const bool aligned = avec && bvec && (int64_t)(TM + BK) * lda * 4 < (1LL << 32) &&
-                         (int64_t)(TN + BK) * ldb * 4 < (1LL << 32);
-    const bool whole = M % TM == 0 && N % TN == 0 && K % BK == 0;
-    if (aligned)
-    {
-        auto kern = whole ? &mm_mfma_fast_kernel<TA, TB, FM, FN, WGM, WGN, false>
-                          : &mm_mfma_fast_kernel<TA, TB, FM, FN, WGM, WGN, true>;
-        if (shmem > 48 * 1024)
-        {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-            if (e != hipSuccess)
-                return (int)e;
-        }
-        hipLaunchKernelGGL(kern, dim3((unsigned)(gx * gy)), dim3(64 * WGM * WGN), shmem, s, A, B, C, bias, M, N, K, gx, gy,
-                           ntiles8);
-        return repdl_launch_status();
-    }
-    auto kern = &mm_mfma_kernel<TA, TB, FM, FN, WGM, WGN>;
-    if (shmem > 48 * 1024)
-    {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)shmem);
-        if (e != hipSuccess)
-            return (int)e;
-    }
-    hipLaunchKernelGGL(kern, dim3((unsigned)(gx * gy)), dim3(64 * WGM * WGN), shmem, s, A, B, C, bias, M, N, K, avec, bvec,
-                       gx, gy, ntiles8);
-    return repdl_launch_status();
-}
-
-template <int FM, int FN, int WGM, int WGN>
-int launch_mfma(const float *A, const float *B, float *C, const float *bias, int64_t M, int64_t N, int64_t K, int transA,
-                int transB, int avec, int bvec, hipStream_t s)
-{
-    if (!transA && !transB)
-        return launch_mfma_t<false, false, FM, FN, WGM, WGN>(A, B, C, bias, M, N, K, avec, bvec, s);
-    if (transA && !transB)
-        return launch_mfma_t<true, false, FM, FN, WGM, WGN>(A, B, C, bias, M, N, K, avec, bvec, s);
-    if (!transA && transB)
-        return launch_mfma_t<false, true, FM, FN, WGM, WGN>(A, B, C, bias, M, N, K, avec, bvec, s);
-    return launch_mfma_t<true, true, FM, FN, WGM, WGN>(A, B, C, bias, M, N, K, avec, bvec, s);
 }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -1411,30 +842,12 @@ REPDL_API int repdl_hip_mm_bias(const float *A, const float *B, const float *bia
     hipStream_t s = repdl_stream(stream);
     if (repdl_mfma_exact())
     {
-        // operand rows on 16-byte boundaries: the kernel that moves them straight into LDS
-        if (avec && bvec)
-        {
-            const int rc = mm_dma_dispatch(A, B, C, bias, nullptr, M, N, K, transA, transB, avec, bvec, 1, MmBatch{0, 0, 0}, s);
-            if (rc != REPDL_E_UNSUPPORTED)
-                return rc;
-        }
-        // Other operands: the kernels that stage them through registers.  A CU runs its tiles one after the other (256x256: one workgroup fills it) or
-        // side by side (smaller tiles), so a configuration costs (most tiles on any CU) x tile area
-        // / rate, with the rates measured per configuration and tiles per CU, relative to the
-        // 256x256 tile (135 TFLOP/s chip-wide): 128x128 0.785 alone on its CU, 0.92 with two, 0.955
-        // from three on; 64x64 0.555 alone, 0.76 with two, 0.85 with three or four, 0.88 beyond
-        // (4096^3: 1.03 / 1.08 / 1.13 ms with 256 / 128 / 64 tiles; 3072^2 x 4096, 144 / 576 / 2304
-        // tiles: 1.02 / 0.79 / 0.65 ms; 1024^3: 0.26 / 0.080 / 0.029 ms).
-        auto per_cu = [&](int64_t tm, int64_t tn) { return repdl_cdiv(repdl_cdiv(M, tm) * repdl_cdiv(N, tn), 256); };
-        const int64_t r256 = per_cu(256, 256), r128 = per_cu(128, 128), r64 = per_cu(64, 64);
-        const double c256 = (double)r256 * 65536.0;
-        const double c128 = (double)r128 * 16384.0 / (r128 >= 3 ? 0.955 : r128 == 2 ? 0.92 : 0.785);
-        const double c64 = (double)r64 * 4096.0 / (r64 >= 5 ? 0.88 : r64 >= 3 ? 0.85 : r64 == 2 ? 0.76 : 0.555);
-        if (c256 <= c128 && c256 <= c64)
-            return launch_mfma<4, 2, 2, 4>(A, B, C, bias, M, N, K, transA, transB, avec, bvec, s);
-        if (c128 <= c64)
-            return launch_mfma<2, 2, 2, 2>(A, B, C, bias, M, N, K, transA, transB, avec, bvec, s);
-        return launch_mfma<1, 1, 2, 2>(A, B, C, bias, M, N, K, transA, transB, avec, bvec, s);
+        // the kernel that moves operands straight into LDS, in 16-byte pieces where rows start on
+        // 16-byte boundaries, else in 4-byte pieces; it declines operands whose tiles span more than
+        // 32 bits of byte offsets (rows of tens of millions of elements), which take the kernel below
+        const int rc = mm_dma_dispatch(A, B, C, bias, nullptr, M, N, K, transA, transB, avec, bvec, 1, MmBatch{0, 0, 0}, s);
+        if (rc != REPDL_E_UNSUPPORTED)
+            return rc;
     }
     const int64_t gx = repdl_cdiv(N, BN), gy = repdl_cdiv(M, BM);
     REPDL_REQUIRE(gx * gy <= REPDL_I32_MAX);

@@ -31,7 +31,8 @@ WHOLE_TILE_SHAPES = [(4096, 4096, 48), (2048, 2048, 80), (512, 512, 96), (512, 5
                      (256, 192, 128), (128, 128, 2048),
                      (260, 132, 1000), (100, 36, 52), (4, 4, 4), (68, 20, 24), (1028, 2052, 36), (2500, 1300, 76), (8, 4100, 12),
                      (132, 260, 1001), (64, 64, 71), (512, 512, 2), (128, 4096, 72), (132, 4100, 40),
-                     (768, 772, 1102), (772, 768, 100), (1100, 1092, 52)]
+                     (768, 772, 1102), (772, 768, 100), (1100, 1092, 52),
+                     (770, 771, 1101), (1029, 2051, 37), (2501, 1299, 75), (4097, 4099, 21)]
 
 @pytest.mark.parametrize("tA,tB", [(0, 0), (1, 0), (0, 1), (1, 1)])
 @pytest.mark.parametrize("shape", WHOLE_TILE_SHAPES, ids=str)
