@@ -51,6 +51,9 @@ __global__ __launch_bounds__(RT) void rowchain_kernel(const float *__restrict__ 
     __shared__ __attribute__((aligned(16))) float tile[RR * RLD + 64]; // + 64: the walk reads ahead past the last row
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
+    // The workgroups that share a CU have ids 256 apart (the same id % 4), and the hardware starts each
+    // one's waves on the next SIMD (wave 0 of four co-resident workgroups was seen on SIMDs 1, 3, 0, 2):
+    // the same wave index in each puts their walks on different SIMDs.
     const int walker = blockIdx.x % (RT / 64);
     const int64_t r0 = (int64_t)blockIdx.x * RR;
     const int64_t tiles_per_seg = (seglen + RC - 1) / RC;
@@ -142,11 +145,13 @@ __global__ __launch_bounds__(RT) void rowchain_kernel(const float *__restrict__ 
         const bool more = t + 1 < ntiles;
         if (more)
             load(t + 1);
-        if (wave == walker && lane < RR)
+        if (wave == walker)
         {
+            // every lane walks (lanes RR and up repeat the first chains): a chain of dependent v_add_f32
+            // issues every 8.6 clocks in a wave with 32 or fewer active lanes, every 6.7 with 48 or more
             const int64_t sgm = t / tiles_per_seg, c0 = (t - sgm * tiles_per_seg) * RC;
             const int64_t rem = MULTI ? (nseg - t * spt < spt ? nseg - t * spt : spt) * seglen : seglen - c0;
-            const float *row = &tile[lane * RLD];
+            const float *row = &tile[(lane % RR) * RLD];
             // 8*WB elements per step, the next ones read from LDS before the adds of the current
             // ones: with few chains per workgroup the walk is the critical path, and it should
             // cost one dependent v_add_f32 per element and little else.  Elements past the end
@@ -244,8 +249,13 @@ __global__ __launch_bounds__(320) void coltile_kernel(const float *__restrict__ 
     const int64_t ntiles = (M + TR - 1) / TR;
 
     float acc = 0.0f;
-    v4f stage[RV];
-    auto load = [&](int64_t t) {
+    // NB = 2: PD tiles on their way from memory at any time, each in its own set of registers.  One is
+    // enough: 65536 x 4096 (256 workgroups, a tile row = half a 128-byte line) takes 0.262 ms with 1, 2, 4
+    // or 6, and also with the walk all but switched off -- a CU's movers bring in 16 GB/s of such half
+    // lines and no more, whatever is in flight.
+    constexpr int PD = 1;
+    v4f stages[PD][RV];
+    auto load = [&](int64_t t, v4f(&stage)[RV]) {
 #pragma unroll
         for (int i = 0; i < RV; i++)
         {
@@ -270,7 +280,7 @@ __global__ __launch_bounds__(320) void coltile_kernel(const float *__restrict__ 
             stage[i] = v;
         }
     };
-    auto store = [&](int buf) {
+    auto store = [&](int buf, const v4f(&stage)[RV]) {
 #pragma unroll
         for (int i = 0; i < RV; i++)
         {
@@ -284,42 +294,54 @@ __global__ __launch_bounds__(320) void coltile_kernel(const float *__restrict__ 
     };
     auto walk = [&](int64_t t, int buf) {
         const int64_t rem = M - t * TR; // rows of this tile that exist; the rest must not be added
-        const float *colp = &tile[buf][lane * TRP];
+        // every lane walks (lanes CW and up repeat the first columns): a chain of dependent v_add_f32 in a
+        // wave with 32 or fewer active lanes issues every 8.6 clocks, with 48 or more every 6.7 (measured)
+        const float *colp = &tile[buf][(lane % CW) * TRP];
         if (rem >= TR)
         {
-            // 16 rows ahead: the reads of the next 16 are issued before the adds of these
+            // batches of NRW reads = 4 NRW rows, two register sets: the reads of the next batch are
+            // issued, then the adds of this one run under their latency (pinned: left to itself
+            // the compiler interleaves them and every add then waits for a read)
+            // (few workgroups, NB = 2: batches of 64 rows, 100000 x 1000 0.38 -> 0.34 ms; with many workgroups
+            // the registers of long batches cost more than they gain: 16 rows)
+            constexpr int NRW = NB == 2 ? (TR / 8 < 16 ? TR / 8 : 16) : 4;
+            static_assert(TR % (8 * NRW) == 0, "a tile is whole pairs of batches");
             const v4f *cp = reinterpret_cast<const v4f *>(colp);
-            v4f va[4], vb[4];
+            v4f va[NRW], vb[NRW];
 #pragma unroll
-            for (int u = 0; u < 4; u++)
+            for (int u = 0; u < NRW; u++)
                 va[u] = cp[u];
-            for (int r = 0; r < TR; r += 32)
+            for (int r = 0; r < TR; r += 8 * NRW)
             {
 #pragma unroll
-                for (int u = 0; u < 4; u++)
-                    vb[u] = cp[(r + 16) / 4 + u];
+                for (int u = 0; u < NRW; u++)
+                    vb[u] = cp[(r + 4 * NRW) / 4 + u];
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int u = 0; u < 4; u++)
+                for (int u = 0; u < NRW; u++)
                 {
                     acc = acc + va[u].x;
                     acc = acc + va[u].y;
                     acc = acc + va[u].z;
                     acc = acc + va[u].w;
                 }
-                if (r + 32 < TR)
+                __builtin_amdgcn_sched_barrier(0);
+                if (r + 8 * NRW < TR)
                 {
 #pragma unroll
-                    for (int u = 0; u < 4; u++)
-                        va[u] = cp[(r + 32) / 4 + u];
+                    for (int u = 0; u < NRW; u++)
+                        va[u] = cp[(r + 8 * NRW) / 4 + u];
                 }
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int u = 0; u < 4; u++)
+                for (int u = 0; u < NRW; u++)
                 {
                     acc = acc + vb[u].x;
                     acc = acc + vb[u].y;
                     acc = acc + vb[u].z;
                     acc = acc + vb[u].w;
                 }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         else
@@ -330,37 +352,56 @@ __global__ __launch_bounds__(320) void coltile_kernel(const float *__restrict__ 
     };
 
     const bool mover = wave < 4;
-    if (ntiles > 0 && mover)
+    if (NB == 2)
     {
-        load(0);
-        store(0);
-        if (NB == 2 && ntiles > 1)
-            load(1);
-    }
-    __syncthreads();
-    for (int64_t t = 0; t < ntiles; t++)
-    {
-        if (NB == 2)
+        // set (t % PD) holds tile t from its request until it is stored
+        if (ntiles > 0 && mover)
         {
-            // tile t + 1 (in registers since the previous round) into the other buffer, tile t + 2 requested
-            if (mover && t + 1 < ntiles)
-                store((int)((t + 1) & 1));
-            if (mover && t + 2 < ntiles)
-                load(t + 2);
-            if (wave == walker && lane < CW)
-                walk(t, (int)(t & 1));
-            __syncthreads(); // tile t + 1 is complete, the walk of tile t is over
+            load(0, stages[0]);
+            store(0, stages[0]);
+#pragma unroll
+            for (int u = 1; u <= PD; u++)
+                if (u < ntiles)
+                    load(u, stages[u % PD]);
         }
-        else
+        __syncthreads();
+        for (int64_t t0 = 0; t0 < ntiles; t0 += PD)
+        {
+#pragma unroll
+            for (int u = 0; u < PD; u++)
+            {
+                const int64_t t = t0 + u;
+                if (t >= ntiles)
+                    break;
+                // tile t + 1 (requested PD tiles ago) into the other buffer, tile t + 1 + PD requested into its registers
+                if (mover && t + 1 < ntiles)
+                    store((int)((t + 1) & 1), stages[(u + 1) % PD]);
+                if (mover && t + 1 + PD < ntiles)
+                    load(t + 1 + PD, stages[(u + 1) % PD]);
+                if (wave == walker)
+                    walk(t, (int)(t & 1));
+                __syncthreads(); // tile t + 1 is complete, the walk of tile t is over
+            }
+        }
+    }
+    else
+    {
+        if (ntiles > 0 && mover)
+        {
+            load(0, stages[0]);
+            store(0, stages[0]);
+        }
+        __syncthreads();
+        for (int64_t t = 0; t < ntiles; t++)
         {
             const bool more = t + 1 < ntiles;
             if (more && mover)
-                load(t + 1);
-            if (wave == walker && lane < CW)
+                load(t + 1, stages[0]);
+            if (wave == walker)
                 walk(t, 0);
             __syncthreads(); // the walk of tile t is over: the buffer may be overwritten
             if (more && mover)
-                store(0);
+                store(0, stages[0]);
             __syncthreads();
         }
     }
