@@ -249,7 +249,9 @@ def cpu_time(fn, reps=1):
 # latency of a dependent instruction (about 10 clocks for v_add_f32 in a lone wave, 35 for a dependent
 # v_mfma_f32_16x16x4_f32 = 8.75 per k), whatever the bandwidth.
 CHAIN_LIMITS = {
-    "sum2d_dim0": "chain latency: 65536 dependent additions per column at ~10 clocks = 0.28 ms",
+    "sum2d_dim0": "one workgroup per CU (256 groups of 16 columns, 65536 rows each), whose tile rows are half cache lines: a CU "
+                  "brings in 16 GB/s of those whatever is in flight or walked (0.262 ms even with the walk switched off); the chains "
+                  "themselves, 65536 dependent additions at 6.7 clocks, would take 0.18 ms",
     "sum4d_dim023": "chain latency: 64 chains of 200704 additions (0.85 ms if every addition were made one after the other; the "
                     "interval maps of the parallel evaluation skip about half of them)",
     "sum1d": "one chain of 2^28 additions (1.1 s at 10 clocks each): evaluated exactly in parallel by interval maps over candidate "
