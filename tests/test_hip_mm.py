@@ -95,6 +95,26 @@ def test_bias_in_the_epilogue(shape, tA, tB):
     assert torch.equal(none.view(torch.int32), oracle.mm(a, b, bool(tA), bool(tB)).view(torch.int32))
 
 
+def test_rows_longer_than_32_bit_tile_offsets():
+    """Rows of 2^25 + 4 elements: a 32-row operand tile spans more than 2^32 bytes, which the kernel that
+    moves tiles global->LDS with 32-bit lane offsets declines; the product must come out right anyway."""
+    from repdl_amd import ops
+
+    M, N, K = 4, 4, (1 << 25) + 4
+    rng = torch.Generator().manual_seed(11)
+    a = torch.randint(-3, 4, (M, K), generator=rng).float()
+    b = torch.randint(-3, 4, (N, K), generator=rng).float()
+    a[:, ::3] *= 0.37  # products and partial sums round
+    got = ops.mm(a.cuda(), b.cuda(), False, True).cpu()
+    want = oracle.mm(a, b, False, True)
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+    # the same with the long rows in an operand whose k runs down the columns
+    a2 = torch.randint(-3, 4, (2, 6), generator=rng).float() * 0.37
+    b2 = torch.randint(-3, 4, (6, K), generator=rng).float()
+    got = ops.mm(a2.cuda(), b2.cuda()).cpu()
+    assert torch.equal(got.view(torch.int32), oracle.mm(a2, b2).view(torch.int32))
+
+
 def test_unaligned_operands():
     from repdl_amd import ops
 
