@@ -2152,14 +2152,22 @@ __global__ __launch_bounds__(256, 6) void conv_point_kernel(const float *__restr
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int C = MODE == MODE_FWD ? d.IC : d.OC, M = MODE == MODE_FWD ? d.OC : d.IC;
     const int P = d.H * d.W; // (1x1, stride 1, no padding: input and output planes coincide)
-    const int n = blockIdx.z, m0 = blockIdx.y * 64, p0 = blockIdx.x * 128;
+    // Workgroup ids go to the 8 XCDs round-robin.  The M / 64 row tiles of one pixel tile read the same
+    // columns of Src: they get ids 8 apart -- the same XCD, dispatched back to back -- so that only the
+    // first of them brings those columns in from memory (256 rows: 412 -> 2xx MB per call).
+    const int mtiles = M / 64, ptiles = (P + 127) / 128;
+    const int group = blockIdx.x / (8 * mtiles), rest = blockIdx.x % (8 * mtiles);
+    const int pt = group * 8 + rest % 8, mt = rest / 8;
+    if (pt >= ptiles * d.N)
+        return;
+    const int n = pt / ptiles, m0 = mt * 64, p0 = (pt % ptiles) * 128;
     const int pix = p0 + wave * 32 + l32;
     const int pc = pix < P ? pix : P - 1;
     const int npair = C / 2;
     const __amdgpu_buffer_rsrc_t brsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(Src + (int64_t)n * C * P), 0, C * P * 4, 0x00020000);
     const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<float *>(PA + (int64_t)blockIdx.y * npair * 128), 0, npair * 128 * 4, 0x00020000);
+        const_cast<float *>(PA + (int64_t)mt * npair * 128), 0, npair * 128 * 4, 0x00020000);
     const int b_voff = (half * P + pc) * 4, a_voff = lane * 4;
     const int pair_bytes = 2 * P * 4;
 
@@ -2203,7 +2211,7 @@ __global__ __launch_bounds__(256, 6) void conv_point_kernel(const float *__restr
                 float v = acc[i][r];
                 if (has_bias)
                     v = v + d.bias[m];
-                Oimg[(int64_t)m * P + pix] = v;
+                __builtin_nontemporal_store(v, &Oimg[(int64_t)m * P + pix]);
             }
     }
 }
@@ -2231,6 +2239,7 @@ bool applies(const ConvDims &d)
     const int64_t P = (int64_t)d.H * d.W;
     return d.groups == 1 && d.KH == 1 && d.KW == 1 && d.sH == 1 && d.sW == 1 && d.pH == 0 && d.pW == 0 && M % 64 == 0 && M / 64 <= 65535 &&
            C % (2 * RING) == 0 && C >= 2 * RING && P >= 1 && d.N <= 65535 && (int64_t)C * P * 4 < (1LL << 31) && (int64_t)M * C * 4 < (1LL << 31) &&
+           (repdl_cdiv(P, 128) * d.N + 8) * (M / 64) < (1LL << 30) &&
            P >= 1024; // (small images: the products over all images at once, see conv_prefers_mm)
 }
 
@@ -2245,7 +2254,8 @@ int launch(const float *gathered, const float *kernel, float *out, const ConvDim
     if (e0 != hipSuccess)
         return (int)e0;
     hipLaunchKernelGGL(conv_point_prep_kernel, dim3((unsigned)repdl_cdiv(wcount, 256)), dim3(256), 0, s, kernel, PA, wcount, MODE, C, M);
-    const dim3 grid((unsigned)repdl_cdiv(P, 128), (unsigned)(M / 64), (unsigned)d.N);
+    const int64_t ptiles = repdl_cdiv(P, 128) * d.N;
+    const dim3 grid((unsigned)(repdl_cdiv(ptiles, 8) * 8 * (M / 64)));
     hipLaunchKernelGGL((conv_point_kernel<MODE>), grid, dim3(256), 0, s, gathered, PA, out, d);
     const int rc = repdl_launch_status();
     const hipError_t e = hipFreeAsync(PA, s);
