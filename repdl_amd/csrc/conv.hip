@@ -1840,7 +1840,14 @@ __global__ __launch_bounds__(128 * WGN) void conv_tapdma_kernel(const float *__r
     const int PH = MODE == MODE_FWD ? d.OH : d.H, PW = MODE == MODE_FWD ? d.OW : d.W; // output plane
     const int P = PH * PW, K = C * 9;
     const int dymin = MODE == MODE_FWD ? -d.pH : d.pH - 2, dxmin = MODE == MODE_FWD ? -d.pW : d.pW - 2;
-    const int n = blockIdx.z, m0 = blockIdx.y * 64, p0 = blockIdx.x * TN;
+    // The row tiles of one pixel tile read the same patch: ids 8 apart, i.e. the same XCD, back to back
+    // (workgroup ids go to the XCDs round-robin), so that only the first brings it in from memory.
+    const int mtiles = (M + 63) / 64, ptiles = (P + TN - 1) / TN;
+    const int group = blockIdx.x / (8 * mtiles), rest = blockIdx.x % (8 * mtiles);
+    const int pt = group * 8 + rest % 8;
+    if (pt >= ptiles * d.N)
+        return;
+    const int n = pt / ptiles, m0 = (rest / 8) * 64, p0 = (pt % ptiles) * TN;
     const int y0 = p0 / PW;
     const int pitch = patch_pitch(SW, VEC), gpr = pitch / VEC, plane = PR * pitch; // gpr: DMA lanes per patch row
     const int nslot = CCH * PR * gpr, nib = (nslot + 63) / 64;
@@ -2034,7 +2041,7 @@ __global__ __launch_bounds__(128 * WGN) void conv_tapdma_kernel(const float *__r
                 }
                 if (has_bias)
                     v = v + bias_s[m - m0];
-                Oimg[(int64_t)m * P + pix[j]] = v;
+                __builtin_nontemporal_store(v, &Oimg[(int64_t)m * P + pix[j]]);
             }
         }
 }
@@ -2077,7 +2084,8 @@ bool applies(const ConvDims &d, const float *gathered, const float *kernel, int 
     const int SH = MODE == MODE_FWD ? d.H : d.OH, SW = MODE == MODE_FWD ? d.W : d.OW;
     const int PH = MODE == MODE_FWD ? d.OH : d.H, PW = MODE == MODE_FWD ? d.OW : d.W;
     if (!(d.groups == 1 && d.KH == 3 && d.KW == 3 && d.sH == 1 && d.sW == 1 && d.pH <= 2 && d.pW <= 2 && M >= 1 && (M + 63) / 64 <= 65535 &&
-          C % CCH == 0 && C >= CCH && PH >= 1 && PW >= 1 && SH >= 1 && SW >= 1 && d.N <= 65535))
+          C % CCH == 0 && C >= CCH && PH >= 1 && PW >= 1 && SH >= 1 && SW >= 1 && d.N <= 65535 &&
+          (repdl_cdiv((int64_t)PH * PW, TN) * d.N + 8) * ((M + 63) / 64) < (1LL << 30)))
         return false;
     if ((reinterpret_cast<uintptr_t>(kernel) & 15) != 0)
         return false;
@@ -2120,7 +2128,7 @@ int launch(const float *gathered, const float *kernel, float *out, const ConvDim
             return (int)e;
         }
     }
-    const dim3 grid((unsigned)repdl_cdiv(P, TN), (unsigned)repdl_cdiv(M, 64), (unsigned)d.N);
+    const dim3 grid((unsigned)(repdl_cdiv(repdl_cdiv(P, TN) * d.N, 8) * 8 * repdl_cdiv(M, 64)));
     hipLaunchKernelGGL(kern, grid, dim3(128 * WGN), shmem, s, gathered, kernel, MODE == MODE_DGRAD ? PA : kernel, out, d,
                        guard_parts(guard, 0), ca, guard_parts(guard, 1), cb, skips ? 1 : 0, patch_rows(TN, PW));
     const int rc = repdl_launch_status();
