@@ -1436,7 +1436,15 @@ static int spec_rounds(int64_t rows, int64_t n)
     if (g_debug_rounds >= 0)
         return g_debug_rounds;
 #endif
-    if (rows != 1 || n < ((int64_t)1 << 22))
+    // Chains that come in rows: three rounds when the chains are very long and their nodes few enough
+    // for one pass of the walkers.  Zero-mean chains gain (16 x 802816: 1.27 -> 0.42 ms, 8 x 2^20: 1.07 ->
+    // 0.37), chains that drift lose the rounds' fifteen launches (0.09 -> 0.14 ms).  At 200704 elements
+    // (64 channels of 64 images of 56x56) gain and loss are the same 0.1 ms (0.50 -> 0.33 against 0.08 ->
+    // 0.18) and a residual block with BatchNorm got 3 % slower with the rounds: not there.  256 x 262144
+    // (4096 nodes) got slower either way.
+    if (rows > 1)
+        return (n >= ((int64_t)1 << 19) && rows * repdl_cdiv(repdl_cdiv(n, BLK), NODEB) <= 2048) ? 3 : 0;
+    if (n < ((int64_t)1 << 22))
         return 0;
     return n < ((int64_t)1 << 24) ? 4 : (n < ((int64_t)1 << 26) ? 8 : MAX_ROUNDS);
 }

@@ -226,6 +226,55 @@ def test_sum1d_speculative_rounds(name, x):
     assert got.view(torch.int32).item() == want.view(torch.int32).item() or (torch.isnan(got) and torch.isnan(want)), name
 
 
+def test_rounds_on_chains_in_rows():
+    """Row sums and channel sums whose chains are long enough (2^19 elements and more) for the speculative
+    rounds: every row a different kind of trouble -- zero crossings, a fall through many binades, stagnation
+    at a power of two, zero stretches, an infinity, NaNs, tiny and huge magnitudes -- and ragged lengths."""
+    from repdl_amd import ops
+
+    r = _rng(77)
+    n = (1 << 19) + 4321
+    rows = []
+    rows.append(r.standard_normal(n))
+    rows.append(r.random(n) * 2 - 1)
+    d = r.standard_normal(n)
+    d[0] = 3.0e5
+    d[1:200_000] = -np.abs(d[1:200_000]) * 1.5
+    rows.append(d)
+    rows.append(0.25 + 0.75 * r.random(n))                 # keeps growing
+    rows.append((0.25 + 0.75 * r.random(n)) * 2.0**7)      # stops growing at 2^24 * 2^7 / ... within the row
+    z = r.standard_normal(n)
+    z[50_000:120_000] = 0.0
+    z[130_000:130_064] = -0.0
+    rows.append(z)
+    w = r.standard_normal(n)
+    w[200_001] = np.inf
+    rows.append(w)
+    v = r.standard_normal(n)
+    v[100_000], v[100_777] = np.inf, -np.inf
+    rows.append(v)
+    rows.append(r.standard_normal(n) * 2.0**-140)
+    rows.append(r.standard_normal(n) * 2.0**100)
+    rows.append(gen.scaled_normal(78, n).numpy())
+    rows.append(np.zeros(n))
+    m = torch.from_numpy(np.stack(rows).astype(np.float32))
+    for avg in (False, True):
+        got = ops.sum2d_dim1(m.cuda(), False, avg).cpu()
+        want = oracle.sum2d_dim1(m, False, avg)
+        same = (got.view(torch.int32) == want.view(torch.int32)) | (torch.isnan(got) & torch.isnan(want))
+        assert bool(same.all()), (avg, torch.nonzero(~same).flatten().tolist())
+    # channel sums: 8 channels of 48 images of 112x112 (602112 elements per chain), zero-mean and shifted channels
+    x = torch.from_numpy(r.standard_normal((48, 8, 112, 112)).astype(np.float32))
+    x[:, 3] += 0.5
+    x[:, 5] = x[:, 5].abs()
+    x[:, 7] *= 2.0**-130
+    x[7, 2, 3, 3] = float("inf")
+    got = ops.sum4d_dim023(x.cuda()).cpu()
+    want = oracle.sum4d_dim023(x)
+    same = (got.view(torch.int32) == want.view(torch.int32)) | (torch.isnan(got) & torch.isnan(want))
+    assert bool(same.all()), torch.nonzero(~same).flatten().tolist()
+
+
 def test_sum1d_long_unaligned_and_workspace():
     """A long chain from a pointer 4 bytes off a 16-byte boundary, and the same through the entry point
     that takes the caller's scratch memory (deliberately filled with junk first)."""
