@@ -263,6 +263,10 @@ def test_rounds_on_chains_in_rows():
         want = oracle.sum2d_dim1(m, False, avg)
         same = (got.view(torch.int32) == want.view(torch.int32)) | (torch.isnan(got) & torch.isnan(want))
         assert bool(same.all()), (avg, torch.nonzero(~same).flatten().tolist())
+    # two rows long enough for more than 16 super-blocks each (the round's kernels stay separate there)
+    m2 = torch.from_numpy(np.stack([r.standard_normal((1 << 23) + 77), r.random((1 << 23) + 77) - 0.5]).astype(np.float32))
+    got = ops.sum2d_dim1(m2.cuda()).cpu()
+    assert torch.equal(got.view(torch.int32), oracle.sum2d_dim1(m2).view(torch.int32))
     # channel sums: 8 channels of 48 images of 112x112 (602112 elements per chain), zero-mean and shifted channels
     x = torch.from_numpy(r.standard_normal((48, 8, 112, 112)).astype(np.float32))
     x[:, 3] += 0.5
