@@ -563,6 +563,53 @@ __device__ __forceinline__ bool lane_tup_apply(uint32_t &s, const LaneTup &l, in
     return ok;
 }
 
+// The same tuples laid out for the single walking wave, whose cost is its instruction count (a lone
+// wave issues an instruction about every 8 clocks whatever it is): node i of 64 sits in lane
+// 2 (i % 32) + parity of register set i / 32, as the start and the LENGTH of the interval of states of
+// that parity to which the map applies, so that a test is (s - smin) < len on the scalar unit after
+// three v_readlane_b32 -- about ten instructions against nineteen for lane_tup_apply.
+// (An interval of all 2^32 states is stored with length 2^32 - 1: the state 0xFFFFFFFF then fails
+// the test and takes the slower way down to real additions, which is always right.)
+struct WalkHalf
+{
+    uint32_t smin, len;
+    int t;
+};
+struct WalkTup
+{
+    WalkHalf A, B; // nodes 0..31 and 32..63
+};
+
+__device__ __forceinline__ WalkTup walk_tup(const LaneTup &l)
+{
+    const int lane = threadIdx.x & 63, node = lane >> 1;
+    const bool odd = (lane & 1) != 0;
+    WalkTup w;
+    auto pick = [&](int nd, WalkHalf &h) {
+        const uint32_t lo0 = (uint32_t)__shfl((int)l.smin0, nd, 64), hi0 = (uint32_t)__shfl((int)l.smax0, nd, 64);
+        const uint32_t lo1 = (uint32_t)__shfl((int)l.smin1, nd, 64), hi1 = (uint32_t)__shfl((int)l.smax1, nd, 64);
+        const int t0 = __shfl(l.t0, nd, 64), t1 = __shfl(l.t1, nd, 64);
+        const uint32_t lo = odd ? lo1 : lo0, hi = odd ? hi1 : hi0;
+        h.smin = lo;
+        h.len = hi < lo ? 0u : (hi - lo == 0xFFFFFFFFu ? 0xFFFFFFFFu : hi - lo + 1u);
+        h.t = odd ? t1 : t0;
+    };
+    pick(node, w.A);
+    pick(node + 32, w.B);
+    return w;
+}
+
+// Try node i5 (wave-uniform, 0..31) of those held in h; false if it does not apply to state s.
+__device__ __forceinline__ bool walk_apply(uint32_t &s, const WalkHalf &h, int i5)
+{
+    const int idx = 2 * i5 + (int)(s & 1u);
+    const uint32_t smin = __builtin_amdgcn_readlane(h.smin, idx), len = __builtin_amdgcn_readlane(h.len, idx);
+    const int tt = __builtin_amdgcn_readlane(h.t, idx);
+    const bool ok = s - smin < len;
+    s = ok ? s + (uint32_t)tt : s;
+    return ok;
+}
+
 // ---- step 3b: tuples of nodes (16 blocks) and super-blocks (64 blocks) -------------------------
 // Per row: where the true state is known exactly so far (a super-block index and the state
 // there); nsup once the whole chain is resolved.
@@ -745,11 +792,16 @@ __global__ __launch_bounds__(64) void sum1d_walk_kernel(const float *__restrict_
     Tup blk_next = (first * SUP + lane < nblk) ? T2[first * SUP + lane] : tup_identity(HYP_ANY);
     for (int64_t g0 = gfirst; g0 < nsup; g0 += 64)
     {
-        const LaneTup ls = lane_tup(nsup_t);
+        const WalkTup ls = walk_tup(lane_tup(nsup_t));
         if (g0 + 64 < nsup) // the next 64 super-block tuples, loaded while these are walked
             nsup_t = (g0 + 64 + lane < nsup) ? T3[g0 + 64 + lane] : tup_identity(HYP_ANY);
         const int cnt = (nsup - g0 < 64) ? (int)(nsup - g0) : 64;
-        for (int i = (g0 == gfirst ? (int)(first - gfirst) : 0); i < cnt; i++)
+        const int i_first = g0 == gfirst ? (int)(first - gfirst) : 0;
+        for (int hs = i_first >> 5; hs < 2 && 32 * hs < cnt; hs++)
+        {
+        const WalkHalf lsh = hs ? ls.B : ls.A;
+        const int i_end = cnt < 32 * hs + 32 ? cnt : 32 * hs + 32;
+        for (int i = i_first > 32 * hs ? i_first : 32 * hs; i < i_end; i++)
         {
             const int64_t sb = g0 + i;
             const Tup blk_cur = blk_next;
@@ -757,22 +809,25 @@ __global__ __launch_bounds__(64) void sum1d_walk_kernel(const float *__restrict_
                 const int64_t b = (sb + 1) * SUP + lane; // always requested: 32 bytes per block
                 blk_next = b < nblk ? T2[b] : tup_identity(HYP_ANY);
             }
-            if (lane_tup_apply(s, ls, i))
+            if (walk_apply(s, lsh, i & 31))
                 continue;
-            const LaneTup lb = lane_tup(blk_cur);
-            for (int bi = 0; bi < SUP; bi++)
+            const WalkTup lb = walk_tup(lane_tup(blk_cur));
+            for (int hb = 0; hb < SUP / 32; hb++)
             {
-                if (lane_tup_apply(s, lb, bi)) // blocks past the end are identities
+            const WalkHalf lbh = hb ? lb.B : lb.A;
+            for (int b5 = 0; b5 < 32; b5++)
+            {
+                if (walk_apply(s, lbh, b5)) // blocks past the end are identities
                     continue;
                 // The block as a whole does not apply.
-                const int64_t blk = sb * SUP + bi;
+                const int64_t blk = sb * SUP + 32 * hb + b5;
                 if (pf_blk != blk)
                     load_block(pf, x, c, T1, TG, blk, lane, vec);
                 __syncthreads();
 #pragma unroll
                 for (int q = 0; q < BLK / 256; q++)
                     *reinterpret_cast<float4 *>(&xd[(q * 64 + lane) * 4]) = pf.f[q];
-                const LaneTup lg = lane_tup(pf.tgr), lc = lane_tup(pf.tch);
+                const WalkTup lg = walk_tup(lane_tup(pf.tgr)), lc = walk_tup(lane_tup(pf.tch));
                 __syncthreads();
                 {
                     const int64_t nb = blk + 1 < nblk ? blk + 1 : blk;
@@ -781,24 +836,28 @@ __global__ __launch_bounds__(64) void sum1d_walk_kernel(const float *__restrict_
                 }
                 for (int gr = 0; gr < GROUPS; gr++)
                 {
-                    if (lane_tup_apply(s, lg, gr))
+                    if (walk_apply(s, lg.A, gr))
                         continue;
                     constexpr int CG = BLK / CH / GROUPS; // 8 chunks, reads one chunk ahead
+                    static_assert(GROUPS <= 32 && (32 % CG) == 0, "a group's chunks lie in one half");
                     const int j0 = gr * CG;
+                    const WalkHalf lch = j0 < 32 ? lc.A : lc.B;
                     f4v va[CH / 4], vb[CH / 4];
                     read_chunk(xd, j0, va);
 #pragma unroll
                     for (int j = 0; j < CG; j += 2)
                     {
                         read_chunk(xd, j0 + j + 1, vb);
-                        if (!lane_tup_apply(s, lc, j0 + j))
+                        if (!walk_apply(s, lch, (j0 + j) & 31))
                             s = replay_chunk(s, va);
                         read_chunk(xd, j0 + j + 2, va);
-                        if (!lane_tup_apply(s, lc, j0 + j + 1))
+                        if (!walk_apply(s, lch, (j0 + j + 1) & 31))
                             s = replay_chunk(s, vb);
                     }
                 }
             }
+            }
+        }
         }
     }
     if (lane == 0)
