@@ -148,9 +148,9 @@ __global__ __launch_bounds__(64) void cross_entropy_rows_kernel(const float *__r
 // threads share a row; thread j of them holds the 16-byte granules j, j + TPR, j + 2 TPR, ...
 // of the row in registers (VPT values), so the row is read from memory once, coalesced.
 // The maximum is a reduction over registers and the TPR lanes; the exponentials stay in
-// the registers and are also laid into LDS, row stride N + 1 floats; after a barrier lane
-// l of wave 0 walks row l of that image in order, one addition per column for all R rows
-// at once (the odd stride keeps the lanes on different banks).  The quotients are then
+// the registers and are also laid into LDS (onchip_stride floats per row); after a barrier lane
+// l of wave 0 walks row l % R of that image in order, one addition per column for all R rows
+// at once, thirty-two values read ahead with ds_read_b128.  The quotients are then
 // taken of the register copy and written once: 8 bytes per element in all (4 for the
 // loss).  Used for many rows (rows_onchip_wanted), where a wave per row saturates the SIMDs
 // with the per-row chain steps, and up to 4096 columns.
@@ -169,6 +169,13 @@ inline bool rows_onchip_wanted(int64_t M, int64_t N)
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
+// LDS row of the image: whole 16-byte granules (the chain is walked with ds_read_b128), one more at
+// least, an odd number of them in all -- sixteen consecutive rows then start in sixteen different
+// groups of four banks, and the walking lanes' reads do not collide
+// (rows of 128 columns and fewer, 32 or 64 of them per workgroup, keep N + 1 floats and 4-byte accesses:
+// the wider layout made cross_entropy on 65536 x 64 slower, 0.054 -> 0.061 ms)
+__host__ __device__ inline int onchip_stride(int N, int R) { return R >= 32 ? N + 1 : 4 * (((N + 3) / 4 + 1) | 1); }
+
 __device__ __forceinline__ float nan_max(float m, float v) { return (v != v) ? v : ((m != m) ? m : (v > m ? v : m)); }
 
 // SOFTMAX: out = softmax rows.  Otherwise: loss[row] = log(sum_j exp(x_j - m)) - (x_target - m).
@@ -183,7 +190,7 @@ __global__ __launch_bounds__(256) void rows_onchip_kernel(const float *__restric
     __shared__ double log_hi[SOFTMAX ? 1 : 128];
     __shared__ float log_invc[SOFTMAX ? 1 : 128], log_lo[SOFTMAX ? 1 : 128];
     __shared__ float rmax[R], rsum[R];
-    extern __shared__ float image[]; // R rows of N + 1 floats
+    extern __shared__ __attribute__((aligned(16))) float image[]; // R rows of onchip_stride(N, R) floats
     const int tid = threadIdx.x;
     exp_tab[tid] = g_exp_tab2[tid];
     if (!SOFTMAX && tid < 128)
@@ -197,7 +204,8 @@ __global__ __launch_bounds__(256) void rows_onchip_kernel(const float *__restric
     const bool live = row0 + r < M;
     const int64_t row = live ? row0 + r : M - 1; // rows past the end repeat the last one and store nothing
     const float *x = in + row * N;
-    const int stride = N + 1;
+    constexpr bool VROW = R < 32; // rows as whole 16-byte granules
+    const int stride = onchip_stride(N, R);
 
     // the row, once
     float v[VPT];
@@ -244,44 +252,94 @@ __global__ __launch_bounds__(256) void rows_onchip_kernel(const float *__restric
 #pragma unroll
             for (int k = 0; k < 4; k++)
                 v[4 * i + k] = crm_exp(v[4 * i + k] - m, exp_tab);
+            if (VROW)
+            {
+                if (c < N) // (columns past N inside the last granule hold exp(-inf) = +0 and are never walked)
+                    *reinterpret_cast<v4f *>(img + c) = (v4f){v[4 * i + 0], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]};
+            }
+            else
+            {
 #pragma unroll
-            for (int k = 0; k < 4; k++)
-                if (c + k < N)
-                    img[c + k] = v[4 * i + k];
+                for (int k = 0; k < 4; k++)
+                    if (c + k < N)
+                        img[c + k] = v[4 * i + k];
+            }
         }
     }
     __syncthreads();
-    if (tid < R)
+    if (tid < 64)
     {
-        // the chain of row `tid`: sixteen values ahead in registers while sixteen are added
-        const float *wr = image + tid * stride;
+        // the chain of row `tid` (lanes R and up of the wave walk the first rows again: a chain of dependent
+        // v_add_f32 issues every 6.7 clocks in a full wave, every 8.6 with most lanes off, and masked walks
+        // on one CU slow each other to 20): sixteen values ahead in registers while sixteen are added
+        const float *wr = image + (tid % R) * stride;
         float acc = 0.0f;
-        float cur[16], nxt[16];
-        const int whole = N & ~15;
-        if (whole > 0)
+        int whole = 0;
+        if (VROW)
         {
+            constexpr int WB = 8; // granules per batch: 32 values ahead in registers while 32 are added
+            v4f cur[WB], nxt[WB];
+            whole = N & ~(4 * WB - 1);
+            const v4f *wq = reinterpret_cast<const v4f *>(wr);
+            if (whole > 0)
+            {
 #pragma unroll
-            for (int u = 0; u < 16; u++)
-                cur[u] = wr[u];
+                for (int u = 0; u < WB; u++)
+                    cur[u] = wq[u];
+            }
+            for (int k = 0; k < whole; k += 4 * WB)
+            {
+                if (k + 4 * WB < whole)
+                {
+#pragma unroll
+                    for (int u = 0; u < WB; u++)
+                        nxt[u] = wq[(k + 4 * WB) / 4 + u];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < WB; u++)
+                {
+                    acc = acc + cur[u].x;
+                    acc = acc + cur[u].y;
+                    acc = acc + cur[u].z;
+                    acc = acc + cur[u].w;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < WB; u++)
+                    cur[u] = nxt[u];
+            }
         }
-        for (int k = 0; k < whole; k += 16)
+        else
         {
-            if (k + 16 < whole)
+            float cur[16], nxt[16]; // sixteen values ahead in registers while sixteen are added
+            whole = N & ~15;
+            if (whole > 0)
             {
 #pragma unroll
                 for (int u = 0; u < 16; u++)
-                    nxt[u] = wr[k + 16 + u];
+                    cur[u] = wr[u];
             }
+            for (int k = 0; k < whole; k += 16)
+            {
+                if (k + 16 < whole)
+                {
 #pragma unroll
-            for (int u = 0; u < 16; u++)
-                acc = acc + cur[u];
+                    for (int u = 0; u < 16; u++)
+                        nxt[u] = wr[k + 16 + u];
+                }
 #pragma unroll
-            for (int u = 0; u < 16; u++)
-                cur[u] = nxt[u];
+                for (int u = 0; u < 16; u++)
+                    acc = acc + cur[u];
+#pragma unroll
+                for (int u = 0; u < 16; u++)
+                    cur[u] = nxt[u];
+            }
         }
         for (int k = whole; k < N; k++)
             acc = acc + wr[k];
-        rsum[tid] = acc;
+        if (tid < R)
+            rsum[tid] = acc;
     }
     __syncthreads();
 
@@ -332,7 +390,7 @@ int launch_rows_onchip(const float *in, float *out, const int64_t *target, float
                        hipStream_t s)
 {
     auto kern = &rows_onchip_kernel<R, VPT, SOFTMAX>;
-    const size_t shmem = (size_t)R * (N + 1) * sizeof(float);
+    const size_t shmem = (size_t)R * onchip_stride((int)N, R) * sizeof(float);
     if (shmem > 40 * 1024)
     {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
