@@ -1744,21 +1744,49 @@ __global__ __launch_bounds__(256) void wgrad_fixup_kernel(const float *__restric
     GK[idx] = conv2d_grad_kernel_exact(GO, X, d, oc, ic, kh, kw);
 }
 
+#ifdef REPDL_DEBUG_HOOKS
+int g_wgrad_route = 0; // 1: always the product, 2: always the chain kernel
+#endif
 // Rough times of the two grad-kernel routes (seconds), from measurements on the layers of a
-// ResNet at batch 64: the chain kernel needs 12 clocks per step of a chain and about 34 us per
-// round of 256 workgroups (one per CU) on top; the product runs at about 100 TFLOP/s once it
-// has enough tiles, never faster than its own k-chain (32 clocks per step with 32x32x2
-// instructions), plus the passes that write its operands.
-inline bool wgrad_prefers_gemm(int64_t OC, int64_t NC, int64_t K)
+// ResNet at batch 64: the chain kernel needs 12 clocks per step of a chain at stride 1 and 18 at
+// stride 2 (64 -> 128, 3x3, stride 2 at 56x56: 0.38 ms for 50176 steps), and about 34 us per round of
+// 256 workgroups (one per CU) on top; the product runs at about 100 TFLOP/s once it has enough
+// tiles, never faster than its own k-chain on small tiles (about 20 clocks per step: 128 x 64 x 50176
+// 0.43 ms), plus the passes that write its operands.  (128 -> 256, 3x3, stride 2 at 28x28: chain
+// 0.37 ms, product 0.26; 256 -> 256 at 14x14: 0.49 / 0.36; 128 -> 128 at 28x28: 0.52 / 0.63.)  On output rows
+// of fewer than 16 pixels the chain kernel's pieces are one or two instructions long and mostly
+// overhead: 256 -> 512, 1x1 at 7x7, 3136 steps, 0.19 ms against 0.065 for the product.  With a 1x1
+// kernel the sixteen columns of a block are sixteen channels, whose rows all have to be staged: about
+// 90 us per round instead of 34 (1024 -> 256 at 14x14, two rounds of 12544 steps: 0.33 ms, product 0.20).
+inline bool wgrad_prefers_gemm(int64_t OC, int64_t NC, int64_t K, int64_t sW, int64_t OW, int64_t KHW)
 {
+#ifdef REPDL_DEBUG_HOOKS
+    if (g_wgrad_route != 0)
+        return g_wgrad_route == 1;
+#endif
     const double clk = 1.0 / 2.35e9;
     const double rounds = (double)repdl_cdiv(repdl_cdiv(NC, 16) * repdl_cdiv(OC, 32), 256);
-    const double step = (double)K * 12.0 * clk;
-    const double t_chain = rounds <= 1.0 ? step : rounds * (step + 34e-6);
+    const int64_t OWr = (OW + 3) / 4 * 4;
+    const double step = (double)K * (sW > 1 ? 18.0 : 12.0) * (OWr < 16 ? 16.0 / (double)OWr : 1.0) * clk;
+    const double t_chain = (rounds < 1.0 ? 1.0 : rounds) * (step + (KHW == 1 ? 90e-6 : 34e-6));
     const double flop = 2.0 * (double)OC * (double)NC * (double)K;
-    const double t_mm = flop / 100e12 > (double)K * 32.0 * clk ? flop / 100e12 : (double)K * 32.0 * clk;
+    const double t_mm = flop / 100e12 > (double)K * 20.0 * clk ? flop / 100e12 : (double)K * 20.0 * clk;
     const double t_gemm = t_mm + (double)K * (double)(NC + OC) * 8.0 / 3e12 + 40e-6;
     return t_gemm < 0.8 * t_chain;
+}
+
+// X'[n][c][oh][ow] = X[n][c][oh * sH][ow * sW]: what a 1x1 kernel at a stride reads of its input
+__global__ __launch_bounds__(256) void conv_subsample_kernel(const float *__restrict__ X, float *__restrict__ Xs, int64_t total,
+                                                             int H, int W, int OH, int OW, int sH, int sW)
+{
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total)
+        return;
+    const int ow = (int)(idx % OW);
+    const int64_t t = idx / OW;
+    const int oh = (int)(t % OH);
+    const int64_t plane = t / OH;
+    Xs[idx] = X[(plane * H + (int64_t)oh * sH) * W + (int64_t)ow * sW];
 }
 
 // ---------------------------------------------------------------------------
@@ -2667,6 +2695,14 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
     return launch_conv_gemm<MODE_DGRAD>(grad_output, kernel, grad_input, d, stream);
 }
 
+#ifdef REPDL_DEBUG_HOOKS
+REPDL_API int repdl_debug_wgrad_route(int r)
+{
+    g_wgrad_route = r;
+    return 0;
+}
+#endif
+
 REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float *input,
                                            float *grad_kernel, int64_t N, int64_t IC, int64_t H,
                                            int64_t W, int64_t OC, int64_t OH, int64_t OW, int64_t KH,
@@ -2686,11 +2722,31 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
                (int)OW, (int)sH, (int)sW, (int)pH, (int)pW, 1};
     hipStream_t s = repdl_stream(stream);
 
+    // A 1x1 kernel at a stride, no padding: the input positions it reads, gathered, are the input of the
+    // same layer at stride 1 -- same chains, same order, nothing skipped.  (The chain kernel on the
+    // strided rows took 47 clocks per step: 64 -> 128 at 56x56, batch 64, 0.99 ms; gathered 0.2x.)
+    if (KH == 1 && KW == 1 && (sH > 1 || sW > 1) && pH == 0 && pW == 0 && N * IC * OH * OW > 0 &&
+        repdl_cdiv(N * IC * OH * OW, 256) <= REPDL_I32_MAX)
+    {
+        const int64_t count = N * IC * OH * OW;
+        float *xs = nullptr;
+        hipError_t e = hipMallocAsync(reinterpret_cast<void **>(&xs), (size_t)count * sizeof(float), s);
+        if (e != hipSuccess)
+            return (int)e;
+        hipLaunchKernelGGL(conv_subsample_kernel, dim3((unsigned)repdl_cdiv(count, 256)), dim3(256), 0, s, input, xs, count, (int)H,
+                           (int)W, (int)OH, (int)OW, (int)sH, (int)sW);
+        int rc = repdl_launch_status();
+        if (rc == REPDL_OK)
+            rc = repdl_hip_conv2d_grad_kernel(grad_output, xs, grad_kernel, N, IC, OH, OW, OC, OH, OW, 1, 1, 1, 1, 0, 0, stream);
+        e = hipFreeAsync(xs, s);
+        return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
+    }
+
     // Many short chains: one matrix product (see wgrad_col_kernel).
     {
         const int64_t NC = IC * KH * KW, K = N * OH * OW;
         if (repdl_mfma_exact() && K > 0 && fits_i32(K) && fits_i32(NC) && K * NC < (1LL << 31) && K * OC < (1LL << 31) &&
-            wgrad_prefers_gemm(OC, NC, K))
+            wgrad_prefers_gemm(OC, NC, K, sW, OW, KH * KW))
         {
             const bool skips = pH > 0 || pW > 0;
             const size_t got_bytes = ((size_t)(K * OC) * sizeof(float) + 255) / 256 * 256;

@@ -176,6 +176,10 @@ WGRAD = [
     (4, 64, 7, 7, 512, 3, 3, 1, 1, 1, 1),    # many short chains: one matrix product over an im2col workspace
     (2, 128, 7, 7, 2048, 1, 1, 1, 1, 0, 0),  # the same, 1x1 without padding (nothing to fix up)
     (3, 64, 15, 15, 512, 3, 3, 2, 2, 1, 1),  # the same with strides
+    (3, 16, 30, 28, 32, 1, 1, 2, 2, 0, 0),   # 1x1 at stride 2: the input gathered, then the stride-1 layer (chain kernel)
+    (2, 8, 17, 23, 12, 1, 1, 3, 2, 0, 0),    # the same with different strides and ragged extents
+    (4, 128, 14, 14, 512, 1, 1, 2, 2, 0, 0), # the same, many short chains: gathered, then one matrix product
+    (2, 24, 28, 28, 96, 3, 3, 2, 2, 1, 1),   # 3x3 at stride 2, enough chains for several rounds of the chain kernel
 ]
 
 
