@@ -1789,6 +1789,25 @@ __global__ __launch_bounds__(256) void conv_subsample_kernel(const float *__rest
     Xs[idx] = X[(plane * H + (int64_t)oh * sH) * W + (int64_t)ow * sW];
 }
 
+// G[n][c][h][w] = G'[n][c][h / sH][w / sW] where a 1x1 kernel at a stride reads (h, w), +0 elsewhere:
+// the grad-input of that layer from the grad-input G' of the same layer at stride 1
+__global__ __launch_bounds__(256) void conv_upsample_kernel(const float *__restrict__ Gs, float *__restrict__ G, int64_t total,
+                                                            int H, int W, int OH, int OW, int sH, int sW)
+{
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total)
+        return;
+    const int w = (int)(idx % W);
+    const int64_t t = idx / W;
+    const int h = (int)(t % H);
+    const int64_t plane = t / H;
+    const int oh = h / sH, ow = w / sW;
+    float v = 0.0f;
+    if (oh * sH == h && ow * sW == w && oh < OH && ow < OW)
+        v = Gs[(plane * OH + oh) * OW + ow];
+    __builtin_nontemporal_store(v, &G[idx]);
+}
+
 // ---------------------------------------------------------------------------
 // Forward and grad-input of 3x3 kernels at stride 1 from an INPUT PATCH in LDS, both operands moved
 // from global memory straight into LDS (global_load_lds, see mm.hip), v_mfma_f32_16x16x4_f32.
@@ -2664,6 +2683,8 @@ REPDL_API int repdl_hip_conv2d_bias(const float *input, const float *kernel, con
     REPDL_REQUIRE(fits_i32(OH * sH + KH + pH) && fits_i32(OW * sW + KW + pW));
     ConvDims d{(int)N, (int)IC, (int)H, (int)W, (int)OC, (int)KH, (int)KW, (int)OH,
                (int)OW, (int)sH, (int)sW, (int)pH, (int)pW, (int)groups, bias};
+    // (A 1x1 kernel at a stride gains nothing from a gathered input here, unlike its two gradients: the
+    // implicit product below reads only the positions it needs; 64 -> 128 at 56x56, stride 2: 0.028 ms both ways.)
     // (3x3 kernels at stride 1 have a kernel of their own that is faster than the product also on small
     // images: 512 -> 512 at 7x7, batch 64, 0.26 -> 0.19 ms; at 10x10 0.48 -> 0.34)
     const bool tap = repdl_mfma_exact() && tapdma::applies<MODE_FWD>(d, input, kernel, 64, 1);
@@ -2687,6 +2708,28 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
     REPDL_REQUIRE(OC * OH * OW == 0 || (grad_output != nullptr && kernel != nullptr));
     REPDL_REQUIRE(fits_i32(H * W) && fits_i32(OH * OW) && fits_i32(OC * KH * KW) && fits_i32(N) && fits_i32(IC));
     REPDL_REQUIRE(fits_i32(H + pH + KH) && fits_i32(W + pW + KW) && fits_i32(IC * KH * KW * 4));
+    // A 1x1 kernel at a stride, no padding: the positions it reads take the grad-input of the same layer
+    // at stride 1 (same chains, same order), every other position an empty chain, +0.  (64 -> 128 at 56x56,
+    // stride 2, batch 64: 0.108 -> 0.059 ms; 256 -> 512 at 56x56: 0.65 -> 0.27.)
+    if (KH == 1 && KW == 1 && (sH > 1 || sW > 1) && pH == 0 && pW == 0 && OC * OH * OW > 0 &&
+        (OH - 1) * sH < H && (OW - 1) * sW < W && repdl_cdiv(total, 256) <= REPDL_I32_MAX)
+    {
+        hipStream_t s = repdl_stream(stream);
+        const int64_t count = N * IC * OH * OW;
+        float *gs = nullptr;
+        hipError_t e = hipMallocAsync(reinterpret_cast<void **>(&gs), (size_t)count * sizeof(float), s);
+        if (e != hipSuccess)
+            return (int)e;
+        int rc = repdl_hip_conv2d_grad_input(grad_output, kernel, gs, N, OC, OH, OW, IC, 1, 1, OH, OW, 1, 1, 0, 0, stream);
+        if (rc == REPDL_OK)
+        {
+            hipLaunchKernelGGL(conv_upsample_kernel, dim3((unsigned)repdl_cdiv(total, 256)), dim3(256), 0, s, gs, grad_input, total,
+                               (int)H, (int)W, (int)OH, (int)OW, (int)sH, (int)sW);
+            rc = repdl_launch_status();
+        }
+        e = hipFreeAsync(gs, s);
+        return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
+    }
     ConvDims d{(int)N, (int)IC, (int)H, (int)W, (int)OC, (int)KH, (int)KW, (int)OH,
                (int)OW, (int)sH, (int)sW, (int)pH, (int)pW, 1};
     const bool tap = repdl_mfma_exact() && OC * OH * OW > 0 && tapdma::applies<MODE_DGRAD>(d, grad_output, kernel, 64, 1);

@@ -58,6 +58,10 @@ FWD = [
     # 1x1 at stride 1 without padding, pixels in fours, channels in fours: a batch of matrix products per image
     (2, 96, 20, 20, 72, 1, 1, 1, 1, 0, 0, 1),      # 400 pixels, 72 rows forward (96 in grad-input): tile edges both ways
     (3, 128, 33, 40, 192, 1, 1, 1, 1, 0, 0, 1),    # chains of 128 (forward) and 192 (grad-input) terms
+    # 1x1 at a stride without padding: grad-input is the stride-1 layer's, scattered (forward: the implicit product)
+    (2, 64, 56, 56, 128, 1, 1, 2, 2, 0, 0, 1),     # 28x28 output: a batch of matrix products per image
+    (3, 16, 33, 41, 64, 1, 1, 2, 3, 0, 0, 1),      # different strides, 17x14 output, rows and columns past the last tap
+    (2, 8, 10, 9, 24, 1, 1, 4, 4, 0, 0, 1),        # 3x3 output, stride wider than half the image
     (1, 68, 6, 6, 20, 1, 1, 1, 1, 0, 0, 1),        # one small image: a k-tile tail of one quad, 20 rows
     (5, 24, 8, 12, 36, 1, 1, 1, 1, 0, 0, 1),       # chains shorter than a k-tile
 ]
