@@ -1445,12 +1445,14 @@ __global__ __launch_bounds__(256) void conv_wgrad_kernel(const float *__restrict
 // conv_wgrad_kernel.
 // ---------------------------------------------------------------------------
 typedef float f4v __attribute__((ext_vector_type(4)));
-constexpr int MW_GS = 16; // float4 staging slots of grad_output per staging thread
+constexpr int MW_GS = 32; // most float4 staging slots of grad_output per staging thread
 constexpr int MW_XS = 8;  // most float4 staging slots of input per staging thread
 constexpr int MW_OC = 32; // oc per workgroup
 constexpr int MW_ST = 128; // staging threads
 
-template <int QP, bool UNIT, int XS> // QP: instructions per piece; XS: input staging slots per thread
+// QP: instructions per piece; XS, GS: staging slots per thread (input, grad_output); XV: the staged input
+// rows are 16-byte aligned in LDS (1x1 kernels without padding: see the launcher)
+template <int QP, bool UNIT, int XS, int GS, bool XV>
 __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__restrict__ GOs, // grad_output, rows of 4*QP*NP floats
                                                               const float *__restrict__ Xs,  // input, rows of xW floats
                                                               const float *__restrict__ GO,  // both as given (epilogue)
@@ -1498,10 +1500,10 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
         }
         // grad_output: slot = (oc, 4 consecutive steps of the chunk)
         const int spo = (R * OWp) >> 2; // float4 per oc and chunk
-        uint32_t g_goff[MW_GS];
-        int g_loff[MW_GS];
+        uint32_t g_goff[GS];
+        int g_loff[GS];
 #pragma unroll
-        for (int i = 0; i < MW_GS; i++)
+        for (int i = 0; i < GS; i++)
         {
             int s = st + MW_ST * i;
             s = s < MW_OC * spo ? s : MW_OC * spo - 1;
@@ -1510,40 +1512,56 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
             g_goff[i] = (uint32_t)((oc - oc0) * d.OH * OWp + t) * 4u;
             g_loff[i] = 64 + o * GP + t;
         }
-        f4v xst[XS], gst[MW_GS]; // plain vectors: they must stay in registers
+        f4v xst[XS], gst[GS]; // plain vectors: they must stay in registers
+        // Bit i: slot i of the chunk in xst is a row of the image (else a row of padding: zeros).  The
+        // zeros go in when the slot is stored, a chunk later: a select on the loaded value at the load
+        // makes the wave wait for the load it has just issued, in front of the barrier the computing
+        // waves are waiting at (3x3, 64 -> 64 at 56x56, batch 64: 0.99 -> 0.955 ms).
+        // (A second set of staging registers, the loads issued two chunks ahead of their store, was
+        // slower: 1.03 ms.  Memory latency is not what the chunks wait for.)
+        unsigned x_ok = 0;
         auto chunk_load = [&](int n, int oh0) {
             const float *Xn = Xs + (int64_t)n * d.IC * d.H * xW;
             const int hbase = oh0 * d.sH - d.pH;
+            x_ok = 0;
 #pragma unroll
             for (int i = 0; i < XS; i++)
-                {
-                    const int h = hbase + x_hr[i];
-                    const bool ok = h >= 0 && h < d.H;
-                    const int hc = h < 0 ? 0 : (h >= d.H ? d.H - 1 : h);
-                    const f4v v = *reinterpret_cast<const f4v *>(Xn + x_goff[i] + hc * xW);
-                    xst[i][0] = ok ? v[0] : 0.0f;
-                    xst[i][1] = ok ? v[1] : 0.0f;
-                    xst[i][2] = ok ? v[2] : 0.0f;
-                    xst[i][3] = ok ? v[3] : 0.0f;
-                }
+            {
+                const int h = hbase + x_hr[i];
+                const bool ok = h >= 0 && h < d.H;
+                const int hc = h < 0 ? 0 : (h >= d.H ? d.H - 1 : h);
+                xst[i] = *reinterpret_cast<const f4v *>(Xn + x_goff[i] + hc * xW);
+                x_ok |= ok ? 1u << i : 0u;
+            }
             const char *Gn = reinterpret_cast<const char *>(GOs + (((int64_t)n * d.OC + oc0) * d.OH + oh0) * OWp);
 #pragma unroll
-            for (int i = 0; i < MW_GS; i++)
+            for (int i = 0; i < GS; i++)
                 gst[i] = *reinterpret_cast<const f4v *>(Gn + g_goff[i]);
         };
         auto stage_store = [&](int buf) {
             float *base = lds + buf * bufsz;
 #pragma unroll
             for (int i = 0; i < XS; i++)
+            {
+                float *p = base + x_loff[i];
+                const bool ok = (x_ok >> i) & 1u;
+                f4v v;
+                v[0] = ok ? xst[i][0] : 0.0f;
+                v[1] = ok ? xst[i][1] : 0.0f;
+                v[2] = ok ? xst[i][2] : 0.0f;
+                v[3] = ok ? xst[i][3] : 0.0f;
+                if (XV)
+                    *reinterpret_cast<f4v *>(p) = v;
+                else
                 {
-                    float *p = base + x_loff[i];
-                    p[0] = xst[i][0];
-                    p[1] = xst[i][1];
-                    p[2] = xst[i][2];
-                    p[3] = xst[i][3];
+                    p[0] = v[0];
+                    p[1] = v[1];
+                    p[2] = v[2];
+                    p[3] = v[3];
                 }
+            }
 #pragma unroll
-            for (int i = 0; i < MW_GS; i++)
+            for (int i = 0; i < GS; i++)
                 *reinterpret_cast<f4v *>(base + g_loff[i]) = gst[i];
         };
         int n1 = 0, oh1 = 0; // the chunk the next chunk_load fetches
@@ -2846,11 +2864,20 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
         const int64_t reach = (OWp - 1) * sW + KW; // the taps of the padded steps must be staged zeros
         if (reach > Wp)
             Wp = reach;
-        while (Wp % 32 != KW % 32)
+        // A 1x1 kernel without padding: the 16 columns of a block are 16 channels, and lane l reads word
+        // CP * (l % 16) + l / 16 of the staged input -- every bank once with CP = 4 mod 32, like
+        // grad_output -- so the rows can sit on 16-byte boundaries and be stored four words at a time
+        // (the staging waves set the pace of these layers: 256 -> 64 at 56x56, batch 64, 0.97 -> ... ms).
+        const bool xv = KHW == 1 && pW == 0 && sW == 1;
+        while (xv ? Wp % 4 != 0 : Wp % 32 != KW % 32)
             Wp++;
         const int64_t span = (15 + KHW - 1) / KHW + 1; // channels a 16-column block can span
         const int64_t nic_max = span < IC ? span : IC;
         const int64_t nw4 = (W + 3) / 4;
+        // grad_output slots per staging thread: 32 let a chunk of a 3x3 layer at stride 1 be twice as long
+        // (64 -> 64 at 56x56, batch 64: 0.955 -> 0.90 ms); where the input slots or LDS set the length
+        // of a chunk anyway, 16 (twice the slots repeat the loads and stores: 1x1, 0.97 -> 1.44 ms)
+        const int64_t gs_max = sW == 1 && !xv ? MW_GS : 16;
         int64_t R = 0, hrows = 0, GP = 0, CP = 0;
         for (int64_t r = OH; r >= 1 && QP > 0; r--)
         {
@@ -2861,9 +2888,9 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
             while (gp % 32 != 4)
                 gp++;
             int64_t cp = hr * Wp;
-            while (cp % 32 != KHW % 32)
+            while (cp % 32 != (xv ? 4 : KHW % 32))
                 cp++;
-            if (MW_OC * r * OWp <= 4 * MW_ST * MW_GS && nic_max * hr * nw4 <= MW_ST * MW_XS &&
+            if (MW_OC * r * OWp <= 4 * MW_ST * gs_max && nic_max * hr * nw4 <= MW_ST * MW_XS &&
                 2 * (64 + MW_OC * gp + nic_max * cp + sH * Wp + 64 + 3) * 4 <= 150 * 1024)
             {
                 R = r;
@@ -2922,31 +2949,40 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
             if (shmem < 84 * 1024)
                 shmem = 84 * 1024; // one workgroup per CU: every wave has a SIMD to itself
             const bool few = nic_max * hrows * nw4 <= 2 * MW_ST; // input slots per staging thread: 2 or MW_XS
-#define REPDL_WGRAD_MFMA(Q, U, X)                                                                                    \
+            const bool wide = MW_OC * R * OWp > 4 * MW_ST * 16;  // grad_output slots per staging thread: MW_GS or 16
+#define REPDL_WGRAD_MFMA(Q, U, X, G, V)                                                                                 \
     do                                                                                                              \
     {                                                                                                               \
-        hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_wgrad_mfma_kernel<Q, U, X>),       \
+        hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_wgrad_mfma_kernel<Q, U, X, G, V>),       \
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);                \
         if (e_ != hipSuccess)                                                                                       \
         {                                                                                                           \
             (void)hipFreeAsync(ws, s);                                                                              \
             return (int)e_;                                                                                         \
         }                                                                                                           \
-        hipLaunchKernelGGL((conv_wgrad_mfma_kernel<Q, U, X>), dim3((unsigned)gx, (unsigned)gy), dim3(256), shmem, s, \
+        hipLaunchKernelGGL((conv_wgrad_mfma_kernel<Q, U, X, G, V>), dim3((unsigned)gx, (unsigned)gy), dim3(256), shmem, s, \
                            gsrc, xsrc, grad_output, input, grad_kernel, d, (int)R, (int)NP, (int)GP, (int)Wp,       \
                            (int)CP, (int)hrows, (int)xoff, (int)bufsz, (int)xW, guard);                             \
     } while (0)
 #define REPDL_WGRAD_MFMA_Q(Q)                     \
     do                                            \
     {                                             \
-        if (sW == 1 && few)                       \
-            REPDL_WGRAD_MFMA(Q, true, 2);         \
-        else if (sW == 1)                         \
-            REPDL_WGRAD_MFMA(Q, true, MW_XS);     \
-        else if (few)                             \
-            REPDL_WGRAD_MFMA(Q, false, 2);        \
-        else                                      \
-            REPDL_WGRAD_MFMA(Q, false, MW_XS);    \
+        if (xv && few)                                  \
+            REPDL_WGRAD_MFMA(Q, true, 2, 16, true);         \
+        else if (xv)                                    \
+            REPDL_WGRAD_MFMA(Q, true, MW_XS, 16, true);     \
+        else if (sW == 1 && few && wide)                \
+            REPDL_WGRAD_MFMA(Q, true, 2, MW_GS, false);     \
+        else if (sW == 1 && wide)                       \
+            REPDL_WGRAD_MFMA(Q, true, MW_XS, MW_GS, false); \
+        else if (sW == 1 && few)                        \
+            REPDL_WGRAD_MFMA(Q, true, 2, 16, false);        \
+        else if (sW == 1)                               \
+            REPDL_WGRAD_MFMA(Q, true, MW_XS, 16, false);    \
+        else if (few)                                   \
+            REPDL_WGRAD_MFMA(Q, false, 2, 16, false);       \
+        else                                            \
+            REPDL_WGRAD_MFMA(Q, false, MW_XS, 16, false);   \
     } while (0)
             if (QP == 16)
                 REPDL_WGRAD_MFMA_Q(16);
