@@ -1450,9 +1450,12 @@ constexpr int MW_XS = 8;  // most float4 staging slots of input per staging thre
 constexpr int MW_OC = 32; // oc per workgroup
 constexpr int MW_ST = 128; // staging threads
 
-// QP: instructions per piece; XS, GS: staging slots per thread (input, grad_output); XV: the staged input
-// rows are 16-byte aligned in LDS (1x1 kernels without padding: see the launcher)
-template <int QP, bool UNIT, int XS, int GS, bool XV>
+// QP: instructions per piece; SW: the stride along a row, 0 when it is neither 1 nor 2 (the taps of a piece
+// then sit at offsets the instructions cannot carry: an addition per read, and no two words per read --
+// 7x7 at stride 2, 3 -> 64 at 224x224, took 18 clocks per step that way); XS, GS: staging slots per thread
+// (input, grad_output); XV: the staged input rows are 16-byte aligned in LDS (1x1 kernels without padding:
+// see the launcher)
+template <int QP, int SW, int XS, int GS, bool XV>
 __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__restrict__ GOs, // grad_output, rows of 4*QP*NP floats
                                                               const float *__restrict__ Xs,  // input, rows of xW floats
                                                               const float *__restrict__ GO,  // both as given (epilogue)
@@ -1609,7 +1612,7 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
     const int rem = colc - ic * KHW;
     const int kh = rem / d.KW, kw = rem - kh * d.KW;
     const int q = lane >> 4;
-    const int sW = UNIT ? 1 : d.sW;
+    const int sW = SW > 0 ? SW : d.sW;
     const int a_lane = 64 + (wave * 16 + (lane & 15)) * GP + q; // 64 zero words lead each buffer
     const int x_lane = xoff + (ic - ic_first) * CP + kh * Wp + kw + q * sW;
     const int npieces = R * NP;
@@ -1785,7 +1788,7 @@ inline bool wgrad_prefers_gemm(int64_t OC, int64_t NC, int64_t K, int64_t sW, in
     const double clk = 1.0 / 2.35e9;
     const double rounds = (double)repdl_cdiv(repdl_cdiv(NC, 16) * repdl_cdiv(OC, 32), 256);
     const int64_t OWr = (OW + 3) / 4 * 4;
-    const double step = (double)K * (sW > 1 ? 18.0 : 12.0) * (OWr < 16 ? 16.0 / (double)OWr : 1.0) * clk;
+    const double step = (double)K * (sW > 2 ? 18.0 : 12.5) * (OWr < 16 ? 16.0 / (double)OWr : 1.0) * clk;
     const double t_chain = (rounds < 1.0 ? 1.0 : rounds) * (step + (KHW == 1 ? 90e-6 : 34e-6));
     const double flop = 2.0 * (double)OC * (double)NC * (double)K;
     const double t_mm = flop / 100e12 > (double)K * 20.0 * clk ? flop / 100e12 : (double)K * 20.0 * clk;
@@ -2968,21 +2971,25 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
     do                                            \
     {                                             \
         if (xv && few)                                  \
-            REPDL_WGRAD_MFMA(Q, true, 2, 16, true);         \
+            REPDL_WGRAD_MFMA(Q, 1, 2, 16, true);            \
         else if (xv)                                    \
-            REPDL_WGRAD_MFMA(Q, true, MW_XS, 16, true);     \
+            REPDL_WGRAD_MFMA(Q, 1, MW_XS, 16, true);        \
         else if (sW == 1 && few && wide)                \
-            REPDL_WGRAD_MFMA(Q, true, 2, MW_GS, false);     \
+            REPDL_WGRAD_MFMA(Q, 1, 2, MW_GS, false);        \
         else if (sW == 1 && wide)                       \
-            REPDL_WGRAD_MFMA(Q, true, MW_XS, MW_GS, false); \
+            REPDL_WGRAD_MFMA(Q, 1, MW_XS, MW_GS, false);    \
         else if (sW == 1 && few)                        \
-            REPDL_WGRAD_MFMA(Q, true, 2, 16, false);        \
+            REPDL_WGRAD_MFMA(Q, 1, 2, 16, false);           \
         else if (sW == 1)                               \
-            REPDL_WGRAD_MFMA(Q, true, MW_XS, 16, false);    \
+            REPDL_WGRAD_MFMA(Q, 1, MW_XS, 16, false);       \
+        else if (sW == 2 && few)                        \
+            REPDL_WGRAD_MFMA(Q, 2, 2, 16, false);           \
+        else if (sW == 2)                               \
+            REPDL_WGRAD_MFMA(Q, 2, MW_XS, 16, false);       \
         else if (few)                                   \
-            REPDL_WGRAD_MFMA(Q, false, 2, 16, false);       \
+            REPDL_WGRAD_MFMA(Q, 0, 2, 16, false);           \
         else                                            \
-            REPDL_WGRAD_MFMA(Q, false, MW_XS, 16, false);   \
+            REPDL_WGRAD_MFMA(Q, 0, MW_XS, 16, false);       \
     } while (0)
             if (QP == 16)
                 REPDL_WGRAD_MFMA_Q(16);
