@@ -1500,9 +1500,11 @@ static int spec_rounds(int64_t rows, int64_t n)
     // 0.37), chains that drift lose the rounds' fifteen launches (0.09 -> 0.14 ms).  At 200704 elements
     // (64 channels of 64 images of 56x56) gain and loss are the same 0.1 ms (0.50 -> 0.33 against 0.08 ->
     // 0.18) and a residual block with BatchNorm got 3 % slower with the rounds: not there.  256 x 262144
-    // (4096 nodes) got slower either way.
+    // (4096 nodes) got slower either way; 64 x 802816 (3136 nodes: the first BatchNorm of a ResNet at batch 64)
+    // 1.37 -> 0.69 ms zero-mean, 0.21 -> 0.33 drifting.  (Rounds from 2^17 elements made a ResNet-18 training step at
+    // batch 64 five milliseconds slower, 49 -> 54.7: they fill the chip that the other streams' kernels would use.)
     if (rows > 1)
-        return (n >= ((int64_t)1 << 19) && rows * repdl_cdiv(repdl_cdiv(n, BLK), NODEB) <= 2048) ? 3 : 0;
+        return (n >= ((int64_t)1 << 19) && rows * repdl_cdiv(repdl_cdiv(n, BLK), NODEB) <= 3200) ? 3 : 0;
     if (n < ((int64_t)1 << 22))
         return 0;
     return n < ((int64_t)1 << 24) ? 4 : (n < ((int64_t)1 << 26) ? 8 : MAX_ROUNDS);

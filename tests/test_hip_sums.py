@@ -267,6 +267,13 @@ def test_rounds_on_chains_in_rows():
     m2 = torch.from_numpy(np.stack([r.standard_normal((1 << 23) + 77), r.random((1 << 23) + 77) - 0.5]).astype(np.float32))
     got = ops.sum2d_dim1(m2.cuda()).cpu()
     assert torch.equal(got.view(torch.int32), oracle.sum2d_dim1(m2).view(torch.int32))
+    # seventy rows of 33 nodes each: 2310 nodes, more than one pass of the round's walkers
+    m3 = torch.from_numpy(r.standard_normal((70, (1 << 19) + 5)).astype(np.float32))
+    m3[::7] += 0.25
+    m3[3] *= 2.0**40
+    got = ops.sum2d_dim1(m3.cuda()).cpu()
+    assert torch.equal(got.view(torch.int32), oracle.sum2d_dim1(m3).view(torch.int32))
+    del m3
     # channel sums: 8 channels of 48 images of 112x112 (602112 elements per chain), zero-mean and shifted channels
     x = torch.from_numpy(r.standard_normal((48, 8, 112, 112)).astype(np.float32))
     x[:, 3] += 0.5
