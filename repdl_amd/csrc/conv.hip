@@ -2790,7 +2790,7 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
     // same layer at stride 1 -- same chains, same order, nothing skipped.  (The chain kernel on the
     // strided rows took 47 clocks per step: 64 -> 128 at 56x56, batch 64, 0.99 ms; gathered 0.2x.)
     if (KH == 1 && KW == 1 && (sH > 1 || sW > 1) && pH == 0 && pW == 0 && N * IC * OH * OW > 0 &&
-        repdl_cdiv(N * IC * OH * OW, 256) <= REPDL_I32_MAX)
+        (OH - 1) * sH < H && (OW - 1) * sW < W && repdl_cdiv(N * IC * OH * OW, 256) <= REPDL_I32_MAX)
     {
         const int64_t count = N * IC * OH * OW;
         float *xs = nullptr;
