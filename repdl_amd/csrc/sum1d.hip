@@ -902,7 +902,11 @@ __device__ __forceinline__ uint32_t nearest_candidate(uint32_t yb, uint32_t base
 __device__ __forceinline__ uint32_t window_base(uint32_t centre)
 {
     const uint32_t lo = centre & 0xFF800000u, hi = centre | 0x007FFFFFu;
-    uint32_t base = centre - lo < (uint32_t)(CAND / 2) ? lo : centre - (uint32_t)(CAND / 2);
+    // The window starts on a multiple of WGRID states (lo is one), the centre 96 to 159 states in: a
+    // centre that moves by a few states from one round to the next keeps its window, and the node its
+    // table (2^28 zero-mean values: 2.47 -> 2.40 ms).
+    constexpr uint32_t WGRID = 64;
+    uint32_t base = centre - lo < (uint32_t)(CAND / 2) ? lo : (centre - (uint32_t)(CAND / 2) + WGRID / 2) & ~(WGRID - 1);
     if (hi - base < (uint32_t)(CAND - 1))
         base = hi - (uint32_t)(CAND - 1);
     return base;
