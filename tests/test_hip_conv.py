@@ -62,6 +62,8 @@ FWD = [
     (2, 64, 56, 56, 128, 1, 1, 2, 2, 0, 0, 1),     # 28x28 output: a batch of matrix products per image
     (3, 16, 33, 41, 64, 1, 1, 2, 3, 0, 0, 1),      # different strides, 17x14 output, rows and columns past the last tap
     (2, 8, 10, 9, 24, 1, 1, 4, 4, 0, 0, 1),        # 3x3 output, stride wider than half the image
+    (2, 8, 9, 20, 16, 1, 1, 1, 2, 0, 0, 1),        # a stride along the rows only
+    (2, 8, 20, 9, 16, 1, 1, 3, 1, 0, 0, 1),        # ... down the columns only
     (1, 68, 6, 6, 20, 1, 1, 1, 1, 0, 0, 1),        # one small image: a k-tile tail of one quad, 20 rows
     (5, 24, 8, 12, 36, 1, 1, 1, 1, 0, 0, 1),       # chains shorter than a k-tile
 ]
@@ -182,6 +184,8 @@ WGRAD = [
     (3, 64, 15, 15, 512, 3, 3, 2, 2, 1, 1),  # the same with strides
     (3, 16, 30, 28, 32, 1, 1, 2, 2, 0, 0),   # 1x1 at stride 2: the input gathered, then the stride-1 layer (chain kernel)
     (2, 8, 17, 23, 12, 1, 1, 3, 2, 0, 0),    # the same with different strides and ragged extents
+    (2, 8, 9, 20, 16, 1, 1, 1, 2, 0, 0),     # a stride along the rows only
+    (2, 8, 20, 9, 16, 1, 1, 3, 1, 0, 0),     # ... down the columns only
     (4, 128, 14, 14, 512, 1, 1, 2, 2, 0, 0), # the same, many short chains: gathered, then one matrix product
     (2, 24, 28, 28, 96, 3, 3, 2, 2, 1, 1),   # 3x3 at stride 2, enough chains for several rounds of the chain kernel
 ]
