@@ -1717,33 +1717,29 @@ __global__ __launch_bounds__(256) void conv_wgrad_mfma_kernel(const float *__res
 __global__ __launch_bounds__(256) void wgrad_got_kernel(const float *__restrict__ GO, float *__restrict__ GOt, int64_t total,
                                                         int OC, int OHW)
 {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; // = k * OC + oc
-    if (idx >= total)
+    // (the launcher takes this route only below 2^31 elements: 32-bit divisions, a fraction of the cost of 64-bit ones)
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x; // = k * OC + oc
+    if ((int64_t)idx >= total)
         return;
-    const int oc = (int)(idx % OC);
-    const int64_t k = idx / OC;
-    const int64_t n = k / OHW;
-    const int p = (int)(k - n * OHW);
-    GOt[idx] = GO[(n * OC + oc) * OHW + p];
+    const uint32_t k = idx / (uint32_t)OC, oc = idx - k * (uint32_t)OC;
+    const uint32_t n = k / (uint32_t)OHW, p = k - n * (uint32_t)OHW;
+    GOt[idx] = GO[((int64_t)n * OC + oc) * OHW + p];
 }
 
 __global__ __launch_bounds__(256) void wgrad_col_kernel(const float *__restrict__ X, float *__restrict__ col, int64_t total,
                                                         ConvDims d, int NC)
 {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; // = k * NC + (ic, kh, kw)
-    if (idx >= total)
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x; // = k * NC + (ic, kh, kw); below 2^31, as above
+    if ((int64_t)idx >= total)
         return;
-    const int c = (int)(idx % NC);
-    const int64_t k = idx / NC;
-    const int KHW = d.KH * d.KW;
-    const int ic = c / KHW, rem = c - ic * KHW;
-    const int kh = rem / d.KW, kw = rem - kh * d.KW;
-    const int ow = (int)(k % d.OW);
-    const int64_t t = k / d.OW;
-    const int oh = (int)(t % d.OH);
-    const int64_t n = t / d.OH;
-    const int h = oh * d.sH - d.pH + kh, w = ow * d.sW - d.pW + kw;
-    col[idx] = (h >= 0 && h < d.H && w >= 0 && w < d.W) ? X[((n * d.IC + ic) * d.H + h) * d.W + w] : 0.0f;
+    const uint32_t k = idx / (uint32_t)NC, c = idx - k * (uint32_t)NC;
+    const uint32_t KHW = (uint32_t)(d.KH * d.KW);
+    const uint32_t ic = c / KHW, rem = c - ic * KHW;
+    const uint32_t kh = rem / (uint32_t)d.KW, kw = rem - kh * (uint32_t)d.KW;
+    const uint32_t t = k / (uint32_t)d.OW, ow = k - t * (uint32_t)d.OW;
+    const uint32_t n = t / (uint32_t)d.OH, oh = t - n * (uint32_t)d.OH;
+    const int h = (int)oh * d.sH - d.pH + (int)kh, w = (int)ow * d.sW - d.pW + (int)kw;
+    col[idx] = (h >= 0 && h < d.H && w >= 0 && w < d.W) ? X[(((int64_t)n * d.IC + ic) * d.H + h) * d.W + w] : 0.0f;
 }
 
 __global__ __launch_bounds__(256) void wgrad_fixup_kernel(const float *__restrict__ GO, const float *__restrict__ X,
