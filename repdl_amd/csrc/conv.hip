@@ -1793,35 +1793,38 @@ inline bool wgrad_prefers_gemm(int64_t OC, int64_t NC, int64_t K, int64_t sW, in
 }
 
 // X'[n][c][oh][ow] = X[n][c][oh * sH][ow * sW]: what a 1x1 kernel at a stride reads of its input
+// (I: uint32_t where the tensors have fewer than 2^31 elements -- 64-bit divisions cost several times more)
+template <typename I>
 __global__ __launch_bounds__(256) void conv_subsample_kernel(const float *__restrict__ X, float *__restrict__ Xs, int64_t total,
                                                              int H, int W, int OH, int OW, int sH, int sW)
 {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= total)
+    const I idx = (I)blockIdx.x * 256 + threadIdx.x;
+    if ((int64_t)idx >= total)
         return;
-    const int ow = (int)(idx % OW);
-    const int64_t t = idx / OW;
-    const int oh = (int)(t % OH);
-    const int64_t plane = t / OH;
-    Xs[idx] = X[(plane * H + (int64_t)oh * sH) * W + (int64_t)ow * sW];
+    const I t = idx / (I)OW;
+    const int ow = (int)(idx - t * (I)OW);
+    const I plane = t / (I)OH;
+    const int oh = (int)(t - plane * (I)OH);
+    Xs[idx] = X[((int64_t)plane * H + (int64_t)oh * sH) * W + (int64_t)ow * sW];
 }
 
 // G[n][c][h][w] = G'[n][c][h / sH][w / sW] where a 1x1 kernel at a stride reads (h, w), +0 elsewhere:
 // the grad-input of that layer from the grad-input G' of the same layer at stride 1
+template <typename I>
 __global__ __launch_bounds__(256) void conv_upsample_kernel(const float *__restrict__ Gs, float *__restrict__ G, int64_t total,
                                                             int H, int W, int OH, int OW, int sH, int sW)
 {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= total)
+    const I idx = (I)blockIdx.x * 256 + threadIdx.x;
+    if ((int64_t)idx >= total)
         return;
-    const int w = (int)(idx % W);
-    const int64_t t = idx / W;
-    const int h = (int)(t % H);
-    const int64_t plane = t / H;
+    const I t = idx / (I)W;
+    const int w = (int)(idx - t * (I)W);
+    const I plane = t / (I)H;
+    const int h = (int)(t - plane * (I)H);
     const int oh = h / sH, ow = w / sW;
     float v = 0.0f;
     if (oh * sH == h && ow * sW == w && oh < OH && ow < OW)
-        v = Gs[(plane * OH + oh) * OW + ow];
+        v = Gs[((int64_t)plane * OH + oh) * OW + ow];
     __builtin_nontemporal_store(v, &G[idx]);
 }
 
@@ -2551,19 +2554,20 @@ template <int MODE>
 __global__ __launch_bounds__(256) void conv_col_kernel(const float *__restrict__ G, float *__restrict__ col, int64_t total,
                                                        ConvDims d, int K)
 {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; // = row * K + k
-    if (idx >= total)
+    // (conv_prefers_mm keeps this route below 2^31 elements: 32-bit divisions)
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x; // = row * K + k
+    if ((int64_t)idx >= total)
         return;
-    const int k = (int)(idx % K);
-    const int64_t row = idx / K;
+    const uint32_t row = idx / (uint32_t)K;
+    const int k = (int)(idx - row * (uint32_t)K);
     const int KHW = d.KH * d.KW;
     const int c = k / KHW, rem = k - c * KHW;
     const int kh = rem / d.KW, kw = rem - kh * d.KW;
-    const int PW = MODE == MODE_FWD ? d.OW : d.W, PH = MODE == MODE_FWD ? d.OH : d.H;
-    const int pw = (int)(row % PW);
-    const int64_t t = row / PW;
-    const int ph = (int)(t % PH);
+    const uint32_t PW = (uint32_t)(MODE == MODE_FWD ? d.OW : d.W), PH = (uint32_t)(MODE == MODE_FWD ? d.OH : d.H);
+    const uint32_t t = row / PW;
+    const int pw = (int)(row - t * PW);
     const int64_t n = t / PH;
+    const int ph = (int)(t - (uint32_t)n * PH);
     float v = 0.0f;
     if (MODE == MODE_FWD)
     {
@@ -2598,15 +2602,15 @@ __global__ __launch_bounds__(256) void conv_mm_out_kernel(const float *__restric
                                                           const float *__restrict__ Wt, float *__restrict__ Out, ConvDims d,
                                                           int64_t total, const unsigned *__restrict__ guard)
 {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; // NCHW index of the output
-    if (idx >= total)
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x; // NCHW index of the output (below 2^31, as above)
+    if ((int64_t)idx >= total)
         return;
     const int P = MODE == MODE_FWD ? d.OH * d.OW : d.H * d.W, PW = MODE == MODE_FWD ? d.OW : d.W;
     const int M = MODE == MODE_FWD ? d.OC : d.IC;
-    const int p = (int)(idx % P);
-    const int64_t t = idx / P;
-    const int ch = (int)(t % M);
-    const int64_t n = t / M;
+    const uint32_t t = idx / (uint32_t)P;
+    const int p = (int)(idx - t * (uint32_t)P);
+    const int64_t n = t / (uint32_t)M;
+    const int ch = (int)(t - (uint32_t)n * (uint32_t)M);
     float v = C[(n * P + p) * M + ch];
     if (guard_suspect(v, guard_tiny(guard)))
     {
@@ -2740,8 +2744,12 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
         int rc = repdl_hip_conv2d_grad_input(grad_output, kernel, gs, N, OC, OH, OW, IC, 1, 1, OH, OW, 1, 1, 0, 0, stream);
         if (rc == REPDL_OK)
         {
-            hipLaunchKernelGGL(conv_upsample_kernel, dim3((unsigned)repdl_cdiv(total, 256)), dim3(256), 0, s, gs, grad_input, total,
-                               (int)H, (int)W, (int)OH, (int)OW, (int)sH, (int)sW);
+            if (total < (1LL << 31))
+                hipLaunchKernelGGL(conv_upsample_kernel<uint32_t>, dim3((unsigned)repdl_cdiv(total, 256)), dim3(256), 0, s, gs, grad_input,
+                                   total, (int)H, (int)W, (int)OH, (int)OW, (int)sH, (int)sW);
+            else
+                hipLaunchKernelGGL(conv_upsample_kernel<int64_t>, dim3((unsigned)repdl_cdiv(total, 256)), dim3(256), 0, s, gs, grad_input,
+                                   total, (int)H, (int)W, (int)OH, (int)OW, (int)sH, (int)sW);
             rc = repdl_launch_status();
         }
         e = hipFreeAsync(gs, s);
@@ -2793,8 +2801,12 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
         hipError_t e = hipMallocAsync(reinterpret_cast<void **>(&xs), (size_t)count * sizeof(float), s);
         if (e != hipSuccess)
             return (int)e;
-        hipLaunchKernelGGL(conv_subsample_kernel, dim3((unsigned)repdl_cdiv(count, 256)), dim3(256), 0, s, input, xs, count, (int)H,
-                           (int)W, (int)OH, (int)OW, (int)sH, (int)sW);
+        if (N * IC * H * W < (1LL << 31))
+            hipLaunchKernelGGL(conv_subsample_kernel<uint32_t>, dim3((unsigned)repdl_cdiv(count, 256)), dim3(256), 0, s, input, xs, count,
+                               (int)H, (int)W, (int)OH, (int)OW, (int)sH, (int)sW);
+        else
+            hipLaunchKernelGGL(conv_subsample_kernel<int64_t>, dim3((unsigned)repdl_cdiv(count, 256)), dim3(256), 0, s, input, xs, count,
+                               (int)H, (int)W, (int)OH, (int)OW, (int)sH, (int)sW);
         int rc = repdl_launch_status();
         if (rc == REPDL_OK)
             rc = repdl_hip_conv2d_grad_kernel(grad_output, xs, grad_kernel, N, IC, OH, OW, OC, OH, OW, 1, 1, 1, 1, 0, 0, stream);
