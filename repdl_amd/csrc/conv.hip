@@ -1828,6 +1828,40 @@ __global__ __launch_bounds__(256) void conv_upsample_kernel(const float *__restr
     __builtin_nontemporal_store(v, &G[idx]);
 }
 
+// Strided grad-input by phases.  Input position h takes the taps kh with (h + pH - kh) a multiple of sH,
+// that is kh = r + a * sH with r = (h + pH) % sH: the positions of one residue pair (rh, rw) are the
+// grad-input of a STRIDE-1 layer without padding whose kernel is the taps of that residue,
+//     G'[n][ic][h'][w'] = sum over (oc, a, b) of GO[n][oc][h' - a][w' - b] * Ws[oc][ic][a][b],
+//     Ws[oc][ic][a][b] = W[oc][ic][rh + a * sH][rw + b * sW],   h = sH * h' + rh - pH,
+// with (oc, a, b) ascending exactly the reference's (oc, kh, kw) over the taps that count.  No product
+// with a zero of a dilated grad_output: a quarter of the work at stride 2.
+__global__ __launch_bounds__(256) void conv_phase_kernel_kernel(const float *__restrict__ Wk, float *__restrict__ Ws, int total, int KH,
+                                                                int KW, int A, int B, int rh, int rw, int sH, int sW)
+{
+    const int idx = blockIdx.x * 256 + threadIdx.x; // = (oc * IC + ic) * A * B + a * B + b
+    if (idx >= total)
+        return;
+    const int b = idx % B, t = idx / B;
+    const int a = t % A, plane = t / A;
+    Ws[idx] = Wk[((int64_t)plane * KH + rh + a * sH) * KW + rw + b * sW];
+}
+
+// G[n][ic][sH * h' + rh - pH][sW * w' + rw - pW] = Gp[n][ic][h'][w'] (Gp == nullptr: +0, a residue without taps)
+__global__ __launch_bounds__(256) void conv_phase_scatter_kernel(const float *__restrict__ Gp, float *__restrict__ G, int64_t total, int HP,
+                                                                 int WP, int H, int W, int sH, int sW, int oh0, int ow0)
+{
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; // index into Gp: (plane, h', w')
+    if (idx >= total)
+        return;
+    const int wp = (int)(idx % WP);
+    const int64_t t = idx / WP;
+    const int hp = (int)(t % HP);
+    const int64_t plane = t / HP;
+    const int h = sH * hp + oh0, w = sW * wp + ow0;
+    if (h >= 0 && h < H && w >= 0 && w < W)
+        G[(plane * H + h) * W + w] = Gp != nullptr ? Gp[idx] : 0.0f;
+}
+
 // ---------------------------------------------------------------------------
 // Forward and grad-input of 3x3 kernels at stride 1 from an INPUT PATCH in LDS, both operands moved
 // from global memory straight into LDS (global_load_lds, see mm.hip), v_mfma_f32_16x16x4_f32.
@@ -2753,6 +2787,55 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
             rc = repdl_launch_status();
         }
         e = hipFreeAsync(gs, s);
+        return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
+    }
+    // Strides, and enough work to pay for a dozen launches (3 GFLOP of products that count): residue by residue,
+    // see conv_phase_kernel_kernel.  Batch 64, 3x3 at stride 2, before -> after: 64 -> 128 at 56x56 0.366 -> 0.275 ms,
+    // 128 -> 256 at 28x28 0.377 -> 0.392, 256 -> 512 at 14x14 0.52 -> 0.35, 512 -> 1024 at 14x14 1.45 -> 0.87; the 7x7
+    // stem 3 -> 64 at 224x224 11.2 -> 3.3; batch 16 of the first layer (1.8 GFLOP) 0.148 -> 0.176: not taken there.
+    if ((sH > 1 || sW > 1) && OC * OH * OW > 0 && sH <= 8 && sW <= 8 && fits_i32(OC * IC * KH * KW) &&
+        repdl_cdiv(N * IC * ((H - 1 + pH) / sH + 1) * ((W - 1 + pW) / sW + 1), 256) <= REPDL_I32_MAX &&
+        2.0 * (double)total * (double)(OC * KH * KW) / (double)(sH * sW) >= 3e9)
+    {
+        hipStream_t s = repdl_stream(stream);
+        const int64_t HPmax = (H - 1 + pH) / sH + 1, WPmax = (W - 1 + pW) / sW + 1;
+        const int64_t Amax = (KH + sH - 1) / sH, Bmax = (KW + sW - 1) / sW;
+        const size_t ws_k = ((size_t)(OC * IC * Amax * Bmax) * sizeof(float) + 255) / 256 * 256;
+        const size_t ws_g = (size_t)(N * IC * HPmax * WPmax) * sizeof(float);
+        char *ws = nullptr;
+        hipError_t e = hipMallocAsync(reinterpret_cast<void **>(&ws), ws_k + ws_g, s);
+        if (e != hipSuccess)
+            return (int)e;
+        float *Ws = reinterpret_cast<float *>(ws), *Gp = reinterpret_cast<float *>(ws + ws_k);
+        int rc = REPDL_OK;
+        for (int64_t rh = 0; rh < sH && rc == REPDL_OK; rh++)
+            for (int64_t rw = 0; rw < sW && rc == REPDL_OK; rw++)
+            {
+                // h = sH * h' + rh - pH for h' = 0 .. HP - 1 (the first of them may lie above the image)
+                if (H - 1 + pH - rh < 0 || W - 1 + pW - rw < 0)
+                    continue; // no position of this residue
+                const int64_t HP = (H - 1 + pH - rh) / sH + 1, WP = (W - 1 + pW - rw) / sW + 1;
+                const int64_t A = rh < KH ? (KH - rh + sH - 1) / sH : 0, B = rw < KW ? (KW - rw + sW - 1) / sW : 0;
+                const int64_t count = N * IC * HP * WP;
+                const float *src = nullptr;
+                if (A > 0 && B > 0)
+                {
+                    const int64_t kt = OC * IC * A * B;
+                    hipLaunchKernelGGL(conv_phase_kernel_kernel, dim3((unsigned)repdl_cdiv(kt, 256)), dim3(256), 0, s, kernel, Ws, (int)kt,
+                                       (int)KH, (int)KW, (int)A, (int)B, (int)rh, (int)rw, (int)sH, (int)sW);
+                    rc = repdl_launch_status();
+                    if (rc == REPDL_OK)
+                        rc = repdl_hip_conv2d_grad_input(grad_output, Ws, Gp, N, OC, OH, OW, IC, A, B, HP, WP, 1, 1, 0, 0, stream);
+                    src = Gp;
+                }
+                if (rc == REPDL_OK)
+                {
+                    hipLaunchKernelGGL(conv_phase_scatter_kernel, dim3((unsigned)repdl_cdiv(count, 256)), dim3(256), 0, s, src, grad_input,
+                                       count, (int)HP, (int)WP, (int)H, (int)W, (int)sH, (int)sW, (int)(rh - pH), (int)(rw - pW));
+                    rc = repdl_launch_status();
+                }
+            }
+        e = hipFreeAsync(ws, s);
         return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
     }
     ConvDims d{(int)N, (int)IC, (int)H, (int)W, (int)OC, (int)KH, (int)KW, (int)OH,

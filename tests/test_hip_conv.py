@@ -146,6 +146,12 @@ DGRAD = [s for s in FWD if s[-1] == 1] + [
     (1, 128, 11, 13, 32, 3, 3, 3, 2, 0, 2, 1),
     (2, 64, 20, 22, 16, 5, 5, 4, 4, 2, 2, 1),
     (1, 64, 9, 9, 16, 2, 2, 1, 1, 3, 3, 1),      # padding beyond the kernel reach, stride 1
+    # strides with enough work (3 GFLOP of products that count) for the route that takes the residues of the stride
+    # one by one: stride-1 layers with the taps of a residue, their results interleaved
+    (64, 64, 56, 56, 128, 3, 3, 2, 2, 1, 1, 1),   # 3x3 at stride 2: kernels of 2x2, 2x1, 1x2 and 1x1 taps
+    (72, 64, 31, 29, 160, 5, 3, 2, 3, 2, 0, 1),   # 5x3 at stride (2, 3): a residue with a single column of taps, ragged extents
+    (64, 192, 30, 30, 320, 2, 2, 3, 3, 0, 0, 1),  # stride wider than the kernel: residues without any tap (+0)
+    (48, 64, 33, 34, 128, 3, 3, 1, 2, 1, 1, 1),   # a stride along the rows only
 ]
 
 
