@@ -1835,7 +1835,7 @@ __global__ __launch_bounds__(256) void conv_upsample_kernel(const float *__restr
 //     Ws[oc][ic][a][b] = W[oc][ic][rh + a * sH][rw + b * sW],   h = sH * h' + rh - pH,
 // with (oc, a, b) ascending exactly the reference's (oc, kh, kw) over the taps that count.  No product
 // with a zero of a dilated grad_output: a quarter of the work at stride 2.
-__global__ __launch_bounds__(256) void conv_phase_kernel_kernel(const float *__restrict__ Wk, float *__restrict__ Ws, int total, int KH,
+__global__ __launch_bounds__(256) void conv_phase_taps_kernel(const float *__restrict__ Wk, float *__restrict__ Ws, int total, int KH,
                                                                 int KW, int A, int B, int rh, int rw, int sH, int sW)
 {
     const int idx = blockIdx.x * 256 + threadIdx.x; // = (oc * IC + ic) * A * B + a * B + b
@@ -2790,7 +2790,7 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
         return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
     }
     // Strides, and enough work to pay for a dozen launches (3 GFLOP of products that count): residue by residue,
-    // see conv_phase_kernel_kernel.  Batch 64, 3x3 at stride 2, before -> after: 64 -> 128 at 56x56 0.366 -> 0.275 ms,
+    // see conv_phase_taps_kernel.  Batch 64, 3x3 at stride 2, before -> after: 64 -> 128 at 56x56 0.366 -> 0.275 ms,
     // 128 -> 256 at 28x28 0.377 -> 0.392, 256 -> 512 at 14x14 0.52 -> 0.35, 512 -> 1024 at 14x14 1.45 -> 0.87; the 7x7
     // stem 3 -> 64 at 224x224 11.2 -> 3.3; batch 16 of the first layer (1.8 GFLOP) 0.148 -> 0.176: not taken there.
     if ((sH > 1 || sW > 1) && OC * OH * OW > 0 && sH <= 8 && sW <= 8 && fits_i32(OC * IC * KH * KW) &&
@@ -2821,7 +2821,7 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
                 if (A > 0 && B > 0)
                 {
                     const int64_t kt = OC * IC * A * B;
-                    hipLaunchKernelGGL(conv_phase_kernel_kernel, dim3((unsigned)repdl_cdiv(kt, 256)), dim3(256), 0, s, kernel, Ws, (int)kt,
+                    hipLaunchKernelGGL(conv_phase_taps_kernel, dim3((unsigned)repdl_cdiv(kt, 256)), dim3(256), 0, s, kernel, Ws, (int)kt,
                                        (int)KH, (int)KW, (int)A, (int)B, (int)rh, (int)rw, (int)sH, (int)sW);
                     rc = repdl_launch_status();
                     if (rc == REPDL_OK)
