@@ -38,6 +38,11 @@ static inline hipStream_t repdl_stream(void *s) { return reinterpret_cast<hipStr
 
 static inline int64_t repdl_cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Scratch memory for the duration of a call, ordered on stream s (workspace.hip): in place of
+// hipMallocAsync / hipFreeAsync, which hold the host until the work in between has run.
+hipError_t repdl_ws_acquire(void **p, size_t bytes, hipStream_t s);
+hipError_t repdl_ws_release(void *p, hipStream_t s);
+
 // sum1d.hip: the exact parallel evaluation of sequential sums, for `rows` chains at once
 // (chain r: nseg segments of seglen contiguous floats, segment s at in + r*row_stride + s*seg_stride;
 // nseg > 1 needs seglen % 16 == 0 and nseg*seglen < 2^31); out[r] = factor * sum.

@@ -2208,7 +2208,7 @@ int launch(const float *gathered, const float *kernel, float *out, const ConvDim
     const bool skips = MODE == MODE_DGRAD || d.pH > 0 || d.pW > 0;
     const size_t pa_bytes = MODE == MODE_DGRAD ? ((size_t)wcount * sizeof(float) + 255) / 256 * 256 : 0;
     char *ws = nullptr;
-    const hipError_t e0 = hipMallocAsync(reinterpret_cast<void **>(&ws), GUARD_BYTES + pa_bytes, s);
+    const hipError_t e0 = repdl_ws_acquire(reinterpret_cast<void **>(&ws), GUARD_BYTES + pa_bytes, s);
     if (e0 != hipSuccess)
         return (int)e0;
     unsigned *guard = reinterpret_cast<unsigned *>(ws);
@@ -2225,7 +2225,7 @@ int launch(const float *gathered, const float *kernel, float *out, const ConvDim
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess)
         {
-            (void)hipFreeAsync(ws, s);
+            (void)repdl_ws_release(ws, s);
             return (int)e;
         }
     }
@@ -2233,7 +2233,7 @@ int launch(const float *gathered, const float *kernel, float *out, const ConvDim
     hipLaunchKernelGGL(kern, grid, dim3(128 * WGN), shmem, s, gathered, kernel, MODE == MODE_DGRAD ? PA : kernel, out, d,
                        guard_parts(guard, 0), ca, guard_parts(guard, 1), cb, skips ? 1 : 0, patch_rows(TN, PW));
     const int rc = repdl_launch_status();
-    const hipError_t e = hipFreeAsync(ws, s);
+    const hipError_t e = repdl_ws_release(ws, s);
     return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
 }
 } // namespace tapdma
@@ -2359,7 +2359,7 @@ int launch(const float *gathered, const float *kernel, float *out, const ConvDim
     const int P = d.H * d.W;
     const int64_t wcount = (int64_t)M * C;
     float *PA = nullptr;
-    const hipError_t e0 = hipMallocAsync(reinterpret_cast<void **>(&PA), (size_t)wcount * sizeof(float), s);
+    const hipError_t e0 = repdl_ws_acquire(reinterpret_cast<void **>(&PA), (size_t)wcount * sizeof(float), s);
     if (e0 != hipSuccess)
         return (int)e0;
     hipLaunchKernelGGL(conv_point_prep_kernel, dim3((unsigned)repdl_cdiv(wcount, 256)), dim3(256), 0, s, kernel, PA, wcount, MODE, C, M);
@@ -2367,7 +2367,7 @@ int launch(const float *gathered, const float *kernel, float *out, const ConvDim
     const dim3 grid((unsigned)(repdl_cdiv(ptiles, 8) * 8 * (M / 64)));
     hipLaunchKernelGGL((conv_point_kernel<MODE>), grid, dim3(256), 0, s, gathered, PA, out, d);
     const int rc = repdl_launch_status();
-    const hipError_t e = hipFreeAsync(PA, s);
+    const hipError_t e = repdl_ws_release(PA, s);
     return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
 }
 } // namespace point
@@ -2469,7 +2469,7 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
             const size_t wt_bytes = panel ? ((size_t)(groups * Mp * Kp) * sizeof(float) + 255) / 256 * 256 : 0;
             const size_t ws_bytes = GUARD_BYTES + tab_bytes + wt_bytes + (pad ? (size_t)d.N * img * sizeof(float) : 0);
             char *ws = nullptr;
-            hipError_t e = hipMallocAsync(reinterpret_cast<void **>(&ws), ws_bytes, s);
+            hipError_t e = repdl_ws_acquire(reinterpret_cast<void **>(&ws), ws_bytes, s);
             if (e != hipSuccess)
                 return (int)e;
             unsigned *guard = reinterpret_cast<unsigned *>(ws);
@@ -2531,7 +2531,7 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
             }
 #undef REPDL_CONV_FAST
             const int rc = repdl_launch_status();
-            e = hipFreeAsync(ws, s);
+            e = repdl_ws_release(ws, s);
             return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
         }
     }
@@ -2541,7 +2541,7 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
     hipError_t ge = hipSuccess;
     if (skips)
     {
-        ge = hipMallocAsync(reinterpret_cast<void **>(&guard), GUARD_BYTES, s);
+        ge = repdl_ws_acquire(reinterpret_cast<void **>(&guard), GUARD_BYTES, s);
         if (ge != hipSuccess)
             return (int)ge;
         int ca = 0, cb = 0;
@@ -2566,7 +2566,7 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
     }
     const int rc = repdl_launch_status();
     if (skips)
-        ge = hipFreeAsync(guard, s);
+        ge = repdl_ws_release(guard, s);
     return rc != REPDL_OK ? rc : (ge == hipSuccess ? REPDL_OK : (int)ge);
 }
 // ---------------------------------------------------------------------------
@@ -2678,7 +2678,7 @@ int launch_conv_mm(const float *gathered, const float *kernel, float *out, const
     const size_t c_bytes = ((size_t)(rows * M) * sizeof(float) + 255) / 256 * 256;
     const size_t wt_bytes = MODE == MODE_FWD ? 0 : ((size_t)(M * K) * sizeof(float) + 255) / 256 * 256;
     char *ws = nullptr;
-    hipError_t e = hipMallocAsync(reinterpret_cast<void **>(&ws), GUARD_BYTES + col_bytes + c_bytes + wt_bytes, s);
+    hipError_t e = repdl_ws_acquire(reinterpret_cast<void **>(&ws), GUARD_BYTES + col_bytes + c_bytes + wt_bytes, s);
     if (e != hipSuccess)
         return (int)e;
     unsigned *guard = reinterpret_cast<unsigned *>(ws);
@@ -2707,7 +2707,7 @@ int launch_conv_mm(const float *gathered, const float *kernel, float *out, const
                            out, d, total, skips ? guard : static_cast<const unsigned *>(nullptr));
         rc = repdl_launch_status();
     }
-    e = hipFreeAsync(ws, s);
+    e = repdl_ws_release(ws, s);
     return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
 }
 } // namespace
@@ -2772,7 +2772,7 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
         hipStream_t s = repdl_stream(stream);
         const int64_t count = N * IC * OH * OW;
         float *gs = nullptr;
-        hipError_t e = hipMallocAsync(reinterpret_cast<void **>(&gs), (size_t)count * sizeof(float), s);
+        hipError_t e = repdl_ws_acquire(reinterpret_cast<void **>(&gs), (size_t)count * sizeof(float), s);
         if (e != hipSuccess)
             return (int)e;
         int rc = repdl_hip_conv2d_grad_input(grad_output, kernel, gs, N, OC, OH, OW, IC, 1, 1, OH, OW, 1, 1, 0, 0, stream);
@@ -2786,7 +2786,7 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
                                    total, (int)H, (int)W, (int)OH, (int)OW, (int)sH, (int)sW);
             rc = repdl_launch_status();
         }
-        e = hipFreeAsync(gs, s);
+        e = repdl_ws_release(gs, s);
         return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
     }
     // Strides, and enough work to pay for a dozen launches (3 GFLOP of products that count): residue by residue,
@@ -2803,7 +2803,7 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
         const size_t ws_k = ((size_t)(OC * IC * Amax * Bmax) * sizeof(float) + 255) / 256 * 256;
         const size_t ws_g = (size_t)(N * IC * HPmax * WPmax) * sizeof(float);
         char *ws = nullptr;
-        hipError_t e = hipMallocAsync(reinterpret_cast<void **>(&ws), ws_k + ws_g, s);
+        hipError_t e = repdl_ws_acquire(reinterpret_cast<void **>(&ws), ws_k + ws_g, s);
         if (e != hipSuccess)
             return (int)e;
         float *Ws = reinterpret_cast<float *>(ws), *Gp = reinterpret_cast<float *>(ws + ws_k);
@@ -2835,7 +2835,7 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
                     rc = repdl_launch_status();
                 }
             }
-        e = hipFreeAsync(ws, s);
+        e = repdl_ws_release(ws, s);
         return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
     }
     ConvDims d{(int)N, (int)IC, (int)H, (int)W, (int)OC, (int)KH, (int)KW, (int)OH,
@@ -2881,7 +2881,7 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
     {
         const int64_t count = N * IC * OH * OW;
         float *xs = nullptr;
-        hipError_t e = hipMallocAsync(reinterpret_cast<void **>(&xs), (size_t)count * sizeof(float), s);
+        hipError_t e = repdl_ws_acquire(reinterpret_cast<void **>(&xs), (size_t)count * sizeof(float), s);
         if (e != hipSuccess)
             return (int)e;
         if (N * IC * H * W < (1LL << 31))
@@ -2893,7 +2893,7 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
         int rc = repdl_launch_status();
         if (rc == REPDL_OK)
             rc = repdl_hip_conv2d_grad_kernel(grad_output, xs, grad_kernel, N, IC, OH, OW, OC, OH, OW, 1, 1, 1, 1, 0, 0, stream);
-        e = hipFreeAsync(xs, s);
+        e = repdl_ws_release(xs, s);
         return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
     }
 
@@ -2907,7 +2907,7 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
             const size_t got_bytes = ((size_t)(K * OC) * sizeof(float) + 255) / 256 * 256;
             const size_t col_bytes = (size_t)(K * NC) * sizeof(float);
             char *ws = nullptr;
-            hipError_t e = hipMallocAsync(reinterpret_cast<void **>(&ws), GUARD_BYTES + got_bytes + col_bytes, s);
+            hipError_t e = repdl_ws_acquire(reinterpret_cast<void **>(&ws), GUARD_BYTES + got_bytes + col_bytes, s);
             if (e != hipSuccess)
                 return (int)e;
             unsigned *guard = reinterpret_cast<unsigned *>(ws);
@@ -2932,7 +2932,7 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
                                    input, grad_kernel, d, total, guard);
                 rc = repdl_launch_status();
             }
-            e = hipFreeAsync(ws, s);
+            e = repdl_ws_release(ws, s);
             return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
         }
     }
@@ -3005,7 +3005,7 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
             const size_t xbytes = xpad ? ((size_t)(N * IC * H * xW) * sizeof(float) + 255) / 256 * 256 : 0;
             const size_t gbytes = gpad ? (size_t)(N * OC * OH * OWp) * sizeof(float) : 0;
             char *ws = nullptr;
-            hipError_t e = hipMallocAsync(reinterpret_cast<void **>(&ws), GUARD_BYTES + xbytes + gbytes, s);
+            hipError_t e = repdl_ws_acquire(reinterpret_cast<void **>(&ws), GUARD_BYTES + xbytes + gbytes, s);
             if (e != hipSuccess)
                 return (int)e;
             unsigned *guard = reinterpret_cast<unsigned *>(ws);
@@ -3051,7 +3051,7 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);                \
         if (e_ != hipSuccess)                                                                                       \
         {                                                                                                           \
-            (void)hipFreeAsync(ws, s);                                                                              \
+            (void)repdl_ws_release(ws, s);                                                                              \
             return (int)e_;                                                                                         \
         }                                                                                                           \
         hipLaunchKernelGGL((conv_wgrad_mfma_kernel<Q, U, X, G, V>), dim3((unsigned)gx, (unsigned)gy), dim3(256), shmem, s, \
@@ -3097,7 +3097,7 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
 #undef REPDL_WGRAD_MFMA_Q
 #undef REPDL_WGRAD_MFMA
             const int rc = repdl_launch_status();
-            e = hipFreeAsync(ws, s);
+            e = repdl_ws_release(ws, s);
             return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
         }
     }
@@ -3143,7 +3143,7 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
     REPDL_REQUIRE(fits_i32(gx) && gy <= 65535);
     const dim3 grid((unsigned)gx, (unsigned)gy);
     unsigned *guard = nullptr;
-    hipError_t ge = hipMallocAsync(reinterpret_cast<void **>(&guard), GUARD_BYTES, s);
+    hipError_t ge = repdl_ws_acquire(reinterpret_cast<void **>(&guard), GUARD_BYTES, s);
     if (ge != hipSuccess)
         return (int)ge;
     int ca = 0, cb = 0;
@@ -3161,7 +3161,7 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);           \
         if (e_ != hipSuccess)                                                                                  \
         {                                                                                                      \
-            (void)hipFreeAsync(guard, s);                                                                      \
+            (void)repdl_ws_release(guard, s);                                                                      \
             return (int)e_;                                                                                    \
         }                                                                                                      \
         hipLaunchKernelGGL((conv_wgrad_kernel<P>), grid, dim3(256), shmem, s, grad_output, input, grad_kernel, \
@@ -3175,6 +3175,6 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
         REPDL_WGRAD(64);
 #undef REPDL_WGRAD
     const int rc = repdl_launch_status();
-    ge = hipFreeAsync(guard, s);
+    ge = repdl_ws_release(guard, s);
     return rc != REPDL_OK ? rc : (ge == hipSuccess ? REPDL_OK : (int)ge);
 }

@@ -423,11 +423,11 @@ static int launch_rowchain(const float *in, float *out, int64_t rows, int64_t ns
     {
         const size_t bytes = repdl_sum_chains_workspace_bytes(rows, len);
         void *ws = nullptr;
-        hipError_t e = hipMallocAsync(&ws, bytes, repdl_stream(stream));
+        hipError_t e = repdl_ws_acquire(&ws, bytes, repdl_stream(stream));
         if (e != hipSuccess)
             return (int)e;
         const int rc = repdl_sum_chains(in, out, rows, nseg, seglen, row_stride, seg_stride, factor, ws, bytes, stream);
-        e = hipFreeAsync(ws, repdl_stream(stream));
+        e = repdl_ws_release(ws, repdl_stream(stream));
         return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
     }
     // Chains per workgroup: enough workgroups to fill 256 CUs two to four times

@@ -1698,11 +1698,11 @@ REPDL_API int repdl_hip_sum1d(const float *in, float *out, int64_t n, int averag
     // no workspace given: take it from the stream-ordered allocator for the duration of the call
     const size_t bytes = repdl_hip_sum1d_workspace_bytes(n);
     void *ws = nullptr;
-    hipError_t e = hipMallocAsync(&ws, bytes, repdl_stream(stream));
+    hipError_t e = repdl_ws_acquire(&ws, bytes, repdl_stream(stream));
     if (e != hipSuccess)
         return (int)e;
     const int rc = repdl_hip_sum1d_ws(in, out, n, average, ws, bytes, stream);
-    e = hipFreeAsync(ws, repdl_stream(stream));
+    e = repdl_ws_release(ws, repdl_stream(stream));
     if (rc != REPDL_OK)
         return rc;
     return e == hipSuccess ? REPDL_OK : (int)e;
