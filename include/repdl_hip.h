@@ -96,8 +96,8 @@ int repdl_hip_mm_bias(const float *A, const float *B, const float *bias, float *
 /* conv2d -- backend/cuda/convolution.cu:153-183 (bound at :385); semantics
  * backend/cpu/convolution.cpp:12-52.  NCHW; kernel is [OC, IC/groups, KH, KW];
  * output is [N, OC, OH, OW] with OH = (H + 2 pH - KH) / sH + 1.
- * Scratch: the three convolutions take scratch memory from the stream-ordered
- * allocator (hipMallocAsync / hipFreeAsync on `stream`): 17 KiB whenever the geometry
+ * Scratch: the three convolutions take scratch memory from the library's scratch cache
+ * (see "Scratch cache" at repdl_hip_sum1d_ws): 17 KiB whenever the geometry
  * makes the reference skip taps (padding, strides of grad-input, kernels wider than one
  * tap in grad-input); on the matrix path also a copy of the kernel in the order the matrix
  * instruction reads it (3x3 kernels at stride 1 in grad-input, and 1x1 kernels with chains of
@@ -149,7 +149,14 @@ int repdl_hip_sum1d(const float *in, float *out, int64_t n, int average, void *s
  * parallel -- exactly: the result is the sequential chain's, bit for bit -- which needs
  * repdl_hip_sum1d_workspace_bytes(n) bytes of 16-byte aligned device memory (about 5n/8
  * bytes; 0 for short inputs).  The memory may hold anything on entry.  repdl_hip_sum1d itself
- * takes it from the stream-ordered allocator (hipMallocAsync / hipFreeAsync on `stream`). */
+ * takes it from the library's scratch cache.
+ * Scratch cache: the entry points that need a workspace and are not given one keep their
+ * buffers, a list per device and stream -- hipMalloc on first use and when a larger size is
+ * asked for (a blocking call), the same buffer for later calls on that stream (whose work is
+ * ordered, so the next call cannot touch it early), held until the process ends.  Requests
+ * beyond 4 GiB go to hipMallocAsync / hipFreeAsync on `stream`.  Two host threads may use one
+ * stream at once (they get different buffers); a graph captured through such an entry point
+ * holds the buffer's address, so nothing else should run on its capture stream while it replays. */
 size_t repdl_hip_sum1d_workspace_bytes(int64_t n);
 int repdl_hip_sum1d_ws(const float *in, float *out, int64_t n, int average, void *workspace,
                        size_t workspace_bytes, void *stream);
@@ -167,8 +174,8 @@ int repdl_hip_sum2d_dim0(const float *in, float *out, int64_t M, int64_t N, int 
                          void *stream);
 /* sum2d_dim1 and sum4d_dim023 with few long chains (at most 512 chains of at least 49152
  * elements; for sum4d_dim023 also H*W a multiple of 16) take the same parallel evaluation,
- * all chains at once, with about half the input's size in bytes from the stream-ordered
- * allocator (hipMallocAsync / hipFreeAsync on `stream`); otherwise they allocate nothing. */
+ * all chains at once, with about half the input's size in bytes from the scratch cache;
+ * otherwise they allocate nothing. */
 int repdl_hip_sum2d_dim1(const float *in, float *out, int64_t M, int64_t N, int average,
                          void *stream);
 int repdl_hip_sum4d_dim023(const float *in, float *out, int64_t N, int64_t C, int64_t H, int64_t W,
@@ -201,7 +208,7 @@ int repdl_hip_softmax(const float *in, float *out, int64_t M, int64_t N, void *s
  * backend/cpu/cross_entropy.cpp:15-24.  in is [M,N], target is [M] int64 class
  * indices in [0,N), out is one float.  workspace: M floats of device memory (the row
  * losses; their mean is repdl_hip_sum1d with average = 1, which from 32768 rows on takes
- * its own scratch from the stream-ordered allocator as described there). */
+ * its own scratch from the scratch cache as described there). */
 int repdl_hip_cross_entropy(const float *in, const int64_t *target, float *out, int64_t M,
                             int64_t N, float *workspace, void *stream);
 

@@ -1695,7 +1695,7 @@ REPDL_API int repdl_hip_sum1d(const float *in, float *out, int64_t n, int averag
     REPDL_REQUIRE(n >= 0 && out != nullptr && (n == 0 || in != nullptr));
     if (n < REPDL_SUM1D_MIN_PARALLEL)
         return repdl_sum1d_serial(in, out, n, average, stream);
-    // no workspace given: take it from the stream-ordered allocator for the duration of the call
+    // no workspace given: take it from the scratch cache for the duration of the call
     const size_t bytes = repdl_hip_sum1d_workspace_bytes(n);
     void *ws = nullptr;
     hipError_t e = repdl_ws_acquire(&ws, bytes, repdl_stream(stream));
