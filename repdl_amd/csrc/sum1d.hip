@@ -1523,7 +1523,8 @@ static int spec_rounds(int64_t rows, int64_t n)
     // 0.18) and a residual block with BatchNorm got 3 % slower with the rounds: not there.  256 x 262144
     // (4096 nodes) got slower either way; 64 x 802816 (3136 nodes: the first BatchNorm of a ResNet at batch 64)
     // 1.37 -> 0.69 ms zero-mean, 0.21 -> 0.33 drifting.  (Rounds from 2^17 elements made a ResNet-18 training step at
-    // batch 64 five milliseconds slower, 49 -> 54.7: they fill the chip that the other streams' kernels would use.)
+    // batch 64 five milliseconds slower, 49 -> 54.7, and still one millisecond slower, 38.8 -> 39.9, once the host no
+    // longer waited for every workspace: they fill the chip that the other streams' kernels would use.)
     if (rows > 1)
         return (n >= ((int64_t)1 << 19) && rows * repdl_cdiv(repdl_cdiv(n, BLK), NODEB) <= 3200) ? 3 : 0;
     if (n < ((int64_t)1 << 22))
