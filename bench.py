@@ -265,8 +265,9 @@ CHAIN_LIMITS = {
 }
 
 
-def leg_entry(name, workload, bound, work, fn, steps, warmup, parity, cpu, traffic_leg=None, default_size=True):
-    """One "also" entry: `work` is the algorithmic bytes (bound "hbm") or flop (bound "mfma") of one call."""
+def leg_entry(name, workload, bound, work, fn, steps, warmup, parity, cpu, traffic_leg=None, default_size=True, short=None):
+    """One "also" entry: `work` is the algorithmic bytes (bound "hbm") or flop (bound "mfma") of one call.
+    `short`: the workload's label in the printed line (`workload` itself goes to the detail file)."""
     wall, ev_mean, ev_min = time_gpu(fn, steps, warmup, SETTLE_MS)
     if bound == "hbm":
         rate, unit, peak = work / (ev_mean * 1e-3) / 1e9, "GB/s", HBM_PEAK_GBS
@@ -281,13 +282,40 @@ def leg_entry(name, workload, bound, work, fn, steps, warmup, parity, cpu, traff
     limit = CHAIN_LIMITS.get(traffic_leg)
     if limit is not None and default_size:
         roof["limited_by"] = limit  # what keeps this leg off the roofline named in "bound"
-    out = {"op": name, "workload": workload, "value": round(value, 2), "unit": vunit, "ms_per_step": round(ev_mean, 4),
-           "ms_min": round(ev_min, 4), "roofline": roof}
+    out = {"op": name, "workload": workload, "short": short or workload, "value": round(value, 2), "unit": vunit,
+           "ms_per_step": round(ev_mean, 4), "ms_min": round(ev_min, 4), "roofline": roof}
     if parity is not None:
         out["parity"] = parity
     if cpu is not None:
         out["cpu_baseline"] = cpu
     return out
+
+
+LINE_LIMIT = 7000  # bytes of the printed line: harnesses that keep only the tail of stdout must still see every leg
+DETAIL_JSON = os.path.join(ROOT, "gpurun_out", "bench_detail.json")
+ALSO_UNITS = {"hbm": {"unit": "GB/s", "peak": HBM_PEAK_GBS}, "mfma": {"unit": "TFLOP/s", "peak": FP32_PEAK_TFLOPS}}
+
+
+def compact_leg(e):
+    """A secondary leg as it is printed: numbers and short labels only.  `roofline.unit` / `roofline.peak` are those of
+    its bound (top-level "also_units"); digests, notes and what limits a leg go to the detail file."""
+    r = e["roofline"]
+    out = {"op": e["op"], "wl": e["short"], "ms": e["ms_per_step"],
+           "roofline": {"bound": r["bound"], "achieved": r["achieved"], "frac": r["frac"], "traffic": r["traffic"]}}
+    if "parity" in e:
+        out["equal"] = e["parity"].get("equal")
+    c = e.get("cpu_baseline")
+    if c is not None:
+        out["cpu_baseline"] = {"value": c["value"], "unit": c["unit"], "cores": c["cores"], "kind": c["kind"], "sample": c["short"]}
+    return out
+
+
+def compact_line(result) -> str:
+    """The one printed line: the headline in full, the secondary legs compacted."""
+    out = {k: v for k, v in result.items() if k != "also"}
+    out["also_units"] = ALSO_UNITS
+    out["also"] = [compact_leg(e) for e in result["also"]]
+    return json.dumps(out, separators=(",", ":"))
 
 
 # ----------------------------------------------------------------------------------------------
@@ -368,9 +396,9 @@ def main() -> int:
     if not args.quick:
         t0 = time.perf_counter()
         y_cpu = oracle.mm(x_h, w_h, False, True)
-        parity["mm"] = {"sha256_gpu": sha_headline, "sha256_cpu": sha(y_cpu), "checker": "oracle (C restatement)",
-                        "checker_s": round(time.perf_counter() - t0, 2)}
-        parity["mm"]["equal"] = parity["mm"]["sha256_gpu"] == parity["mm"]["sha256_cpu"]
+        sha_cpu = sha(y_cpu)
+        parity["mm"] = {"equal": sha_headline == sha_cpu, "sha256_gpu": sha_headline[:16], "sha256_cpu": sha_cpu[:16],
+                        "checker": "oracle, whole output", "checker_s": round(time.perf_counter() - t0, 2)}
         del y_cpu
 
     # CPU baseline: the reference's own CPU backend on a row slab of the same product
@@ -384,19 +412,16 @@ def main() -> int:
     slab_equal = torch.equal(y_slab, y_gpu[:rows].cpu())
     cpu_baseline = {
         "value": round(2.0 * rows * S * S / dt / 1e9, 3), "unit": "GFLOP/s", "cores": cores, "kind": kind,
-        "sample": "first %d of %d output rows of the same %dx%dx%d NT product (%.1f s); GPU rows bit-equal: %s"
-                  % (rows, S, S, S, S, dt, slab_equal),
+        "sample": "first %d of %d output rows of the same product (%.1f s); GPU rows bit-equal: %s" % (rows, S, dt, slab_equal),
     }
     del y_gpu, out_holder
 
     if _lib.lib().repdl_hip_matrix_path() == 1:
-        kernel_name = "mm_dma_kernel<NT, 128x128x16 tile, 512 threads, operands DMA'd global->LDS>"
-        kernel_note = ("fp32 matrix-instruction peak; v_mfma_f32_16x16x4_f32, checked on this device to be a "
-                       "k-ascending chain of single-rounding FMAs before use")
+        kernel_name = "mm_dma_kernel<NT>"
+        kernel_note = "v_mfma_f32_16x16x4_f32, checked on this device to be a k-ascending chain of single-rounding FMAs"
     else:
         kernel_name = "mm_kernel<NT>"
-        kernel_note = ("fp32 compute peak; the matrix-instruction check failed on this device, so the kernel issues "
-                       "v_fma_f32 only, whose issue-rate ceiling is half of this peak")
+        kernel_note = "matrix-instruction check failed on this device: v_fma_f32 only, ceiling half of this peak"
     traffic, why = measured_traffic("mm", S == 8192)
     result = {
         "metric": "bit-exact fp32 mm GFLOP/s at 8192^3",
@@ -410,8 +435,8 @@ def main() -> int:
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
-        "data": "synthetic (seeded host randn / uniform, same bytes for GPU and CPU checker)",
-        "config": {"workload": "repdl.ops.mm fp32 %dx%dx%d, transB (nn.Linear forward), configs[3]" % (S, S, S),
+        "data": "synthetic (seeded, same bytes for GPU and CPU checker)",
+        "config": {"workload": "repdl.ops.mm fp32 %dx%dx%d transB (nn.Linear forward), configs[3]" % (S, S, S),
                    "device": props.name, "cus": props.multi_processor_count},
         "roofline": {"bound": "mfma", "achieved": round(kern_tflops, 3), "peak": FP32_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(kern_tflops / FP32_PEAK_TFLOPS, 4), "traffic": traffic,
@@ -437,7 +462,7 @@ def main() -> int:
             f()
             par = {"equal": sha(hold["y"]) == sha_headline, "against": "the matrix-instruction kernel's output (itself checked against the oracle)"}
             also.append(leg_entry("mm (v_fma_f32 kernels)", "the headline's %dx%dx%d NT product, matrix instructions off" % (S, S, S), "mfma", flop,
-                                  f, max(2, args.steps // 2), 1, par, dict(cpu_baseline), "mm_fma", S == 8192))
+                                  f, max(2, args.steps // 2), 1, par, dict(cpu_baseline, short="as headline"), "mm_fma", S == 8192, short="%d^3 NT, matrix path off" % S))
             also[-1]["roofline"]["note"] = "v_fma_f32 only: the issue-rate ceiling of this path is 78.6 TFLOP/s, half the peak quoted"
             _lib.call("repdl_hip_set_matrix_path", -1)
             hold.clear()
@@ -452,8 +477,9 @@ def main() -> int:
             f()
             dt, y_cpu = cpu_time(lambda: (refmods[0].mm(a_h, b_h, False, False) if refmods else oracle.mm(a_h, b_h, False, False)))
             par = {"equal": sha(hold["y"]) == sha(y_cpu), "sha256_gpu": sha(hold["y"])}
-            cpu = {"value": round(2.0 * 1024 ** 3 / dt / 1e9, 3), "unit": "GFLOP/s", "cores": cores, "kind": kind, "sample": "the full product"}
-            also.append(leg_entry("mm", "1024x1024x1024 NN, N(0,1) entries (configs[0])", "mfma", 2.0 * 1024 ** 3, f, args.steps * 4, args.warmup, par, cpu, "mm1024"))
+            cpu = {"value": round(2.0 * 1024 ** 3 / dt / 1e9, 3), "unit": "GFLOP/s", "cores": cores, "kind": kind, "sample": "the full product", "short": "full"}
+            also.append(leg_entry("mm", "1024x1024x1024 NN, N(0,1) entries (configs[0])", "mfma", 2.0 * 1024 ** 3, f, args.steps * 4, args.warmup, par, cpu, "mm1024",
+                                  short="1024^3 NN cfg0"))
             del a_d, b_d
 
         if want("sum2d"):
@@ -467,9 +493,9 @@ def main() -> int:
             y_cpu = oracle.sum2d_dim1(m_h)
             par = {"equal": sha(hold["y"]) == sha(y_cpu), "sha256_gpu": sha(hold["y"])}
             dt, _ = cpu_time(lambda: (refmods[0].sum2d_dim1(m_h[:2048], False, False) if refmods else oracle.sum2d_dim1(m_h[:2048])))
-            cpu = {"value": round(2048 * R * 4 / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": kind, "sample": "first 2048 rows"}
+            cpu = {"value": round(2048 * R * 4 / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": kind, "sample": "first 2048 rows", "short": "2048 rows"}
             also.append(leg_entry("sum2d_dim1", "row sums of 16384x16384 N(0,1)*2^U(-20,20)", "hbm", 4.0 * R * R + 4 * R, f, args.steps, args.warmup,
-                                  par, cpu, "sum2d_dim1"))
+                                  par, cpu, "sum2d_dim1", short="16384^2 rows cfg1"))
             del m_d, m_h, hold
 
         if want("sum2d_dim0"):
@@ -482,9 +508,9 @@ def main() -> int:
             f()
             dt, y_cpu = cpu_time(lambda: (refmods[0].sum2d_dim0(m_h, False, False) if refmods else oracle.sum2d_dim0(m_h)))
             par = {"equal": sha(hold["y"]) == sha(y_cpu), "sha256_gpu": sha(hold["y"])}
-            cpu = {"value": round(M * N * 4 / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": kind, "sample": "the full matrix"}
+            cpu = {"value": round(M * N * 4 / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": kind, "sample": "the full matrix", "short": "full"}
             also.append(leg_entry("sum2d_dim0", "column sums of 65536x4096 N(0,1) (Linear grad-bias shape)", "hbm", 4.0 * M * N + 4 * N, f, args.steps,
-                                  args.warmup, par, cpu, "sum2d_dim0"))
+                                  args.warmup, par, cpu, "sum2d_dim0", short="65536x4096 cols"))
             del m_d, m_h, hold
 
         if want("sum4d"):
@@ -497,9 +523,9 @@ def main() -> int:
             f()
             dt, y_cpu = cpu_time(lambda: (refmods[0].sum4d_dim023(t_h, False, False) if refmods else oracle.sum4d_dim023(t_h)))
             par = {"equal": sha(hold["y"]) == sha(y_cpu), "sha256_gpu": sha(hold["y"])}
-            cpu = {"value": round(t_h.numel() * 4 / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": kind, "sample": "the full tensor"}
+            cpu = {"value": round(t_h.numel() * 4 / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": kind, "sample": "the full tensor", "short": "full"}
             also.append(leg_entry("sum4d_dim023", "channel sums of [64,64,56,56] N(0,1) (conv grad-bias shape)", "hbm", 4.0 * t_h.numel(), f,
-                                  args.steps, args.warmup, par, cpu, "sum4d_dim023"))
+                                  args.steps, args.warmup, par, cpu, "sum4d_dim023", short="[64,64,56,56]"))
             del t_d, t_h, hold
 
         if want("sum1d"):
@@ -512,14 +538,17 @@ def main() -> int:
             dt, y_cpu = cpu_time(lambda: (refmods[0].sum1d(v_h, False) if refmods else oracle.sum1d(v_h)))
             par = {"equal": sha(hold["y"]) == sha(y_cpu), "gpu": float(hold["y"]), "cpu": float(y_cpu)}
             cpu = {"value": round(n * 4 / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": kind,
-                   "sample": "the full 2^28 vector (the reference's sum1d is single-threaded)"}
-            also.append(leg_entry("sum1d", "sequential sum of 2^28 uniform[-1,1)", "hbm", 4.0 * n, f, args.steps, args.warmup, par, cpu, "sum1d"))
+                   "sample": "the full 2^28 vector (the reference's sum1d is single-threaded)", "short": "full"}
+            also.append(leg_entry("sum1d", "sequential sum of 2^28 uniform[-1,1)", "hbm", 4.0 * n, f, args.steps, args.warmup, par, cpu, "sum1d",
+                                  short="2^28 U[-1,1) cfg1"))
             v_d.abs_()  # the drifting case: uniform[0,1), the sum stops growing at 2^24
             v_h.abs_()
             f()
-            y_cpu = oracle.sum1d(v_h)
+            dt, y_cpu = cpu_time(lambda: (refmods[0].sum1d(v_h, False) if refmods else oracle.sum1d(v_h)))
             par = {"equal": sha(hold["y"]) == sha(y_cpu), "gpu": float(hold["y"]), "cpu": float(y_cpu)}
-            also.append(leg_entry("sum1d", "sequential sum of 2^28 uniform[0,1) (drifting)", "hbm", 4.0 * n, f, args.steps, args.warmup, par, None, "sum1d_drift"))
+            cpu = {"value": round(n * 4 / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": kind, "sample": "the full 2^28 vector", "short": "full"}
+            also.append(leg_entry("sum1d", "sequential sum of 2^28 uniform[0,1) (drifting)", "hbm", 4.0 * n, f, args.steps, args.warmup, par, cpu, "sum1d_drift",
+                                  short="2^28 U[0,1) drift"))
             del v_d, v_h, hold
 
         ew = [k for k in ("exp", "log", "sqrt", "div") if want(k)]
@@ -559,8 +588,9 @@ def main() -> int:
                     par["reference_sample_equal"] = torch.equal(y_ref.reshape(-1).view(torch.int32), y_cpu[:ns].view(torch.int32))
                     del y_cpu, y_ref
                     cpu = {"value": round(nbytes / n * ns / dt / 1e9, 3), "unit": "GB/s", "cores": rcores,
-                           "kind": "reference" if (refmods is not None or k in ("sqrt", "div")) else "port", "sample": "first 2^24 elements; " + rnote}
-                    also.append(leg_entry(name, wl, "hbm", nbytes, f, args.steps, args.warmup, par, cpu, name))
+                           "kind": "reference" if (refmods is not None or k in ("sqrt", "div")) else "port", "sample": "first 2^24 elements; " + rnote,
+                           "short": "2^24"}
+                    also.append(leg_entry(name, wl, "hbm", nbytes, f, args.steps, args.warmup, par, cpu, name, short="2^28 mix cfg2"))
                     hold.clear()
             del e_d, e_h
 
@@ -583,9 +613,10 @@ def main() -> int:
                 y_cpu = ofn()
                 par = {"equal": sha(hold["y"]) == sha(y_cpu), "sha256_gpu": sha(hold["y"])}
                 dt, _ = cpu_time(rfn)
-                cpu = {"value": round(nbytes / M * ms / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": kind, "sample": "first %d rows" % ms}
+                cpu = {"value": round(nbytes / M * ms / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": kind, "sample": "first %d rows" % ms,
+                       "short": "%d rows" % ms}
                 also.append(leg_entry(name, "%s of 65536x1000 logits N(0,16)" % name, "hbm", nbytes, f, args.steps, args.warmup, par, cpu,
-                                      name))
+                                      name, short="65536x1000"))
                 del y_cpu
             del z_d, z_h
 
@@ -620,10 +651,11 @@ def main() -> int:
                     par = {"equal": sha(hold["y"]) == sha(y_cpu), "sha256_gpu": sha(hold["y"])}
                     dt, _ = cpu_time(rfn)
                     cpu = {"value": round(cflop * nb / N / dt / 1e9, 2), "unit": "GFLOP/s", "cores": cores, "kind": kind,
-                           "sample": "the first %d of %d images (for grad-kernel: chains %d times shorter)" % (nb, N, N // nb)}
+                           "sample": "the first %d of %d images (for grad-kernel: chains %d times shorter)" % (nb, N, N // nb),
+                           "short": "%d/%d img" % (nb, N)}
                     tleg = "conv%dx%d_%s" % (Kk, Kk, {"conv2d": "fwd", "conv2d_grad_input": "dgrad", "conv2d_grad_kernel": "wgrad"}[name])
                     also.append(leg_entry(name, "batch %d, %dx%d conv %d->%d at %dx%d" % (N, Kk, Kk, IC, OC, H, W), "mfma", cflop, f, args.steps,
-                                          args.warmup, par, cpu, tleg))
+                                          args.warmup, par, cpu, tleg, short="b%d %dx%d %d>%d @%d cfg4" % (N, Kk, Kk, IC, OC, H)))
                     del y_cpu
                 del x_d, w_d, go_d
 
@@ -644,8 +676,9 @@ def main() -> int:
                 dt, y_slab = cpu_time(lambda: (refmods[0].mm(slab, b_h, bool(tA), False) if refmods else oracle.mm(slab, b_h, bool(tA), False)))
                 par = {"equal": torch.equal(y_slab, hold["y"][:rws].cpu()), "rows_checked": rws, "sha256_gpu": sha(hold["y"])}
                 cpu = {"value": round(2.0 * rws * N * K / dt / 1e9, 2), "unit": "GFLOP/s", "cores": cores, "kind": kind,
-                       "sample": "first %d of %d output rows" % (rws, M)}
-                also.append(leg_entry("mm", "%dx%dx%d %s" % (M, N, K, what), "mfma", 2.0 * M * N * K, f, max(2, args.steps // 2), 1, par, cpu))
+                       "sample": "first %d of %d output rows" % (rws, M), "short": "%d rows" % rws}
+                also.append(leg_entry("mm", "%dx%dx%d %s" % (M, N, K, what), "mfma", 2.0 * M * N * K, f, max(2, args.steps // 2), 1, par, cpu,
+                                      short="4096^2xK%d %s cfg3" % (K, "TN" if tA else "NN")))
                 del a_d, b_d, a_h, b_h, hold
 
         if want("adam"):
@@ -664,13 +697,27 @@ def main() -> int:
             stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
             def f(): _lib.call("repdl_hip_adam_step", desc, 1, betas[0], 1 - betas[0], betas[1], 1 - betas[1], eps, wd, stream)
             f()  # one step on both sides, compared before the timed steps run on
-            dt, _ = cpu_time(lambda: oracle.adam_step(p_h, g_h, m_h, v_h, None, t, lr, betas, eps, wd))
-            par = {"equal": all(sha(a) == sha(b) for a, b in zip(dev_t, (p_h, g_h, m_h, v_h))), "sha256_gpu": sha(dev_t[0])}
-            cpu = {"value": round(28.0 * na / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-                   "sample": "the full 2^26 elements, one step (the reference's Adam is a sequence of PyTorch tensor operations, repdl/optim.py:56-83; "
-                             "the oracle evaluates that sequence per element)"}
+
+            def reference_adam_step(p, grad, m, v):
+                """repdl/optim.py:64-83 on CPU tensors, ops.sqrt / ops.div as their CPU branches (repdl/ops.py:98-103, 122-123)."""
+                bc1, bc2 = 1 - betas[0] ** t, 1 - betas[1] ** t
+                grad = grad.add(p, alpha=wd)
+                m.mul_(betas[0]).add_(grad, alpha=1 - betas[0])
+                v.mul_(betas[1]).add_(torch.mul(grad, grad).mul(1 - betas[1]))
+                denom = v.to(dtype=torch.float64).sqrt().to(dtype=torch.float32).div(math.sqrt(bc2)).add_(eps)
+                p.add_(torch.div(m, denom).mul(-(lr / bc1)))
+
+            ref_t = [x.clone() for x in (p_h, g_h, m_h, v_h)]
+            dt, _ = cpu_time(lambda: reference_adam_step(*ref_t))
+            oracle.adam_step(p_h, g_h, m_h, v_h, None, t, lr, betas, eps, wd)
+            par = {"equal": all(sha(a) == sha(b) for a, b in zip(dev_t, (p_h, g_h, m_h, v_h))), "sha256_gpu": sha(dev_t[0]),
+                   "reference_equal": all(sha(a) == sha(b) for a, b in zip(dev_t, ref_t))}
+            cpu = {"value": round(28.0 * na / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "reference",
+                   "sample": "the full 2^26 elements, one step of the reference's own sequence of PyTorch CPU tensor operations (repdl/optim.py:64-83)",
+                   "short": "full"}
             also.append(leg_entry("adam_step", "one fused Adam step (weight decay on) over 2^26 parameters", "hbm", 28.0 * na, f, args.steps, args.warmup,
-                                  par, cpu, "adam_step"))
+                                  par, cpu, "adam_step", short="2^26 params"))
+            del ref_t
             del dev_t
 
         if want("cnn"):
@@ -706,13 +753,15 @@ def main() -> int:
                     optc.step()
                 dt, _ = cpu_time(fc, 3)
             also.append({"op": "cnn_step", "workload": "2-conv + 2-FC CNN via from_torch_module, batch 64 of 1x28x28, SGD lr 0.01 (forward, backward, update)",
+                         "short": "b64 1x28x28 SGD cfg4",
                          "value": round(1e3 / wall, 1), "unit": "steps/s", "ms_per_step": round(wall, 4),
                          "roofline": {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": None, "traffic": None,
                                       "traffic_note": "a chain of ~60 small launches: bound by launch latency, not by a roofline"},
                          "parity": {"equal": hashes["cpu"] == hashes["cuda"], "sha256_weights_after_3_steps": hashes["cuda"][0],
                                     "sha256_logits_after_3_steps": hashes["cuda"][1]},
                          "cpu_baseline": {"value": round(1.0 / dt, 2), "unit": "steps/s", "cores": cores, "kind": "port",
-                                          "sample": "the same step through the same glue with the oracle's operators on CPU tensors"}})
+                                          "sample": "the same step through the same glue with the oracle's operators on CPU tensors",
+                                          "short": "same glue on oracle"}})
 
     if args.copy_probe:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -721,7 +770,17 @@ def main() -> int:
             torch.trunc(src, out=dst)  # an elementwise kernel no leg uses: reads 1 GiB, writes 1 GiB
         torch.cuda.synchronize()
 
-    print(json.dumps(result))
+    try:
+        os.makedirs(os.path.dirname(DETAIL_JSON), exist_ok=True)
+        with open(DETAIL_JSON, "w") as f:
+            json.dump(result, f, indent=1)
+            f.write("\n")
+    except OSError as err:  # (a read-only tree: the printed line is what counts)
+        print("bench.py: detail file not written: %s" % err, file=sys.stderr)
+    line = compact_line(result)
+    if len(line) > LINE_LIMIT:
+        print("bench.py: the printed line has %d bytes, more than %d" % (len(line), LINE_LIMIT), file=sys.stderr)
+    print(line)
     return 0
 
 

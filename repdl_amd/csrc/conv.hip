@@ -2346,7 +2346,10 @@ bool applies(const ConvDims &d)
 {
     const int C = MODE == MODE_FWD ? d.IC : d.OC, M = MODE == MODE_FWD ? d.OC : d.IC;
     const int64_t P = (int64_t)d.H * d.W;
-    return d.groups == 1 && d.KH == 1 && d.KW == 1 && d.sH == 1 && d.sW == 1 && d.pH == 0 && d.pW == 0 && M % 64 == 0 && M / 64 <= 65535 &&
+    // (the kernel takes the source plane for the output plane: a grad-input call whose input extents are not
+    // those of grad_output -- the residues of a strided layer make such calls -- has to go elsewhere)
+    return d.groups == 1 && d.KH == 1 && d.KW == 1 && d.sH == 1 && d.sW == 1 && d.pH == 0 && d.pW == 0 && d.H == d.OH && d.W == d.OW &&
+           M % 64 == 0 && M / 64 <= 65535 &&
            C % (2 * RING) == 0 && C >= 2 * RING && P >= 1 && d.N <= 65535 && (int64_t)C * P * 4 < (1LL << 31) && (int64_t)M * C * 4 < (1LL << 31) &&
            (repdl_cdiv(P, 128) * d.N + 8) * (M / 64) < (1LL << 30) &&
            P >= 1024; // (small images: the products over all images at once, see conv_prefers_mm)
@@ -2408,7 +2411,7 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
     // (chains of 64 terms or fewer: the streaming kernel, which has no prologue to fill -- batch 64,
     // 56x56, 64 channels in, 256 out: 0.087 against 0.098 ms)
     const bool short_chain = K <= 64 && point::applies<MODE>(d);
-    if (mfma && !short_chain && d.groups == 1 && KHW == 1 && d.sH == 1 && d.sW == 1 && d.pH == 0 && d.pW == 0)
+    if (mfma && !short_chain && d.groups == 1 && KHW == 1 && d.sH == 1 && d.sW == 1 && d.pH == 0 && d.pW == 0 && d.H == d.OH && d.W == d.OW)
     {
         // a 1x1 kernel at stride 1: per image Out[M][P] = A[M][C] . Src[C][P], A = W (forward) or W^T
         // (grad-input) -- a batch of plain products, and the reference skips no tap here (batch 64:

@@ -152,6 +152,12 @@ DGRAD = [s for s in FWD if s[-1] == 1] + [
     (72, 64, 31, 29, 160, 5, 3, 2, 3, 2, 0, 1),   # 5x3 at stride (2, 3): a residue with a single column of taps, ragged extents
     (64, 192, 30, 30, 320, 2, 2, 3, 3, 0, 0, 1),  # stride wider than the kernel: residues without any tap (+0)
     (48, 64, 33, 34, 128, 3, 3, 1, 2, 1, 1, 1),   # a stride along the rows only
+    # residues whose positions outnumber the rows / columns of grad_output (their trailing positions have no tap, +0):
+    # the single-tap residues are 1x1 layers whose input and output planes differ
+    (44, 64, 32, 32, 256, 3, 3, 2, 2, 0, 0, 1),   # 15x15 outputs, residue 1 has 16x16 positions: products per image
+    (32, 128, 31, 31, 384, 2, 2, 2, 2, 0, 0, 1),  # every residue a single tap, 16 against 15 positions
+    (32, 128, 29, 29, 448, 3, 3, 3, 3, 0, 0, 1),  # stride 3: 10 against 9
+    (40, 64, 66, 66, 64, 3, 3, 2, 2, 0, 0, 1),    # 33x33 positions against 32x32 outputs, chains of 64: the streaming 1x1 kernel's shape
 ]
 
 
