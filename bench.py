@@ -300,13 +300,14 @@ def compact_leg(e):
     """A secondary leg as it is printed: numbers and short labels only.  `roofline.unit` / `roofline.peak` are those of
     its bound (top-level "also_units"); digests, notes and what limits a leg go to the detail file."""
     r = e["roofline"]
+    sig4 = lambda x: x if x is None else float("%.4g" % x)
     out = {"op": e["op"], "wl": e["short"], "ms": e["ms_per_step"],
-           "roofline": {"bound": r["bound"], "achieved": r["achieved"], "frac": r["frac"], "traffic": r["traffic"]}}
+           "roofline": {"bound": r["bound"], "achieved": sig4(r["achieved"]), "frac": r["frac"], "traffic": r["traffic"]}}
     if "parity" in e:
         out["equal"] = e["parity"].get("equal")
     c = e.get("cpu_baseline")
     if c is not None:
-        out["cpu_baseline"] = {"value": c["value"], "unit": c["unit"], "cores": c["cores"], "kind": c["kind"], "sample": c["short"]}
+        out["cpu_baseline"] = {"value": sig4(c["value"]), "unit": c["unit"], "cores": c["cores"], "kind": c["kind"], "sample": c["short"]}
     return out
 
 

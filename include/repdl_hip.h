@@ -45,6 +45,44 @@ extern "C" {
 const char *repdl_hip_error_string(int code);
 int repdl_hip_abi_version(void);
 
+/* Scratch memory.  No counterpart in the reference, whose device functions allocate their output
+ * and nothing else (backend/cuda/convolution.cu:153-183, 259-287, 359-383; summation.cu:33-147).
+ * Some entry points here need scratch for the duration of a call (they say so below).  Each of them
+ * comes in two forms:
+ *   repdl_hip_<op>_ws(..., workspace, workspace_bytes, stream) with
+ *   repdl_hip_<op>_workspace_bytes(...): the caller provides the memory -- device memory of at least
+ *     the size the query returns for the same arguments, any alignment, any contents.  The call
+ *     allocates, frees and keeps nothing, so it can be captured into a graph, and the memory can come
+ *     from the caller's own allocator (PyTorch's, in this library's bindings).  A workspace that is
+ *     missing or too small gives REPDL_E_WORKSPACE (nothing is written outside the workspace; the
+ *     output is then undefined).  A query is host arithmetic
+ *     only (it runs the entry point's own choice of kernels with the launches switched off; no device
+ *     is needed); where it takes operand pointers they are only looked at for their alignment, which
+ *     some kernels depend on, and may be NULL for a bound that holds for any pointers.  The bound
+ *     covers both settings of the matrix path.
+ *   repdl_hip_<op>(..., stream): the library's scratch cache provides it -- a list of buffers per
+ *     device and stream: hipMalloc on first use and when a larger size is asked for (a blocking
+ *     call), the same buffer for later calls on that stream (whose work is ordered, so the next call
+ *     cannot touch it early), held until repdl_hip_scratch_trim() or the end of the process; at most
+ *     4 GiB + 25 % per buffer (larger requests go to hipMallocAsync / hipFreeAsync on `stream`).  Two
+ *     host threads may use one stream at once (they get different buffers).  While `stream` is being
+ *     captured into a graph the cache neither allocates nor frees: the call succeeds only if a buffer
+ *     of sufficient size is already there -- from an earlier call with the same arguments on that
+ *     stream -- and fails with hipErrorStreamCaptureUnsupported (900) otherwise; a buffer used under
+ *     capture is never freed or moved afterwards, since the graph holds its address.  Nothing else
+ *     that takes scratch should run on the capture stream while such a graph replays.
+ *   repdl_hip_scratch_trim: frees every cache buffer that no call and no captured graph is using
+ *     (waits for the device).  repdl_hip_scratch_bytes: bytes the cache holds now. */
+int repdl_hip_scratch_trim(void);
+size_t repdl_hip_scratch_bytes(void);
+
+/* Which kernels ran.  No counterpart in the reference.  The operators choose among several kernel
+ * families by shape, alignment and the matrix path; every family that launches sets its bit in a
+ * process-wide mask.  repdl_hip_routes_taken returns the mask (and clears it when `reset` is not 0);
+ * repdl_hip_route_name names bit `route` (NULL past the last).  For tests that must reach every family. */
+uint64_t repdl_hip_routes_taken(int reset);
+const char *repdl_hip_route_name(int route);
+
 /* Matrix path.  No counterpart in the reference: its CUDA kernels use one FMA per
  * term (backend/cuda/matrix_multiplication.cu:18-60, convolution.cu:62-151).
  * mm and the three convolutions have two implementations of the same chains: one on
@@ -96,8 +134,7 @@ int repdl_hip_mm_bias(const float *A, const float *B, const float *bias, float *
 /* conv2d -- backend/cuda/convolution.cu:153-183 (bound at :385); semantics
  * backend/cpu/convolution.cpp:12-52.  NCHW; kernel is [OC, IC/groups, KH, KW];
  * output is [N, OC, OH, OW] with OH = (H + 2 pH - KH) / sH + 1.
- * Scratch: the three convolutions take scratch memory from the library's scratch cache
- * (see "Scratch cache" at repdl_hip_sum1d_ws): 17 KiB whenever the geometry
+ * Scratch (see "Scratch memory" above): 17 KiB whenever the geometry
  * makes the reference skip taps (padding, strides of grad-input, kernels wider than one
  * tap in grad-input); on the matrix path also a copy of the kernel in the order the matrix
  * instruction reads it (3x3 kernels at stride 1 in grad-input, and 1x1 kernels with chains of
@@ -121,6 +158,15 @@ int repdl_hip_conv2d_bias(const float *input, const float *kernel, const float *
                           int64_t IC, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t sH,
                           int64_t sW, int64_t pH, int64_t pW, int64_t groups, void *stream);
 
+/* conv2d / conv2d_bias with the caller's workspace (bias may be NULL). */
+size_t repdl_hip_conv2d_workspace_bytes(const float *input, const float *kernel, int64_t N, int64_t IC, int64_t H,
+                                        int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t sH, int64_t sW,
+                                        int64_t pH, int64_t pW, int64_t groups);
+int repdl_hip_conv2d_ws(const float *input, const float *kernel, const float *bias, float *output, int64_t N,
+                        int64_t IC, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t sH,
+                        int64_t sW, int64_t pH, int64_t pW, int64_t groups, void *workspace,
+                        size_t workspace_bytes, void *stream);
+
 /* conv2d_grad_input -- backend/cuda/convolution.cu:259-287 (bound at :386);
  * semantics backend/cpu/convolution.cpp:54-90.  groups == 1.
  * grad_output is [N, OC, OH, OW], kernel [OC, IC, KH, KW], grad_input [N, IC, H, W]. */
@@ -129,6 +175,15 @@ int repdl_hip_conv2d_grad_input(const float *grad_output, const float *kernel, f
                                 int64_t KH, int64_t KW, int64_t H, int64_t W, int64_t sH,
                                 int64_t sW, int64_t pH, int64_t pW, void *stream);
 
+size_t repdl_hip_conv2d_grad_input_workspace_bytes(const float *grad_output, const float *kernel, int64_t N,
+                                                   int64_t OC, int64_t OH, int64_t OW, int64_t IC, int64_t KH,
+                                                   int64_t KW, int64_t H, int64_t W, int64_t sH, int64_t sW,
+                                                   int64_t pH, int64_t pW);
+int repdl_hip_conv2d_grad_input_ws(const float *grad_output, const float *kernel, float *grad_input, int64_t N,
+                                   int64_t OC, int64_t OH, int64_t OW, int64_t IC, int64_t KH, int64_t KW,
+                                   int64_t H, int64_t W, int64_t sH, int64_t sW, int64_t pH, int64_t pW,
+                                   void *workspace, size_t workspace_bytes, void *stream);
+
 /* conv2d_grad_kernel -- backend/cuda/convolution.cu:359-383 (bound at :387);
  * semantics backend/cpu/convolution.cpp:92-128.  groups == 1.
  * grad_kernel is [OC, IC, KH, KW]. */
@@ -136,6 +191,14 @@ int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float *input, f
                                  int64_t N, int64_t IC, int64_t H, int64_t W, int64_t OC,
                                  int64_t OH, int64_t OW, int64_t KH, int64_t KW, int64_t sH,
                                  int64_t sW, int64_t pH, int64_t pW, void *stream);
+size_t repdl_hip_conv2d_grad_kernel_workspace_bytes(const float *grad_output, const float *input, int64_t N,
+                                                    int64_t IC, int64_t H, int64_t W, int64_t OC, int64_t OH,
+                                                    int64_t OW, int64_t KH, int64_t KW, int64_t sH, int64_t sW,
+                                                    int64_t pH, int64_t pW);
+int repdl_hip_conv2d_grad_kernel_ws(const float *grad_output, const float *input, float *grad_kernel, int64_t N,
+                                    int64_t IC, int64_t H, int64_t W, int64_t OC, int64_t OH, int64_t OW,
+                                    int64_t KH, int64_t KW, int64_t sH, int64_t sW, int64_t pH, int64_t pW,
+                                    void *workspace, size_t workspace_bytes, void *stream);
 
 /* sums -- backend/cuda/summation.cu:33-147 (bound at :149-155); semantics
  * backend/cpu/summation.cpp:12-78: strict left-to-right binary32 chains from
@@ -149,14 +212,7 @@ int repdl_hip_sum1d(const float *in, float *out, int64_t n, int average, void *s
  * parallel -- exactly: the result is the sequential chain's, bit for bit -- which needs
  * repdl_hip_sum1d_workspace_bytes(n) bytes of 16-byte aligned device memory (about 5n/8
  * bytes; 0 for short inputs).  The memory may hold anything on entry.  repdl_hip_sum1d itself
- * takes it from the library's scratch cache.
- * Scratch cache: the entry points that need a workspace and are not given one keep their
- * buffers, a list per device and stream -- hipMalloc on first use and when a larger size is
- * asked for (a blocking call), the same buffer for later calls on that stream (whose work is
- * ordered, so the next call cannot touch it early), held until the process ends.  Requests
- * beyond 4 GiB go to hipMallocAsync / hipFreeAsync on `stream`.  Two host threads may use one
- * stream at once (they get different buffers); a graph captured through such an entry point
- * holds the buffer's address, so nothing else should run on its capture stream while it replays. */
+ * takes it from the library's scratch cache (see "Scratch memory" above). */
 size_t repdl_hip_sum1d_workspace_bytes(int64_t n);
 int repdl_hip_sum1d_ws(const float *in, float *out, int64_t n, int average, void *workspace,
                        size_t workspace_bytes, void *stream);
@@ -180,6 +236,12 @@ int repdl_hip_sum2d_dim1(const float *in, float *out, int64_t M, int64_t N, int 
                          void *stream);
 int repdl_hip_sum4d_dim023(const float *in, float *out, int64_t N, int64_t C, int64_t H, int64_t W,
                            int average, void *stream);
+size_t repdl_hip_sum2d_dim1_workspace_bytes(int64_t M, int64_t N);
+int repdl_hip_sum2d_dim1_ws(const float *in, float *out, int64_t M, int64_t N, int average, void *workspace,
+                            size_t workspace_bytes, void *stream);
+size_t repdl_hip_sum4d_dim023_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W);
+int repdl_hip_sum4d_dim023_ws(const float *in, float *out, int64_t N, int64_t C, int64_t H, int64_t W, int average,
+                              void *workspace, size_t workspace_bytes, void *stream);
 
 /* exp, log -- backend/cuda/math.cu:15-18, 42-45 (drivers :30-39, :56-65; declared
  * backend/cuda/math.h, not bound to Python by the reference); semantics
@@ -211,6 +273,10 @@ int repdl_hip_softmax(const float *in, float *out, int64_t M, int64_t N, void *s
  * its own scratch from the scratch cache as described there). */
 int repdl_hip_cross_entropy(const float *in, const int64_t *target, float *out, int64_t M,
                             int64_t N, float *workspace, void *stream);
+/* cross_entropy with one caller's workspace for both the row losses and the scratch of their mean. */
+size_t repdl_hip_cross_entropy_workspace_bytes(int64_t M, int64_t N);
+int repdl_hip_cross_entropy_ws(const float *in, const int64_t *target, float *out, int64_t M, int64_t N,
+                               void *workspace, size_t workspace_bytes, void *stream);
 
 /* Batch normalisation, the elementwise passes -- the reference has no backend function for
  * these: repdl/nn/batchnorm.py:12-66 composes them from PyTorch tensor operations, one

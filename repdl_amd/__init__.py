@@ -13,8 +13,19 @@ import torch
 
 from . import func, nn, ops, optim, utils
 
-__all__ = ["func", "nn", "ops", "optim", "utils", "from_torch_module"]
+__all__ = ["func", "nn", "ops", "optim", "utils", "from_torch_module", "init"]
 __version__ = "0.1.0"
+
+
+def init() -> None:
+    """Runs the library's one-time device check (are the matrix instructions chains of single-rounding FMAs on
+    this GPU?) for the current device now, instead of inside the first GEMM-shaped call.  Importing the package
+    touches no device, so a launcher may still re-launch itself after the import; a program that captures graphs
+    calls this before its first capture (the check cannot run under capture, and calls made before it has run
+    take the slower ``v_fma_f32`` kernels -- same bits)."""
+    from . import _lib
+
+    _lib.init()
 
 
 def _bn_args(m):

@@ -44,6 +44,16 @@ def _stream(t: torch.Tensor) -> _P:
     return _P(torch.cuda.current_stream(t.device).cuda_stream)
 
 
+def _scratch(query: str, like: torch.Tensor, *args):
+    """Scratch memory of a call from PyTorch's allocator, sized by the entry point's own query: (tensor or None,
+    pointer, size).  The library then allocates, frees and keeps nothing, so the call can be captured into a graph."""
+    nbytes = int(getattr(_lib.lib(), query)(*args))
+    if nbytes == 0:
+        return None, None, ctypes.c_size_t(0)
+    work = torch.empty((nbytes,), dtype=torch.uint8, device=like.device)
+    return work, _ptr(work), ctypes.c_size_t(nbytes)
+
+
 def _same_device(a: torch.Tensor, b: torch.Tensor) -> None:
     if a.device != b.device:
         raise RuntimeError("tensors are on different devices: %s and %s" % (a.device, b.device))
@@ -98,8 +108,9 @@ def conv2d_bias(input, kernel, bias, strideH, strideW, paddingH, paddingW, group
     hold, bp = _bias(bias, x, OC)
     out = torch.empty((N, OC, OH, OW), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
-        _lib.call("repdl_hip_conv2d_bias", _ptr(x), _ptr(k), bp, _ptr(out), N, IC, H, W, OC, KH, KW, strideH, strideW,
-                  paddingH, paddingW, groups, _stream(x))
+        dims = (N, IC, H, W, OC, KH, KW, strideH, strideW, paddingH, paddingW, groups)
+        work, wp, wn = _scratch("repdl_hip_conv2d_workspace_bytes", x, _ptr(x), _ptr(k), *dims)
+        _lib.call("repdl_hip_conv2d_ws", _ptr(x), _ptr(k), bp, _ptr(out), *dims, wp, wn, _stream(x))
     return out
 
 
@@ -112,8 +123,9 @@ def conv2d_grad_input(grad_output, kernel, H, W, strideH, strideW, paddingH, pad
         raise RuntimeError("conv2d_grad_input: grad_output has %d channels, kernel has %d" % (OC, OCk))
     out = torch.empty((N, IC, H, W), dtype=torch.float32, device=go.device)
     with torch.cuda.device(go.device):
-        _lib.call("repdl_hip_conv2d_grad_input", _ptr(go), _ptr(k), _ptr(out), N, OC, OH, OW, IC, KH, KW, H, W,
-                  strideH, strideW, paddingH, paddingW, _stream(go))
+        dims = (N, OC, OH, OW, IC, KH, KW, H, W, strideH, strideW, paddingH, paddingW)
+        work, wp, wn = _scratch("repdl_hip_conv2d_grad_input_workspace_bytes", go, _ptr(go), _ptr(k), *dims)
+        _lib.call("repdl_hip_conv2d_grad_input_ws", _ptr(go), _ptr(k), _ptr(out), *dims, wp, wn, _stream(go))
     return out
 
 
@@ -126,8 +138,9 @@ def conv2d_grad_kernel(grad_output, input, KH, KW, strideH, strideW, paddingH, p
         raise RuntimeError("conv2d_grad_kernel: batch sizes differ (%d vs %d)" % (N, Ng))
     out = torch.empty((OC, IC, KH, KW), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
-        _lib.call("repdl_hip_conv2d_grad_kernel", _ptr(go), _ptr(x), _ptr(out), N, IC, H, W, OC, OH, OW, KH, KW,
-                  strideH, strideW, paddingH, paddingW, _stream(x))
+        dims = (N, IC, H, W, OC, OH, OW, KH, KW, strideH, strideW, paddingH, paddingW)
+        work, wp, wn = _scratch("repdl_hip_conv2d_grad_kernel_workspace_bytes", x, _ptr(go), _ptr(x), *dims)
+        _lib.call("repdl_hip_conv2d_grad_kernel_ws", _ptr(go), _ptr(x), _ptr(out), *dims, wp, wn, _stream(x))
     return out
 
 
@@ -135,15 +148,10 @@ def sum1d(input, average: bool = False) -> torch.Tensor:
     x = _check(input, "input", 1)
     out = torch.empty((), dtype=torch.float32, device=x.device)
     n = x.shape[0]
-    nbytes = int(_lib.lib().repdl_hip_sum1d_workspace_bytes(n))
     with torch.cuda.device(x.device):
-        if nbytes:
-            # scratch for the parallel evaluation of the sequential chain, from PyTorch's allocator
-            work = torch.empty((nbytes,), dtype=torch.uint8, device=x.device)
-            _lib.call("repdl_hip_sum1d_ws", _ptr(x), _ptr(out), n, int(bool(average)), _ptr(work),
-                      ctypes.c_size_t(nbytes), _stream(x))
-        else:
-            _lib.call("repdl_hip_sum1d", _ptr(x), _ptr(out), n, int(bool(average)), _stream(x))
+        # scratch for the parallel evaluation of the sequential chain
+        work, wp, wn = _scratch("repdl_hip_sum1d_workspace_bytes", x, n)
+        _lib.call("repdl_hip_sum1d_ws", _ptr(x), _ptr(out), n, int(bool(average)), wp, wn, _stream(x))
     return out
 
 
@@ -161,7 +169,8 @@ def sum2d_dim1(input, keepdim: bool = False, average: bool = False) -> torch.Ten
     M, N = x.shape
     out = torch.empty((M, 1), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
-        _lib.call("repdl_hip_sum2d_dim1", _ptr(x), _ptr(out), M, N, int(bool(average)), _stream(x))
+        work, wp, wn = _scratch("repdl_hip_sum2d_dim1_workspace_bytes", x, M, N)
+        _lib.call("repdl_hip_sum2d_dim1_ws", _ptr(x), _ptr(out), M, N, int(bool(average)), wp, wn, _stream(x))
     return out if keepdim else out.squeeze()
 
 
@@ -170,7 +179,8 @@ def sum4d_dim023(input, keepdim: bool = False, average: bool = False) -> torch.T
     N, C, H, W = x.shape
     out = torch.empty((1, C, 1, 1), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
-        _lib.call("repdl_hip_sum4d_dim023", _ptr(x), _ptr(out), N, C, H, W, int(bool(average)), _stream(x))
+        work, wp, wn = _scratch("repdl_hip_sum4d_dim023_workspace_bytes", x, N, C, H, W)
+        _lib.call("repdl_hip_sum4d_dim023_ws", _ptr(x), _ptr(out), N, C, H, W, int(bool(average)), wp, wn, _stream(x))
     return out if keepdim else out.squeeze()
 
 
@@ -236,10 +246,10 @@ def cross_entropy(input: torch.Tensor, target: torch.Tensor) -> torch.Tensor:
     if t.shape[0] != x.shape[0]:
         raise RuntimeError("cross_entropy: %d rows but %d targets" % (x.shape[0], t.shape[0]))
     out = torch.empty((), dtype=torch.float32, device=x.device)
-    work = torch.empty((max(x.shape[0], 1),), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
-        _lib.call("repdl_hip_cross_entropy", _ptr(x), _ptr(t), _ptr(out), x.shape[0], x.shape[1], _ptr(work),
-                  _stream(x))
+        # the row losses and the scratch of their mean
+        work, wp, wn = _scratch("repdl_hip_cross_entropy_workspace_bytes", x, x.shape[0], x.shape[1])
+        _lib.call("repdl_hip_cross_entropy_ws", _ptr(x), _ptr(t), _ptr(out), x.shape[0], x.shape[1], wp, wn, _stream(x))
     return out
 
 

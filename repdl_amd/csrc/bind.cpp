@@ -41,6 +41,21 @@ void same_device(const torch::Tensor &a, const torch::Tensor &b)
 }
 
 void ok(int rc, const char *what) { TORCH_CHECK(rc == 0, what, " failed with code ", rc, ": ", repdl_hip_error_string(rc)); }
+
+// Scratch memory of a call from PyTorch's allocator (the *_ws entry points): the library then allocates,
+// frees and keeps nothing of its own, and the call can be captured into a graph like any PyTorch operator.
+// The tensor dies when the binding returns; PyTorch hands its memory to later work on the same stream only.
+struct Scratch
+{
+    torch::Tensor hold;
+    size_t bytes;
+    Scratch(size_t nbytes, const torch::Tensor &like) : bytes(nbytes)
+    {
+        if (nbytes > 0)
+            hold = torch::empty({(int64_t)nbytes}, like.options().dtype(torch::kUInt8));
+    }
+    void *ptr() const { return bytes > 0 ? hold.data_ptr() : nullptr; }
+};
 } // namespace
 
 namespace
@@ -99,9 +114,12 @@ torch::Tensor conv2d_bias(const torch::Tensor &input, const torch::Tensor &kerne
     torch::Tensor hold;
     const float *bp = bias_pointer(bias, hold, x, OC);
     auto out = torch::empty({N, OC, OH, OW}, x.options());
-    ok(repdl_hip_conv2d_bias(x.data_ptr<float>(), k.data_ptr<float>(), bp, out.data_ptr<float>(), N, IC, H, W, OC, KH, KW,
-                             sH, sW, pH, pW, groups, current_stream()),
-       "repdl_hip_conv2d");
+    const Scratch work(repdl_hip_conv2d_workspace_bytes(x.data_ptr<float>(), k.data_ptr<float>(), N, IC, H, W, OC, KH, KW, sH, sW,
+                                                        pH, pW, groups),
+                       x);
+    ok(repdl_hip_conv2d_ws(x.data_ptr<float>(), k.data_ptr<float>(), bp, out.data_ptr<float>(), N, IC, H, W, OC, KH, KW, sH,
+                           sW, pH, pW, groups, work.ptr(), work.bytes, current_stream()),
+       "repdl_hip_conv2d_ws");
     return out;
 }
 
@@ -121,9 +139,12 @@ torch::Tensor conv2d_grad_input(const torch::Tensor &grad_output, const torch::T
     TORCH_CHECK(k.size(0) == OC, "conv2d_grad_input: grad_output has ", OC, " channels, kernel has ", k.size(0));
     const DeviceGuard guard(go.device());
     auto out = torch::empty({N, IC, H, W}, go.options());
-    ok(repdl_hip_conv2d_grad_input(go.data_ptr<float>(), k.data_ptr<float>(), out.data_ptr<float>(), N, OC, OH, OW, IC,
-                                   KH, KW, H, W, sH, sW, pH, pW, current_stream()),
-       "repdl_hip_conv2d_grad_input");
+    const Scratch work(repdl_hip_conv2d_grad_input_workspace_bytes(go.data_ptr<float>(), k.data_ptr<float>(), N, OC, OH, OW, IC, KH,
+                                                                   KW, H, W, sH, sW, pH, pW),
+                       go);
+    ok(repdl_hip_conv2d_grad_input_ws(go.data_ptr<float>(), k.data_ptr<float>(), out.data_ptr<float>(), N, OC, OH, OW, IC,
+                                      KH, KW, H, W, sH, sW, pH, pW, work.ptr(), work.bytes, current_stream()),
+       "repdl_hip_conv2d_grad_input_ws");
     return out;
 }
 
@@ -137,9 +158,12 @@ torch::Tensor conv2d_grad_kernel(const torch::Tensor &grad_output, const torch::
     TORCH_CHECK(go.size(0) == N, "conv2d_grad_kernel: batch sizes differ (", N, " vs ", go.size(0), ")");
     const DeviceGuard guard(x.device());
     auto out = torch::empty({OC, IC, KH, KW}, x.options());
-    ok(repdl_hip_conv2d_grad_kernel(go.data_ptr<float>(), x.data_ptr<float>(), out.data_ptr<float>(), N, IC, H, W, OC,
-                                    OH, OW, KH, KW, sH, sW, pH, pW, current_stream()),
-       "repdl_hip_conv2d_grad_kernel");
+    const Scratch work(repdl_hip_conv2d_grad_kernel_workspace_bytes(go.data_ptr<float>(), x.data_ptr<float>(), N, IC, H, W, OC, OH,
+                                                                    OW, KH, KW, sH, sW, pH, pW),
+                       x);
+    ok(repdl_hip_conv2d_grad_kernel_ws(go.data_ptr<float>(), x.data_ptr<float>(), out.data_ptr<float>(), N, IC, H, W, OC,
+                                       OH, OW, KH, KW, sH, sW, pH, pW, work.ptr(), work.bytes, current_stream()),
+       "repdl_hip_conv2d_grad_kernel_ws");
     return out;
 }
 
@@ -149,11 +173,9 @@ torch::Tensor sum1d(const torch::Tensor &input, bool average)
     const int64_t n = x.size(0);
     const DeviceGuard guard(x.device());
     auto out = torch::empty({}, x.options());
-    const size_t nbytes = repdl_hip_sum1d_workspace_bytes(n);
-    // scratch for the parallel evaluation of the sequential chain, from PyTorch's allocator
-    auto work = torch::empty({(int64_t)nbytes}, x.options().dtype(torch::kUInt8));
-    ok(repdl_hip_sum1d_ws(x.data_ptr<float>(), out.data_ptr<float>(), n, average, nbytes ? work.data_ptr() : nullptr,
-                          nbytes, current_stream()),
+    // scratch for the parallel evaluation of the sequential chain
+    const Scratch work(repdl_hip_sum1d_workspace_bytes(n), x);
+    ok(repdl_hip_sum1d_ws(x.data_ptr<float>(), out.data_ptr<float>(), n, average, work.ptr(), work.bytes, current_stream()),
        "repdl_hip_sum1d_ws");
     return out;
 }
@@ -173,8 +195,10 @@ torch::Tensor sum2d_dim1(const torch::Tensor &input, bool keepdim, bool average)
     const auto x = checked(input, "input", 2);
     const DeviceGuard guard(x.device());
     auto out = torch::empty({x.size(0), 1}, x.options());
-    ok(repdl_hip_sum2d_dim1(x.data_ptr<float>(), out.data_ptr<float>(), x.size(0), x.size(1), average, current_stream()),
-       "repdl_hip_sum2d_dim1");
+    const Scratch work(repdl_hip_sum2d_dim1_workspace_bytes(x.size(0), x.size(1)), x);
+    ok(repdl_hip_sum2d_dim1_ws(x.data_ptr<float>(), out.data_ptr<float>(), x.size(0), x.size(1), average, work.ptr(), work.bytes,
+                               current_stream()),
+       "repdl_hip_sum2d_dim1_ws");
     return keepdim ? out : out.squeeze();
 }
 
@@ -183,9 +207,10 @@ torch::Tensor sum4d_dim023(const torch::Tensor &input, bool keepdim, bool averag
     const auto x = checked(input, "input", 4);
     const DeviceGuard guard(x.device());
     auto out = torch::empty({1, x.size(1), 1, 1}, x.options());
-    ok(repdl_hip_sum4d_dim023(x.data_ptr<float>(), out.data_ptr<float>(), x.size(0), x.size(1), x.size(2), x.size(3),
-                              average, current_stream()),
-       "repdl_hip_sum4d_dim023");
+    const Scratch work(repdl_hip_sum4d_dim023_workspace_bytes(x.size(0), x.size(1), x.size(2), x.size(3)), x);
+    ok(repdl_hip_sum4d_dim023_ws(x.data_ptr<float>(), out.data_ptr<float>(), x.size(0), x.size(1), x.size(2), x.size(3),
+                                 average, work.ptr(), work.bytes, current_stream()),
+       "repdl_hip_sum4d_dim023_ws");
     return keepdim ? out : out.squeeze();
 }
 
@@ -251,10 +276,11 @@ torch::Tensor cross_entropy(const torch::Tensor &input, const torch::Tensor &tar
     TORCH_CHECK(t.size(0) == x.size(0), "cross_entropy: ", x.size(0), " rows but ", t.size(0), " targets");
     const DeviceGuard guard(x.device());
     auto out = torch::empty({}, x.options());
-    auto work = torch::empty({std::max<int64_t>(x.size(0), 1)}, x.options());
-    ok(repdl_hip_cross_entropy(x.data_ptr<float>(), t.data_ptr<int64_t>(), out.data_ptr<float>(), x.size(0), x.size(1),
-                               work.data_ptr<float>(), current_stream()),
-       "repdl_hip_cross_entropy");
+    // the row losses and the scratch of their mean
+    const Scratch work(repdl_hip_cross_entropy_workspace_bytes(x.size(0), x.size(1)), x);
+    ok(repdl_hip_cross_entropy_ws(x.data_ptr<float>(), t.data_ptr<int64_t>(), out.data_ptr<float>(), x.size(0), x.size(1),
+                                  work.ptr(), work.bytes, current_stream()),
+       "repdl_hip_cross_entropy_ws");
     return out;
 }
 namespace
@@ -334,9 +360,13 @@ torch::Tensor bn_gweight_term(const torch::Tensor &input, const torch::Tensor &m
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {
     namespace h = repdl::hip;
-    // the one-time check of the matrix instructions, at import instead of inside the first
-    // GEMM-shaped call (an error here -- no device yet -- leaves it to that call)
-    (void)repdl_hip_init();
+    // Importing the module touches no device.  The one-time check of the matrix instructions runs inside the
+    // first GEMM-shaped call on a device, or when the program calls init() -- which a program that captures
+    // graphs does before its first capture (a check cannot run under capture).
+    m.def("init", []() {
+        const int rc = repdl_hip_init();
+        TORCH_CHECK(rc == 0, "repdl_hip_init failed with code ", rc, ": ", repdl_hip_error_string(rc));
+    });
     m.def("conv2d", &h::conv2d);
     m.def("conv2d_grad_input", &h::conv2d_grad_input);
     m.def("conv2d_grad_kernel", &h::conv2d_grad_kernel);

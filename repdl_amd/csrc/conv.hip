@@ -258,13 +258,13 @@ inline void launch_guard_scan(const float *a, int64_t na, const float *b, int64_
     count_a = a ? guard_blocks(na) : 0;
     count_b = b ? guard_blocks(nb) : 0;
     if (count_a + count_b > 0)
-        hipLaunchKernelGGL(conv_guard_kernel, dim3((unsigned)(count_a + count_b)), dim3(256), 0, s, a, a ? na : 0, b,
+        REPDL_LAUNCH(conv_guard_kernel, dim3((unsigned)(count_a + count_b)), dim3(256), 0, s, a, a ? na : 0, b,
                            b ? nb : 0, count_a, guard_parts(guard, 0), guard_parts(guard, 1));
 }
 
 inline void launch_guard_final(unsigned *guard, int count_a, int count_b, hipStream_t s)
 {
-    hipLaunchKernelGGL(conv_guard_final_kernel, dim3(1), dim3(256), 0, s, guard, count_a, count_b);
+    REPDL_LAUNCH(conv_guard_final_kernel, dim3(1), dim3(256), 0, s, guard, count_a, count_b);
 }
 
 // ---------------------------------------------------------------------------
@@ -1761,9 +1761,6 @@ __global__ __launch_bounds__(256) void wgrad_fixup_kernel(const float *__restric
     GK[idx] = conv2d_grad_kernel_exact(GO, X, d, oc, ic, kh, kw);
 }
 
-#ifdef REPDL_DEBUG_HOOKS
-int g_wgrad_route = 0; // 1: always the product, 2: always the chain kernel
-#endif
 // Rough times of the two grad-kernel routes (seconds), from measurements on the layers of a
 // ResNet at batch 64: the chain kernel needs 12 clocks per step of a chain at stride 1 and 18 at
 // stride 2 (64 -> 128, 3x3, stride 2 at 56x56: 0.38 ms for 50176 steps), and about 34 us per round of
@@ -1777,10 +1774,6 @@ int g_wgrad_route = 0; // 1: always the product, 2: always the chain kernel
 // 90 us per round instead of 34 (1024 -> 256 at 14x14, two rounds of 12544 steps: 0.33 ms, product 0.20).
 inline bool wgrad_prefers_gemm(int64_t OC, int64_t NC, int64_t K, int64_t sW, int64_t OW, int64_t KHW)
 {
-#ifdef REPDL_DEBUG_HOOKS
-    if (g_wgrad_route != 0)
-        return g_wgrad_route == 1;
-#endif
     const double clk = 1.0 / 2.35e9;
     const double rounds = (double)repdl_cdiv(repdl_cdiv(NC, 16) * repdl_cdiv(OC, 32), 256);
     const int64_t OWr = (OW + 3) / 4 * 4;
@@ -2216,13 +2209,13 @@ int launch(const float *gathered, const float *kernel, float *out, const ConvDim
     const int ca = skips ? guard_blocks(gcount) : 0, cb = skips ? guard_blocks(wcount) : 0;
     const int wb = MODE == MODE_DGRAD ? (int)repdl_cdiv(wcount, 256) : 0;
     if (ca + cb + wb > 0)
-        hipLaunchKernelGGL(conv_tapdma_prep_kernel, dim3((unsigned)(ca + cb + wb)), dim3(256), 0, s, gathered, gcount, ca, kernel, wcount,
+        REPDL_LAUNCH(conv_tapdma_prep_kernel, dim3((unsigned)(ca + cb + wb)), dim3(256), 0, s, gathered, gcount, ca, kernel, wcount,
                            cb, guard_parts(guard, 0), guard_parts(guard, 1), PA, d.IC, d.OC);
     constexpr size_t shmem = (size_t)NB * (OPA + BSTR) * sizeof(float);
     auto kern = &conv_tapdma_kernel<MODE, WGN, VEC>;
     if (shmem > 48 * 1024)
     {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        const hipError_t e = REPDL_FUNC_SET_ATTRIBUTE(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess)
         {
             (void)repdl_ws_release(ws, s);
@@ -2230,7 +2223,7 @@ int launch(const float *gathered, const float *kernel, float *out, const ConvDim
         }
     }
     const dim3 grid((unsigned)(repdl_cdiv(repdl_cdiv(P, TN) * d.N, 8) * 8 * repdl_cdiv(M, 64)));
-    hipLaunchKernelGGL(kern, grid, dim3(128 * WGN), shmem, s, gathered, kernel, MODE == MODE_DGRAD ? PA : kernel, out, d,
+    REPDL_LAUNCH(kern, grid, dim3(128 * WGN), shmem, s, gathered, kernel, MODE == MODE_DGRAD ? PA : kernel, out, d,
                        guard_parts(guard, 0), ca, guard_parts(guard, 1), cb, skips ? 1 : 0, patch_rows(TN, PW));
     const int rc = repdl_launch_status();
     const hipError_t e = repdl_ws_release(ws, s);
@@ -2365,10 +2358,10 @@ int launch(const float *gathered, const float *kernel, float *out, const ConvDim
     const hipError_t e0 = repdl_ws_acquire(reinterpret_cast<void **>(&PA), (size_t)wcount * sizeof(float), s);
     if (e0 != hipSuccess)
         return (int)e0;
-    hipLaunchKernelGGL(conv_point_prep_kernel, dim3((unsigned)repdl_cdiv(wcount, 256)), dim3(256), 0, s, kernel, PA, wcount, MODE, C, M);
+    REPDL_LAUNCH(conv_point_prep_kernel, dim3((unsigned)repdl_cdiv(wcount, 256)), dim3(256), 0, s, kernel, PA, wcount, MODE, C, M);
     const int64_t ptiles = repdl_cdiv(P, 128) * d.N;
     const dim3 grid((unsigned)(repdl_cdiv(ptiles, 8) * 8 * (M / 64)));
-    hipLaunchKernelGGL((conv_point_kernel<MODE>), grid, dim3(256), 0, s, gathered, PA, out, d);
+    REPDL_LAUNCH((conv_point_kernel<MODE>), grid, dim3(256), 0, s, gathered, PA, out, d);
     const int rc = repdl_launch_status();
     const hipError_t e = repdl_ws_release(PA, s);
     return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
@@ -2404,10 +2397,16 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
     // 3x3 at stride 1: the input-patch kernel (batch 64: 64 -> 64 at 56x56 0.213 -> 0.149 ms, 128 -> 128 at
     // 28x28 0.208 -> 0.143, 256 -> 256 at 14x14 0.28 -> 0.18)
     if (mfma && tapdma::applies<MODE>(d, gathered, kernel, 64, 4))
+    {
+        repdl_route_note(REPDL_ROUTE_CONV_PATCH_16);
         return tapdma::launch<MODE, 2, 4>(gathered, kernel, out, d, s);
+    }
     // any other width, 4 bytes per DMA lane
     if (mfma && tapdma::applies<MODE>(d, gathered, kernel, 64, 1))
+    {
+        repdl_route_note(REPDL_ROUTE_CONV_PATCH_4);
         return tapdma::launch<MODE, 2, 1>(gathered, kernel, out, d, s);
+    }
     // (chains of 64 terms or fewer: the streaming kernel, which has no prologue to fill -- batch 64,
     // 56x56, 64 channels in, 256 out: 0.087 against 0.098 ms)
     const bool short_chain = K <= 64 && point::applies<MODE>(d);
@@ -2420,10 +2419,16 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
         const int rc = repdl_mm_batched(kernel, gathered, out, MODE == MODE_FWD ? d.bias : nullptr, M, P, K, MODE == MODE_DGRAD, 0,
                                         d.N, 0, (int64_t)K * P, (int64_t)M * P, s);
         if (rc != REPDL_E_UNSUPPORTED)
+        {
+            repdl_route_note(REPDL_ROUTE_CONV_POINT_MM);
             return rc;
+        }
     }
     if (mfma && point::applies<MODE>(d))
+    {
+        repdl_route_note(REPDL_ROUTE_CONV_POINT);
         return point::launch<MODE>(gathered, kernel, out, d, s);
+    }
     const int64_t gathered_count =
         (int64_t)d.N * (MODE == MODE_FWD ? (int64_t)d.IC * d.H * d.W : (int64_t)d.OC * d.OH * d.OW);
     const int64_t kernel_count = (int64_t)d.OC * (d.IC / d.groups) * KHW;
@@ -2489,14 +2494,14 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
             if (skips)
                 cb = guard_blocks(kernel_count);
             const int64_t wt_blocks = panel ? repdl_cdiv(groups * Mp * Kp, 256) : 0;
-            hipLaunchKernelGGL(conv_ktab_kernel, dim3((unsigned)(repdl_cdiv(Kp, 256) + wt_blocks + cb)), dim3(256), 0, s, tabB,
+            REPDL_LAUNCH(conv_ktab_kernel, dim3((unsigned)(repdl_cdiv(Kp, 256) + wt_blocks + cb)), dim3(256), 0, s, tabB,
                                (int)K, (int)Kp, M, (int)Mp, groups, d.KH, d.KW, (int)plane, (int)Wp, MODE, d.IC, d.pH + PT,
                                d.pW + PL, kernel, WT, (int)wt_blocks, kernel_count, cb, guard_parts(guard, 1));
             if (pad)
             {
                 const int64_t planes = (int64_t)d.N * C;
                 ca = (int)pad_blocks(planes);
-                hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)ca), dim3(256), 0, s, gathered, Gp, planes, SH, SW,
+                REPDL_LAUNCH(conv_pad_kernel, dim3((unsigned)ca), dim3(256), 0, s, gathered, Gp, planes, SH, SW,
                                    (int)Hp, (int)Wp, PT, PL, DH, DW, guard_parts(guard, 0));
             }
             if (skips)
@@ -2508,9 +2513,10 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
             const bool small_tiles = bm == 64 && conv_small_tiles(gx * (Mp / bm) * gz);
             dim3 grid((unsigned)(small_tiles ? repdl_cdiv(P, BN / 2) : gx), (unsigned)(Mp / bm), (unsigned)gz);
 #define REPDL_CONV_FAST(BM_, PB_, RG_)                                                                                  \
-    hipLaunchKernelGGL((conv_gemm_fast_kernel<BM_, MODE, PB_, RG_>), grid, dim3(2 * BM_), 0, s, src, gathered, kernel, \
+    REPDL_LAUNCH((conv_gemm_fast_kernel<BM_, MODE, PB_, RG_>), grid, dim3(2 * BM_), 0, s, src, gathered, kernel, \
                        Wa, out, d, tabB, (int)plane, (int)Wp, img, guard, (int)Mp, (int)Kp)
             const bool ragged = Mp != M;
+            repdl_route_note(bm == 64 && small_tiles ? REPDL_ROUTE_CONV_PADDED_64_HALF : bm == 64 ? REPDL_ROUTE_CONV_PADDED_64 : REPDL_ROUTE_CONV_PADDED_128);
             if (bm == 64 && small_tiles)
             {
                 if (ragged)
@@ -2551,21 +2557,22 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
         launch_guard_scan(gathered, gathered_count, kernel, kernel_count, guard, s, ca, cb);
         launch_guard_final(guard, ca, cb, s);
     }
+    repdl_route_note(M <= 64 ? REPDL_ROUTE_CONV_GATHER_64 : REPDL_ROUTE_CONV_GATHER_128);
     if (M <= 64)
     {
         dim3 grid((unsigned)gx, (unsigned)repdl_cdiv(M, 64), (unsigned)gz);
         if (mfma)
-            hipLaunchKernelGGL((conv_gemm_kernel<64, MODE, true>), grid, dim3(128), 0, s, gathered, kernel, out, d, wvec, ovec, guard);
+            REPDL_LAUNCH((conv_gemm_kernel<64, MODE, true>), grid, dim3(128), 0, s, gathered, kernel, out, d, wvec, ovec, guard);
         else
-            hipLaunchKernelGGL((conv_gemm_kernel<64, MODE, false>), grid, dim3(128), 0, s, gathered, kernel, out, d, wvec, ovec, guard);
+            REPDL_LAUNCH((conv_gemm_kernel<64, MODE, false>), grid, dim3(128), 0, s, gathered, kernel, out, d, wvec, ovec, guard);
     }
     else
     {
         dim3 grid((unsigned)gx, (unsigned)repdl_cdiv(M, 128), (unsigned)gz);
         if (mfma)
-            hipLaunchKernelGGL((conv_gemm_kernel<128, MODE, true>), grid, dim3(256), 0, s, gathered, kernel, out, d, wvec, ovec, guard);
+            REPDL_LAUNCH((conv_gemm_kernel<128, MODE, true>), grid, dim3(256), 0, s, gathered, kernel, out, d, wvec, ovec, guard);
         else
-            hipLaunchKernelGGL((conv_gemm_kernel<128, MODE, false>), grid, dim3(256), 0, s, gathered, kernel, out, d, wvec, ovec, guard);
+            REPDL_LAUNCH((conv_gemm_kernel<128, MODE, false>), grid, dim3(256), 0, s, gathered, kernel, out, d, wvec, ovec, guard);
     }
     const int rc = repdl_launch_status();
     if (skips)
@@ -2676,6 +2683,7 @@ int launch_conv_mm(const float *gathered, const float *kernel, float *out, const
     const int64_t P = MODE == MODE_FWD ? (int64_t)d.OH * d.OW : (int64_t)d.H * d.W;
     const int64_t rows = (int64_t)d.N * P;
     hipStream_t s = repdl_stream(stream);
+    repdl_route_note(REPDL_ROUTE_CONV_IM2COL);
     const bool skips = MODE == MODE_FWD ? (d.pH > 0 || d.pW > 0) : (KHW > 1 || d.sH > 1 || d.sW > 1 || d.pH > 0 || d.pW > 0);
     const size_t col_bytes = ((size_t)(rows * K) * sizeof(float) + 255) / 256 * 256;
     const size_t c_bytes = ((size_t)(rows * M) * sizeof(float) + 255) / 256 * 256;
@@ -2695,10 +2703,10 @@ int launch_conv_mm(const float *gathered, const float *kernel, float *out, const
         launch_guard_scan(gathered, gathered_count, kernel, (int64_t)d.OC * d.IC * KHW, guard, s, ca, cb);
         launch_guard_final(guard, ca, cb, s);
     }
-    hipLaunchKernelGGL((conv_col_kernel<MODE>), dim3((unsigned)repdl_cdiv(rows * K, 256)), dim3(256), 0, s, gathered, col,
+    REPDL_LAUNCH((conv_col_kernel<MODE>), dim3((unsigned)repdl_cdiv(rows * K, 256)), dim3(256), 0, s, gathered, col,
                        rows * K, d, (int)K);
     if (MODE == MODE_DGRAD)
-        hipLaunchKernelGGL(conv_wt_kernel, dim3((unsigned)repdl_cdiv(M * K, 256)), dim3(256), 0, s, kernel, WT, M * K, d.IC, KHW,
+        REPDL_LAUNCH(conv_wt_kernel, dim3((unsigned)repdl_cdiv(M * K, 256)), dim3(256), 0, s, kernel, WT, M * K, d.IC, KHW,
                            (int)K);
     int rc = repdl_launch_status();
     if (rc == REPDL_OK)
@@ -2706,7 +2714,7 @@ int launch_conv_mm(const float *gathered, const float *kernel, float *out, const
     if (rc == REPDL_OK)
     {
         const int64_t total = rows * M;
-        hipLaunchKernelGGL((conv_mm_out_kernel<MODE>), dim3((unsigned)repdl_cdiv(total, 256)), dim3(256), 0, s, C, gathered, kernel,
+        REPDL_LAUNCH((conv_mm_out_kernel<MODE>), dim3((unsigned)repdl_cdiv(total, 256)), dim3(256), 0, s, C, gathered, kernel,
                            out, d, total, skips ? guard : static_cast<const unsigned *>(nullptr));
         rc = repdl_launch_status();
     }
@@ -2773,6 +2781,7 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
         (OH - 1) * sH < H && (OW - 1) * sW < W && repdl_cdiv(total, 256) <= REPDL_I32_MAX)
     {
         hipStream_t s = repdl_stream(stream);
+        repdl_route_note(REPDL_ROUTE_DGRAD_POINT_SCATTER);
         const int64_t count = N * IC * OH * OW;
         float *gs = nullptr;
         hipError_t e = repdl_ws_acquire(reinterpret_cast<void **>(&gs), (size_t)count * sizeof(float), s);
@@ -2782,10 +2791,10 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
         if (rc == REPDL_OK)
         {
             if (total < (1LL << 31))
-                hipLaunchKernelGGL(conv_upsample_kernel<uint32_t>, dim3((unsigned)repdl_cdiv(total, 256)), dim3(256), 0, s, gs, grad_input,
+                REPDL_LAUNCH(conv_upsample_kernel<uint32_t>, dim3((unsigned)repdl_cdiv(total, 256)), dim3(256), 0, s, gs, grad_input,
                                    total, (int)H, (int)W, (int)OH, (int)OW, (int)sH, (int)sW);
             else
-                hipLaunchKernelGGL(conv_upsample_kernel<int64_t>, dim3((unsigned)repdl_cdiv(total, 256)), dim3(256), 0, s, gs, grad_input,
+                REPDL_LAUNCH(conv_upsample_kernel<int64_t>, dim3((unsigned)repdl_cdiv(total, 256)), dim3(256), 0, s, gs, grad_input,
                                    total, (int)H, (int)W, (int)OH, (int)OW, (int)sH, (int)sW);
             rc = repdl_launch_status();
         }
@@ -2801,6 +2810,7 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
         2.0 * (double)total * (double)(OC * KH * KW) / (double)(sH * sW) >= 3e9)
     {
         hipStream_t s = repdl_stream(stream);
+        repdl_route_note(REPDL_ROUTE_DGRAD_RESIDUES);
         const int64_t HPmax = (H - 1 + pH) / sH + 1, WPmax = (W - 1 + pW) / sW + 1;
         const int64_t Amax = (KH + sH - 1) / sH, Bmax = (KW + sW - 1) / sW;
         const size_t ws_k = ((size_t)(OC * IC * Amax * Bmax) * sizeof(float) + 255) / 256 * 256;
@@ -2824,7 +2834,7 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
                 if (A > 0 && B > 0)
                 {
                     const int64_t kt = OC * IC * A * B;
-                    hipLaunchKernelGGL(conv_phase_taps_kernel, dim3((unsigned)repdl_cdiv(kt, 256)), dim3(256), 0, s, kernel, Ws, (int)kt,
+                    REPDL_LAUNCH(conv_phase_taps_kernel, dim3((unsigned)repdl_cdiv(kt, 256)), dim3(256), 0, s, kernel, Ws, (int)kt,
                                        (int)KH, (int)KW, (int)A, (int)B, (int)rh, (int)rw, (int)sH, (int)sW);
                     rc = repdl_launch_status();
                     if (rc == REPDL_OK)
@@ -2833,7 +2843,7 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
                 }
                 if (rc == REPDL_OK)
                 {
-                    hipLaunchKernelGGL(conv_phase_scatter_kernel, dim3((unsigned)repdl_cdiv(count, 256)), dim3(256), 0, s, src, grad_input,
+                    REPDL_LAUNCH(conv_phase_scatter_kernel, dim3((unsigned)repdl_cdiv(count, 256)), dim3(256), 0, s, src, grad_input,
                                        count, (int)HP, (int)WP, (int)H, (int)W, (int)sH, (int)sW, (int)(rh - pH), (int)(rw - pW));
                     rc = repdl_launch_status();
                 }
@@ -2849,13 +2859,6 @@ REPDL_API int repdl_hip_conv2d_grad_input(const float *grad_output, const float 
     return launch_conv_gemm<MODE_DGRAD>(grad_output, kernel, grad_input, d, stream);
 }
 
-#ifdef REPDL_DEBUG_HOOKS
-REPDL_API int repdl_debug_wgrad_route(int r)
-{
-    g_wgrad_route = r;
-    return 0;
-}
-#endif
 
 REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float *input,
                                            float *grad_kernel, int64_t N, int64_t IC, int64_t H,
@@ -2883,15 +2886,16 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
         (OH - 1) * sH < H && (OW - 1) * sW < W && repdl_cdiv(N * IC * OH * OW, 256) <= REPDL_I32_MAX)
     {
         const int64_t count = N * IC * OH * OW;
+        repdl_route_note(REPDL_ROUTE_WGRAD_POINT_GATHER);
         float *xs = nullptr;
         hipError_t e = repdl_ws_acquire(reinterpret_cast<void **>(&xs), (size_t)count * sizeof(float), s);
         if (e != hipSuccess)
             return (int)e;
         if (N * IC * H * W < (1LL << 31))
-            hipLaunchKernelGGL(conv_subsample_kernel<uint32_t>, dim3((unsigned)repdl_cdiv(count, 256)), dim3(256), 0, s, input, xs, count,
+            REPDL_LAUNCH(conv_subsample_kernel<uint32_t>, dim3((unsigned)repdl_cdiv(count, 256)), dim3(256), 0, s, input, xs, count,
                                (int)H, (int)W, (int)OH, (int)OW, (int)sH, (int)sW);
         else
-            hipLaunchKernelGGL(conv_subsample_kernel<int64_t>, dim3((unsigned)repdl_cdiv(count, 256)), dim3(256), 0, s, input, xs, count,
+            REPDL_LAUNCH(conv_subsample_kernel<int64_t>, dim3((unsigned)repdl_cdiv(count, 256)), dim3(256), 0, s, input, xs, count,
                                (int)H, (int)W, (int)OH, (int)OW, (int)sH, (int)sW);
         int rc = repdl_launch_status();
         if (rc == REPDL_OK)
@@ -2907,6 +2911,7 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
             wgrad_prefers_gemm(OC, NC, K, sW, OW, KH * KW))
         {
             const bool skips = pH > 0 || pW > 0;
+            repdl_route_note(REPDL_ROUTE_WGRAD_PRODUCT);
             const size_t got_bytes = ((size_t)(K * OC) * sizeof(float) + 255) / 256 * 256;
             const size_t col_bytes = (size_t)(K * NC) * sizeof(float);
             char *ws = nullptr;
@@ -2922,16 +2927,16 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
                 launch_guard_scan(grad_output, N * OC * OH * OW, input, N * IC * H * W, guard, s, ca, cb);
                 launch_guard_final(guard, ca, cb, s);
             }
-            hipLaunchKernelGGL(wgrad_got_kernel, dim3((unsigned)repdl_cdiv(K * OC, 256)), dim3(256), 0, s, grad_output, GOt,
+            REPDL_LAUNCH(wgrad_got_kernel, dim3((unsigned)repdl_cdiv(K * OC, 256)), dim3(256), 0, s, grad_output, GOt,
                                K * OC, (int)OC, (int)(OH * OW));
-            hipLaunchKernelGGL(wgrad_col_kernel, dim3((unsigned)repdl_cdiv(K * NC, 256)), dim3(256), 0, s, input, col, K * NC,
+            REPDL_LAUNCH(wgrad_col_kernel, dim3((unsigned)repdl_cdiv(K * NC, 256)), dim3(256), 0, s, input, col, K * NC,
                                d, (int)NC);
             int rc = repdl_launch_status();
             if (rc == REPDL_OK)
                 rc = repdl_hip_mm(GOt, col, grad_kernel, OC, NC, K, 1, 0, stream);
             if (rc == REPDL_OK && skips)
             {
-                hipLaunchKernelGGL(wgrad_fixup_kernel, dim3((unsigned)repdl_cdiv(total, 256)), dim3(256), 0, s, grad_output,
+                REPDL_LAUNCH(wgrad_fixup_kernel, dim3((unsigned)repdl_cdiv(total, 256)), dim3(256), 0, s, grad_output,
                                    input, grad_kernel, d, total, guard);
                 rc = repdl_launch_status();
             }
@@ -3003,6 +3008,7 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
             fits_i32(repdl_cdiv(NC, 16)) &&
             repdl_cdiv(OC, MW_OC) <= 65535)
         {
+            repdl_route_note(REPDL_ROUTE_WGRAD_CHAIN);
             // workspace: the guard words, then the operands with rows rounded up to whole
             // instructions (grad_output) / whole float4 (input), when they are not
             const size_t xbytes = xpad ? ((size_t)(N * IC * H * xW) * sizeof(float) + 255) / 256 * 256 : 0;
@@ -3023,14 +3029,14 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
             if (xpad)
             {
                 cb = (int)pad_blocks(N * IC);
-                hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)cb), dim3(256), 0, s, input, xws, N * IC, (int)H, (int)W,
+                REPDL_LAUNCH(conv_pad_kernel, dim3((unsigned)cb), dim3(256), 0, s, input, xws, N * IC, (int)H, (int)W,
                                    (int)H, (int)xW, 0, 0, 1, 1, guard_parts(guard, 1));
             }
             const float *xsrc = xpad ? xws : input;
             if (gpad)
             {
                 ca = (int)pad_blocks(N * OC);
-                hipLaunchKernelGGL(conv_pad_kernel, dim3((unsigned)ca), dim3(256), 0, s, grad_output, gws, N * OC, (int)OH,
+                REPDL_LAUNCH(conv_pad_kernel, dim3((unsigned)ca), dim3(256), 0, s, grad_output, gws, N * OC, (int)OH,
                                    (int)OW, (int)OH, (int)OWp, 0, 0, 1, 1, guard_parts(guard, 0));
             }
             if (skips)
@@ -3050,14 +3056,14 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
 #define REPDL_WGRAD_MFMA(Q, U, X, G, V)                                                                                 \
     do                                                                                                              \
     {                                                                                                               \
-        hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_wgrad_mfma_kernel<Q, U, X, G, V>),       \
+        hipError_t e_ = REPDL_FUNC_SET_ATTRIBUTE(reinterpret_cast<const void *>(&conv_wgrad_mfma_kernel<Q, U, X, G, V>),       \
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);                \
         if (e_ != hipSuccess)                                                                                       \
         {                                                                                                           \
             (void)repdl_ws_release(ws, s);                                                                              \
             return (int)e_;                                                                                         \
         }                                                                                                           \
-        hipLaunchKernelGGL((conv_wgrad_mfma_kernel<Q, U, X, G, V>), dim3((unsigned)gx, (unsigned)gy), dim3(256), shmem, s, \
+        REPDL_LAUNCH((conv_wgrad_mfma_kernel<Q, U, X, G, V>), dim3((unsigned)gx, (unsigned)gy), dim3(256), shmem, s, \
                            gsrc, xsrc, grad_output, input, grad_kernel, d, (int)R, (int)NP, (int)GP, (int)Wp,       \
                            (int)CP, (int)hrows, (int)xoff, (int)bufsz, (int)xW, guard);                             \
     } while (0)
@@ -3145,6 +3151,7 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
     const int64_t gx = repdl_cdiv(NC, 64), gy = repdl_cdiv(OC, 4);
     REPDL_REQUIRE(fits_i32(gx) && gy <= 65535);
     const dim3 grid((unsigned)gx, (unsigned)gy);
+    repdl_route_note(REPDL_ROUTE_WGRAD_FMA);
     unsigned *guard = nullptr;
     hipError_t ge = repdl_ws_acquire(reinterpret_cast<void **>(&guard), GUARD_BYTES, s);
     if (ge != hipSuccess)
@@ -3160,14 +3167,14 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
 #define REPDL_WGRAD(P)                                                                                          \
     do                                                                                                         \
     {                                                                                                          \
-        hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_wgrad_kernel<P>),             \
+        hipError_t e_ = REPDL_FUNC_SET_ATTRIBUTE(reinterpret_cast<const void *>(&conv_wgrad_kernel<P>),             \
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);           \
         if (e_ != hipSuccess)                                                                                  \
         {                                                                                                      \
             (void)repdl_ws_release(guard, s);                                                                      \
             return (int)e_;                                                                                    \
         }                                                                                                      \
-        hipLaunchKernelGGL((conv_wgrad_kernel<P>), grid, dim3(256), shmem, s, grad_output, input, grad_kernel, \
+        REPDL_LAUNCH((conv_wgrad_kernel<P>), grid, dim3(256), shmem, s, grad_output, input, grad_kernel, \
                            d, (int)R, (int)NP, (int)Wp, (int)CP, (int)hrows, (int)bufsz, xvec, guard);         \
     } while (0)
     if (piece == 16)
@@ -3180,4 +3187,88 @@ REPDL_API int repdl_hip_conv2d_grad_kernel(const float *grad_output, const float
     const int rc = repdl_launch_status();
     ge = repdl_ws_release(guard, s);
     return rc != REPDL_OK ? rc : (ge == hipSuccess ? REPDL_OK : (int)ge);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The three convolutions with the caller's workspace.  The *_ws entry point installs the buffer
+// and runs the plain one under it (every scratch request of the call, nested calls included, is a
+// piece of that buffer); the size query runs the same host logic with the launches switched off,
+// so the two cannot disagree about the route.  Operand pointers not given to a query are tried on
+// and off a 16-byte boundary, the matrix path both ways; the largest need counts.
+// ---------------------------------------------------------------------------------------------
+namespace
+{
+template <typename F>
+size_t conv_ws_query(const float *a, const float *b, F call)
+{
+    size_t need = 0;
+    for (int ia = 0; ia < 2; ia++)
+        for (int ib = 0; ib < 2; ib++)
+        {
+            if ((a != nullptr && ia == 1) || (b != nullptr && ib == 1))
+                continue;
+            const float *pa = a != nullptr ? a : repdl_ws_fake_pointer(ia == 0);
+            const float *pb = b != nullptr ? b : repdl_ws_fake_pointer(ib == 0);
+            const size_t n = repdl_ws_query([&]() { return call(pa, pb); });
+            need = n > need ? n : need;
+        }
+    return need;
+}
+float *conv_ws_fake_output() { return const_cast<float *>(repdl_ws_fake_pointer(true)); }
+} // namespace
+
+REPDL_API size_t repdl_hip_conv2d_workspace_bytes(const float *input, const float *kernel, int64_t N, int64_t IC, int64_t H,
+                                                  int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t sH, int64_t sW,
+                                                  int64_t pH, int64_t pW, int64_t groups)
+{
+    return conv_ws_query(input, kernel, [&](const float *x, const float *k) {
+        return repdl_hip_conv2d_bias(x, k, nullptr, conv_ws_fake_output(), N, IC, H, W, OC, KH, KW, sH, sW, pH, pW, groups, nullptr);
+    });
+}
+
+REPDL_API int repdl_hip_conv2d_ws(const float *input, const float *kernel, const float *bias, float *output, int64_t N,
+                                  int64_t IC, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW, int64_t sH,
+                                  int64_t sW, int64_t pH, int64_t pW, int64_t groups, void *workspace,
+                                  size_t workspace_bytes, void *stream)
+{
+    RepdlWorkspace ws(workspace, workspace_bytes);
+    return repdl_hip_conv2d_bias(input, kernel, bias, output, N, IC, H, W, OC, KH, KW, sH, sW, pH, pW, groups, stream);
+}
+
+REPDL_API size_t repdl_hip_conv2d_grad_input_workspace_bytes(const float *grad_output, const float *kernel, int64_t N,
+                                                             int64_t OC, int64_t OH, int64_t OW, int64_t IC, int64_t KH,
+                                                             int64_t KW, int64_t H, int64_t W, int64_t sH, int64_t sW,
+                                                             int64_t pH, int64_t pW)
+{
+    return conv_ws_query(grad_output, kernel, [&](const float *g, const float *k) {
+        return repdl_hip_conv2d_grad_input(g, k, conv_ws_fake_output(), N, OC, OH, OW, IC, KH, KW, H, W, sH, sW, pH, pW, nullptr);
+    });
+}
+
+REPDL_API int repdl_hip_conv2d_grad_input_ws(const float *grad_output, const float *kernel, float *grad_input, int64_t N,
+                                             int64_t OC, int64_t OH, int64_t OW, int64_t IC, int64_t KH, int64_t KW,
+                                             int64_t H, int64_t W, int64_t sH, int64_t sW, int64_t pH, int64_t pW,
+                                             void *workspace, size_t workspace_bytes, void *stream)
+{
+    RepdlWorkspace ws(workspace, workspace_bytes);
+    return repdl_hip_conv2d_grad_input(grad_output, kernel, grad_input, N, OC, OH, OW, IC, KH, KW, H, W, sH, sW, pH, pW, stream);
+}
+
+REPDL_API size_t repdl_hip_conv2d_grad_kernel_workspace_bytes(const float *grad_output, const float *input, int64_t N,
+                                                              int64_t IC, int64_t H, int64_t W, int64_t OC, int64_t OH,
+                                                              int64_t OW, int64_t KH, int64_t KW, int64_t sH, int64_t sW,
+                                                              int64_t pH, int64_t pW)
+{
+    return conv_ws_query(grad_output, input, [&](const float *g, const float *x) {
+        return repdl_hip_conv2d_grad_kernel(g, x, conv_ws_fake_output(), N, IC, H, W, OC, OH, OW, KH, KW, sH, sW, pH, pW, nullptr);
+    });
+}
+
+REPDL_API int repdl_hip_conv2d_grad_kernel_ws(const float *grad_output, const float *input, float *grad_kernel, int64_t N,
+                                              int64_t IC, int64_t H, int64_t W, int64_t OC, int64_t OH, int64_t OW,
+                                              int64_t KH, int64_t KW, int64_t sH, int64_t sW, int64_t pH, int64_t pW,
+                                              void *workspace, size_t workspace_bytes, void *stream)
+{
+    RepdlWorkspace ws(workspace, workspace_bytes);
+    return repdl_hip_conv2d_grad_kernel(grad_output, input, grad_kernel, N, IC, H, W, OC, OH, OW, KH, KW, sH, sW, pH, pW, stream);
 }

@@ -390,15 +390,16 @@ int launch_rows_onchip(const float *in, float *out, const int64_t *target, float
                        hipStream_t s)
 {
     auto kern = &rows_onchip_kernel<R, VPT, SOFTMAX>;
+    repdl_route_note(REPDL_ROUTE_LOSS_ONCHIP);
     const size_t shmem = (size_t)R * onchip_stride((int)N, R) * sizeof(float);
     if (shmem > 40 * 1024)
     {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+        hipError_t e = REPDL_FUNC_SET_ATTRIBUTE(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)shmem);
         if (e != hipSuccess)
             return (int)e;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)repdl_cdiv(M, R)), dim3(256), shmem, s, in, out, target, loss, M, (int)N, vec_ok);
+    REPDL_LAUNCH(kern, dim3((unsigned)repdl_cdiv(M, R)), dim3(256), shmem, s, in, out, target, loss, M, (int)N, vec_ok);
     return repdl_launch_status();
 }
 
@@ -438,7 +439,8 @@ REPDL_API int repdl_hip_softmax(const float *in, float *out, int64_t M, int64_t 
     REPDL_REQUIRE(in != nullptr && out != nullptr && M <= REPDL_I32_MAX);
     if (rows_onchip_wanted(M, N))
         return rows_onchip<true>(in, out, nullptr, nullptr, M, N, repdl_stream(stream));
-    hipLaunchKernelGGL(softmax_kernel, dim3((unsigned)M), dim3(64), 0, repdl_stream(stream), in, out, M, N);
+    repdl_route_note(REPDL_ROUTE_LOSS_ROW_PER_WAVE);
+    REPDL_LAUNCH(softmax_kernel, dim3((unsigned)M), dim3(64), 0, repdl_stream(stream), in, out, M, N);
     return repdl_launch_status();
 }
 
@@ -456,7 +458,8 @@ REPDL_API int repdl_hip_cross_entropy(const float *in, const int64_t *target, fl
             rc = rows_onchip<false>(in, nullptr, target, workspace, M, N, repdl_stream(stream));
         else
         {
-            hipLaunchKernelGGL(cross_entropy_rows_kernel, dim3((unsigned)M), dim3(64), 0, repdl_stream(stream),
+            repdl_route_note(REPDL_ROUTE_LOSS_ROW_PER_WAVE);
+            REPDL_LAUNCH(cross_entropy_rows_kernel, dim3((unsigned)M), dim3(64), 0, repdl_stream(stream),
                                in, target, workspace, M, N);
             rc = repdl_launch_status();
         }
@@ -464,4 +467,31 @@ REPDL_API int repdl_hip_cross_entropy(const float *in, const int64_t *target, fl
             return rc;
     }
     return repdl_hip_sum1d(workspace, out, M, 1, stream);
+}
+
+// cross_entropy with one caller's workspace for the row losses and for the scratch of their mean
+REPDL_API size_t repdl_hip_cross_entropy_workspace_bytes(int64_t M, int64_t N)
+{
+    if (M <= 0 || N <= 0)
+        return 0;
+    const float *fake = repdl_ws_fake_pointer(true);
+    return repdl_ws_query([&]() {
+        return repdl_hip_cross_entropy_ws(fake, reinterpret_cast<const int64_t *>(fake), const_cast<float *>(fake), M, N, nullptr, 0, nullptr);
+    });
+}
+
+REPDL_API int repdl_hip_cross_entropy_ws(const float *in, const int64_t *target, float *out, int64_t M, int64_t N,
+                                         void *workspace, size_t workspace_bytes, void *stream)
+{
+    REPDL_REQUIRE(M >= 0);
+    // (a size query calls this with its own dry workspace installed: the caller's buffer only otherwise)
+    const bool dry = repdl_ws_dry();
+    RepdlWorkspace *ws = dry ? nullptr : new RepdlWorkspace(workspace, workspace_bytes);
+    float *rows = nullptr;
+    hipError_t e = repdl_ws_acquire(reinterpret_cast<void **>(&rows), (size_t)M * sizeof(float), repdl_stream(stream)); // (nothing for M = 0)
+    int rc = e == hipSuccess ? repdl_hip_cross_entropy(in, target, out, M, N, rows, stream) : (int)e;
+    if (e == hipSuccess)
+        e = repdl_ws_release(rows, repdl_stream(stream));
+    delete ws;
+    return rc != REPDL_OK ? rc : (e == hipSuccess ? REPDL_OK : (int)e);
 }

@@ -230,6 +230,10 @@ int device_verdict(int *rc_out)
 // Whether the GEMM-shaped operators may use the matrix instructions on the current device.
 bool repdl_mfma_exact()
 {
+    // (a workspace-size query asks about both settings without touching the device)
+    const int dry = repdl_ws_dry_matrix_path();
+    if (dry >= 0)
+        return dry == 1;
     std::lock_guard<std::mutex> guard(g_lock);
     if (g_mode == 0)
         return false;

@@ -653,12 +653,12 @@ int launch_dma_t(const float *A, const float *B, float *C, const float *cbias, c
     auto kern = &mm_dma_kernel<TA, TB, FM, FN, WGM, WGN, NQ, D, NB, DW, VEC>;
     if (shmem > 48 * 1024)
     {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+        hipError_t e = REPDL_FUNC_SET_ATTRIBUTE(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)shmem);
         if (e != hipSuccess)
             return (int)e;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)(gx * gy), (unsigned)nbatch), dim3(64 * (WGM * WGN + DW)), shmem, s, A, B, C, cbias, rbias, M,
+    REPDL_LAUNCH(kern, dim3((unsigned)(gx * gy), (unsigned)nbatch), dim3(64 * (WGM * WGN + DW)), shmem, s, A, B, C, cbias, rbias, M,
                        N, K, gx, gy, ntiles8, batch);
     return repdl_launch_status();
 }
@@ -701,9 +701,6 @@ int launch_dma(const float *A, const float *B, float *C, const float *cbias, con
 // Operand rows off 16-byte boundaries: the same tiles with 4-byte DMA lanes, four times the DMA
 // instructions (8190^3 NT / NN / TN: 120 / 124 / 137 TFLOP/s, against 96 through registers); the
 // one-workgroup-per-CU forms then take eight moving waves.
-#ifdef REPDL_DEBUG_HOOKS
-int g_force_tile = 0; // 1..7: that configuration whatever the shape
-#endif
 int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias, const float *rbias, int64_t M, int64_t N,
                     int64_t K, int transA, int transB, int avec, int bvec, int64_t nbatch, MmBatch batch, hipStream_t s)
 {
@@ -739,14 +736,11 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
         if (c < best)
             best = c, pick = 5;
     }
-#ifdef REPDL_DEBUG_HOOKS
-    if (g_force_tile > 0)
-        pick = g_force_tile;
-#endif
     if (!vec4)
         switch (pick)
         {
         case 1:
+            repdl_route_note(REPDL_ROUTE_MM_UNALIGNED_128);
             return launch_dma<4, 2, 2, 4, 4, 1, 3, 0, 1>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
         case 2:
         case 6:
@@ -754,12 +748,18 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
             // one 64x64 tile per CU: eight waves that only move (1001^2 x 2049: 54 TFLOP/s on the
             // four-wave form, 87 with four movers, 96 with eight)
             if (rounds(64, 64) == 1)
+            {
+                repdl_route_note(REPDL_ROUTE_MM_UNALIGNED_64_MOVERS);
                 return launch_dma<1, 2, 4, 2, 8, 1, 4, 8, 1>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+            }
+            repdl_route_note(REPDL_ROUTE_MM_UNALIGNED_64);
             return launch_dma<1, 2, 4, 2, 8, 1, 3, 0, 1>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
         case 3:
+            repdl_route_note(REPDL_ROUTE_MM_UNALIGNED_QUAD);
             return launch_dma<2, 2, 2, 2, 4, 1, 3, 0, 1>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
         case 4:
         case 5:
+            repdl_route_note(REPDL_ROUTE_MM_UNALIGNED_32);
             return launch_dma<1, 1, 2, 2, 16, 7, 5, 8, 1>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
         default:
             return REPDL_E_UNSUPPORTED;
@@ -773,19 +773,29 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
         // of an XCD stop sharing their operand rows as they drift apart along K), with four at 140; on
         // every other shape and layout the eight-wave form is the faster one by 4-6 %.
         if (transA && !transB && K >= 4 * (M > N ? M : N))
+        {
+            repdl_route_note(REPDL_ROUTE_MM_128_TALL);
             return launch_dma_t<true, false, 4, 4, 2, 2, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, nbatch, batch, s);
+        }
+        repdl_route_note(REPDL_ROUTE_MM_128);
         return launch_dma<4, 2, 2, 4, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 2:
+        repdl_route_note(REPDL_ROUTE_MM_64_FOUR_BUFFERS);
         return launch_dma<1, 2, 4, 2, 8, 1, 4, 4>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 6:
+        repdl_route_note(REPDL_ROUTE_MM_64_THREE_BUFFERS);
         return launch_dma<1, 2, 4, 2, 8, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 3:
+        repdl_route_note(REPDL_ROUTE_MM_64_QUAD);
         return launch_dma<2, 2, 2, 2, 4, 1, 3>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 7:
+        repdl_route_note(REPDL_ROUTE_MM_64_MOVERS);
         return launch_dma<1, 2, 4, 2, 8, 1, 3, 4>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 4:
+        repdl_route_note(REPDL_ROUTE_MM_32);
         return launch_dma<1, 1, 2, 2, 16, 7, 5, 4>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 5:
+        repdl_route_note(REPDL_ROUTE_MM_64X32);
         return launch_dma<1, 1, 4, 2, 16, 7, 5, 4>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     default:
         return REPDL_E_UNSUPPORTED;
@@ -795,13 +805,6 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 } // namespace
 
-#ifdef REPDL_DEBUG_HOOKS
-REPDL_API int repdl_debug_mm_tile(int t)
-{
-    g_force_tile = t;
-    return 0;
-}
-#endif
 
 int repdl_mm_batched(const float *A, const float *B, float *C, const float *row_bias, int64_t M, int64_t N, int64_t K,
                      int transA, int transB, int64_t nbatch, int64_t strideA, int64_t strideB, int64_t strideC,
@@ -809,10 +812,6 @@ int repdl_mm_batched(const float *A, const float *B, float *C, const float *row_
 {
     if (!repdl_mfma_exact() || M < 1 || N < 1 || K < 1 || nbatch < 1)
         return REPDL_E_UNSUPPORTED;
-#ifdef REPDL_DEBUG_HOOKS
-    if (g_force_tile == 99)
-        return REPDL_E_UNSUPPORTED;
-#endif
     const int64_t lda = transA ? M : K, ldb = transB ? K : N;
     const int avec = aligned16(A) && lda % 4 == 0 && strideA % 4 == 0;
     const int bvec = aligned16(B) && ldb % 4 == 0 && strideB % 4 == 0;
@@ -854,17 +853,18 @@ REPDL_API int repdl_hip_mm_bias(const float *A, const float *B, const float *bia
     const int64_t ntiles8 = (gx * gy) & ~(int64_t)7; // tiles covered by whole rounds over the 8 XCDs
     const int cvec = aligned16(C) && (N % 4 == 0);
     dim3 grid((unsigned)(gx * gy)), block(NT);
+    repdl_route_note(REPDL_ROUTE_MM_FMA);
     if (!transA && !transB)
-        hipLaunchKernelGGL((mm_kernel<false, false>), grid, block, 0, s, A, B, C, bias, M, N, K, avec, bvec, cvec, gx, gy,
+        REPDL_LAUNCH((mm_kernel<false, false>), grid, block, 0, s, A, B, C, bias, M, N, K, avec, bvec, cvec, gx, gy,
                            ntiles8);
     else if (transA && !transB)
-        hipLaunchKernelGGL((mm_kernel<true, false>), grid, block, 0, s, A, B, C, bias, M, N, K, avec, bvec, cvec, gx, gy,
+        REPDL_LAUNCH((mm_kernel<true, false>), grid, block, 0, s, A, B, C, bias, M, N, K, avec, bvec, cvec, gx, gy,
                            ntiles8);
     else if (!transA && transB)
-        hipLaunchKernelGGL((mm_kernel<false, true>), grid, block, 0, s, A, B, C, bias, M, N, K, avec, bvec, cvec, gx, gy,
+        REPDL_LAUNCH((mm_kernel<false, true>), grid, block, 0, s, A, B, C, bias, M, N, K, avec, bvec, cvec, gx, gy,
                            ntiles8);
     else
-        hipLaunchKernelGGL((mm_kernel<true, true>), grid, block, 0, s, A, B, C, bias, M, N, K, avec, bvec, cvec, gx, gy,
+        REPDL_LAUNCH((mm_kernel<true, true>), grid, block, 0, s, A, B, C, bias, M, N, K, avec, bvec, cvec, gx, gy,
                            ntiles8);
     return repdl_launch_status();
 }

@@ -433,6 +433,7 @@ static int launch_rowchain(const float *in, float *out, int64_t rows, int64_t ns
     // Chains per workgroup: enough workgroups to fill 256 CUs two to four times
     // over, all resident at once, and as many walking lanes as that allows.
     const bool vec = (reinterpret_cast<uintptr_t>(in) & 15) == 0 && row_stride % 4 == 0 && seg_stride % 4 == 0;
+    repdl_route_note(REPDL_ROUTE_SUM_ROW_WALK);
     const int rr = rows >= 49152 ? 64 : rows >= 12288 ? 32 : rows >= 6144 ? 16 : 4;
     const int64_t grid = repdl_cdiv(rows, rr);
     REPDL_REQUIRE(grid <= REPDL_I32_MAX);
@@ -452,12 +453,12 @@ static int launch_rowchain(const float *in, float *out, int64_t rows, int64_t ns
     {                                                                                                              \
         if (lds_pad != 0)                                                                                          \
         {                                                                                                          \
-            hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void *>(&rowchain_kernel<RRv, RTv, V, MU>), \
+            hipError_t e_ = REPDL_FUNC_SET_ATTRIBUTE(reinterpret_cast<const void *>(&rowchain_kernel<RRv, RTv, V, MU>), \
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_pad);         \
             if (e_ != hipSuccess)                                                                                  \
                 return (int)e_;                                                                                    \
         }                                                                                                          \
-        hipLaunchKernelGGL((rowchain_kernel<RRv, RTv, V, MU>), g, dim3(RTv), lds_pad, st, in, out, rows, nseg,     \
+        REPDL_LAUNCH((rowchain_kernel<RRv, RTv, V, MU>), g, dim3(RTv), lds_pad, st, in, out, rows, nseg,     \
                            seglen, row_stride, seg_stride, factor, spt);                                           \
     } while (0)
 #define REPDL_ROWCHAIN_V(RRv, RTv, V)              \
@@ -495,6 +496,7 @@ static int launch_rowchain(const float *in, float *out, int64_t rows, int64_t ns
 int repdl_sum1d_serial(const float *in, float *out, int64_t n, int average, void *stream)
 {
     REPDL_REQUIRE(n >= 0 && out != nullptr && (n == 0 || in != nullptr));
+    repdl_route_note(REPDL_ROUTE_SUM_SERIAL);
     return launch_rowchain(in, out, 1, 1, n, n, 0, repdl_sum_factor(average, n), stream);
 }
 
@@ -514,6 +516,34 @@ REPDL_API int repdl_hip_sum4d_dim023(const float *in, float *out, int64_t N, int
                            stream);
 }
 
+// The same two with the caller's workspace (see RepdlWorkspace): the size query runs the host logic
+// above with the launches switched off.
+REPDL_API size_t repdl_hip_sum2d_dim1_workspace_bytes(int64_t M, int64_t N)
+{
+    float *fake = const_cast<float *>(repdl_ws_fake_pointer(true));
+    return repdl_ws_query([&]() { return repdl_hip_sum2d_dim1(fake, fake, M, N, 0, nullptr); });
+}
+
+REPDL_API int repdl_hip_sum2d_dim1_ws(const float *in, float *out, int64_t M, int64_t N, int average, void *workspace,
+                                      size_t workspace_bytes, void *stream)
+{
+    RepdlWorkspace ws(workspace, workspace_bytes);
+    return repdl_hip_sum2d_dim1(in, out, M, N, average, stream);
+}
+
+REPDL_API size_t repdl_hip_sum4d_dim023_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W)
+{
+    float *fake = const_cast<float *>(repdl_ws_fake_pointer(true));
+    return repdl_ws_query([&]() { return repdl_hip_sum4d_dim023(fake, fake, N, C, H, W, 0, nullptr); });
+}
+
+REPDL_API int repdl_hip_sum4d_dim023_ws(const float *in, float *out, int64_t N, int64_t C, int64_t H, int64_t W, int average,
+                                        void *workspace, size_t workspace_bytes, void *stream)
+{
+    RepdlWorkspace ws(workspace, workspace_bytes);
+    return repdl_hip_sum4d_dim023(in, out, N, C, H, W, average, stream);
+}
+
 REPDL_API int repdl_hip_sum2d_dim0(const float *in, float *out, int64_t M, int64_t N, int average,
                                    void *stream)
 {
@@ -527,15 +557,16 @@ REPDL_API int repdl_hip_sum2d_dim0(const float *in, float *out, int64_t M, int64
     const dim3 g((unsigned)grid);
     hipStream_t st = repdl_stream(stream);
     const float factor = repdl_sum_factor(average, M);
+    repdl_route_note(REPDL_ROUTE_SUM_COLUMN_WALK);
     // few workgroups, long columns: the walk of each is the critical path -- two LDS buffers
     const bool two = grid <= 512 && M >= 4096;
 #define REPDL_COLTILE(CWv, NBv)                                                                               \
     do                                                                                                       \
     {                                                                                                        \
         if (vec)                                                                                             \
-            hipLaunchKernelGGL((coltile_kernel<CWv, true, NBv>), g, dim3(320), 0, st, in, out, M, N, factor); \
+            REPDL_LAUNCH((coltile_kernel<CWv, true, NBv>), g, dim3(320), 0, st, in, out, M, N, factor); \
         else                                                                                                 \
-            hipLaunchKernelGGL((coltile_kernel<CWv, false, NBv>), g, dim3(320), 0, st, in, out, M, N, factor); \
+            REPDL_LAUNCH((coltile_kernel<CWv, false, NBv>), g, dim3(320), 0, st, in, out, M, N, factor); \
     } while (0)
     if (cw == 64)
         REPDL_COLTILE(64, 1);

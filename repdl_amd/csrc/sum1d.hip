@@ -1106,14 +1106,6 @@ __global__ __launch_bounds__(64) void sum1d_plan_kernel(const double *__restrict
     }
 }
 
-#ifdef REPDL_DEBUG_HOOKS
-__device__ unsigned long long g_dbg[8]; // wave-level counts: nodes, blocks failed, groups failed, chunk replays
-#endif
-#if defined(REPDL_DEBUG_HOOKS) && defined(REPDL_DEBUG_COUNTS) // (the counting itself slows the walks many times over)
-#define DBG_COUNT(i) do { if ((threadIdx.x & 63) == 0) atomicAdd(&g_dbg[i], 1ull); } while (0)
-#else
-#define DBG_COUNT(i) do { } while (0)
-#endif
 
 // The walks of a round: workgroups of 256 threads take nodes off the list until it is empty
 // (every workgroup leaves the loop: the list's length is fixed before the launch).  Thread t
@@ -1157,10 +1149,8 @@ __global__ __launch_bounds__(256) void sum1d_cand_walk_kernel(
             __syncthreads();
             if (b + 1 < NODEB)
                 load_node_block(r, xr, c, T1r, TGr, T2r, nd * NODEB + b + 1, tid, vec);
-            DBG_COUNT(0);
             if (apply_all(s, lmap[buf][BLK / CH + GROUPS]))
                 continue;
-            DBG_COUNT(1);
             // Where the sum is small against its elements nothing applies, block after block; a
             // test costs a quarter of a replay there, and a replay is always right.  So after two
             // failures in a row the rest of the unit (the groups of a block, the chunks of a group)
@@ -1174,7 +1164,6 @@ __global__ __launch_bounds__(256) void sum1d_cand_walk_kernel(
                     continue;
                 }
                 gfail++;
-                DBG_COUNT(2);
                 constexpr int CG = BLK / CH / GROUPS; // 8 chunks; their data is read half a chunk ahead of the additions
                 const float *xg = &xd[buf][gr * CG * CH];
                 f4v ha[CH / 8], hb[CH / 8];
@@ -1187,7 +1176,6 @@ __global__ __launch_bounds__(256) void sum1d_cand_walk_kernel(
                     const bool replay = cfail >= 2 || !apply_all(s, lmap[buf][gr * CG + j]);
                     if (replay)
                     {
-                        DBG_COUNT(3);
                         s = add_half(s, ha);
                     }
                     if (j + 1 < CG)
@@ -1506,16 +1494,8 @@ int repdl_sum1d_serial(const float *in, float *out, int64_t n, int average, void
 // Number of speculative rounds for `rows` chains of n elements (0: step 4 alone).  Rounds pay
 // from a few million elements on; chains that come in rows are short and many, and their walks
 // already run side by side.
-#ifdef REPDL_DEBUG_HOOKS
-static int g_debug_rounds = -1;
-static int g_debug_norefine = 0;
-#endif
 static int spec_rounds(int64_t rows, int64_t n)
 {
-#ifdef REPDL_DEBUG_HOOKS
-    if (g_debug_rounds >= 0)
-        return g_debug_rounds;
-#endif
     // Chains that come in rows: three rounds when the chains are very long and their nodes few enough
     // for one pass of the walkers.  Zero-mean chains gain (16 x 802816: 1.27 -> 0.42 ms, 8 x 2^20: 1.07 ->
     // 0.37), chains that drift lose the rounds' fifteen launches (0.09 -> 0.14 ms).  At 200704 elements
@@ -1623,24 +1603,20 @@ int repdl_sum_chains(const float *in, float *out, int64_t rows, int64_t nseg, in
     const dim3 g2((unsigned)nblk, (unsigned)rows);
     double *babs = reinterpret_cast<double *>(w + l.babs);
     int *refine = reinterpret_cast<int *>(w + l.refine);
-    hipLaunchKernelGGL(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(nullptr), bsum, babs,
+    REPDL_LAUNCH(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(nullptr), bsum, babs,
                        static_cast<const int *>(refine), vec);
-    hipLaunchKernelGGL(sum1d_prefix_kernel, dim3((unsigned)rows), dim3(1024), 0, s, bsum, prefix, nblk,
+    REPDL_LAUNCH(sum1d_prefix_kernel, dim3((unsigned)rows), dim3(1024), 0, s, bsum, prefix, nblk,
                        static_cast<const double *>(babs), refine, n);
     // one refinement of the prediction (see quantum_of)
-#ifdef REPDL_DEBUG_HOOKS
-    if (!g_debug_norefine)
-#endif
-    {
-    hipLaunchKernelGGL(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(prefix), bsum, babs,
-                       static_cast<const int *>(refine), vec);
-    hipLaunchKernelGGL(sum1d_prefix_kernel, dim3((unsigned)rows), dim3(1024), 0, s, bsum, prefix, nblk,
-                       static_cast<const double *>(nullptr), refine, n);
-    }
-    hipLaunchKernelGGL(sum1d_tuple_kernel, g2, dim3(256), 0, s, in, c, prefix, T1, TG, T2, vec);
-    hipLaunchKernelGGL(sum1d_super_kernel, dim3((unsigned)repdl_cdiv(nsup, 4), (unsigned)rows), dim3(256), 0, s, T2, TN, T3, ctl,
+    REPDL_LAUNCH(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(prefix), bsum, babs,
+                 static_cast<const int *>(refine), vec);
+    REPDL_LAUNCH(sum1d_prefix_kernel, dim3((unsigned)rows), dim3(1024), 0, s, bsum, prefix, nblk,
+                 static_cast<const double *>(nullptr), refine, n);
+    REPDL_LAUNCH(sum1d_tuple_kernel, g2, dim3(256), 0, s, in, c, prefix, T1, TG, T2, vec);
+    REPDL_LAUNCH(sum1d_super_kernel, dim3((unsigned)repdl_cdiv(nsup, 4), (unsigned)rows), dim3(256), 0, s, T2, TN, T3, ctl,
                        work, nblk, nnode, nsup);
     const int rounds = spec_rounds(rows, n);
+    repdl_route_note(rounds > 0 ? REPDL_ROUTE_SUM_CHAINS_ROUNDS : REPDL_ROUTE_SUM_CHAINS);
     if (rounds > 0)
     {
         float *sc = reinterpret_cast<float *>(w + l.sc);
@@ -1657,21 +1633,21 @@ int repdl_sum_chains(const float *in, float *out, int64_t rows, int64_t nseg, in
         for (int r = 0; r < rounds; r++)
         {
             const int cur = r & 1, old = cur ^ 1;
-            hipLaunchKernelGGL(sum1d_plan_kernel, dim3((unsigned)nsup, (unsigned)rows), dim3(64), 0, s, prefix, TN, ctl, sc, hc, SA, sbase,
+            REPDL_LAUNCH(sum1d_plan_kernel, dim3((unsigned)nsup, (unsigned)rows), dim3(64), 0, s, prefix, TN, ctl, sc, hc, SA, sbase,
                                nbase[old], tab[old], nbase[cur], tab[cur], worklist, work, nblk, nnode, nsup, r);
             const int64_t walkers = nnode * rows < 1024 ? nnode * rows : 1024; // four workgroups per CU
-            hipLaunchKernelGGL(sum1d_cand_walk_kernel, dim3((unsigned)walkers), dim3(256), 0, s, in, c, T1, TG, T2, nbase[cur], tab[cur],
+            REPDL_LAUNCH(sum1d_cand_walk_kernel, dim3((unsigned)walkers), dim3(256), 0, s, in, c, T1, TG, T2, nbase[cur], tab[cur],
                                worklist, work, nnode, (int)(nnode * rows), r, vec);
-            hipLaunchKernelGGL(sum1d_compose_kernel, dim3((unsigned)nsup, (unsigned)rows), dim3(256), 0, s, nbase[cur], tab[cur], ctl,
+            REPDL_LAUNCH(sum1d_compose_kernel, dim3((unsigned)nsup, (unsigned)rows), dim3(256), 0, s, nbase[cur], tab[cur], ctl,
                                SE, SA, SOK, sbase, nnode, nsup);
-            hipLaunchKernelGGL(sum1d_compose2_kernel, dim3((unsigned)nhyp, (unsigned)rows), dim3(256), 0, s, SE, SA, SOK, sbase, ctl, HE,
+            REPDL_LAUNCH(sum1d_compose2_kernel, dim3((unsigned)nhyp, (unsigned)rows), dim3(256), 0, s, SE, SA, SOK, sbase, ctl, HE,
                                HA, HOK, hbase, nsup, nhyp);
-            hipLaunchKernelGGL(sum1d_resolve_kernel, dim3((unsigned)rows), dim3(256), 0, s, HE, HA, HOK, hbase, SE, SA, SOK, sbase, sc,
+            REPDL_LAUNCH(sum1d_resolve_kernel, dim3((unsigned)rows), dim3(256), 0, s, HE, HA, HOK, hbase, SE, SA, SOK, sbase, sc,
                                hc, ctl, factor, out, nsup, nhyp);
         }
     }
     // whatever the rounds left (everything, without rounds), from the front
-    hipLaunchKernelGGL(sum1d_walk_kernel, dim3((unsigned)rows), dim3(64), 0, s, in, c, T1, TG, T2, T3, ctl, factor, out, vec);
+    REPDL_LAUNCH(sum1d_walk_kernel, dim3((unsigned)rows), dim3(64), 0, s, in, c, T1, TG, T2, T3, ctl, factor, out, vec);
     return repdl_launch_status();
 }
 
@@ -1771,35 +1747,3 @@ REPDL_API int repdl_hip_sum1d_static(const float *in, float *out, int64_t n, int
     return repdl_hip_sum1d_ws(in, out, n, average, ptr, STATIC_SCRATCH_BYTES, stream);
 }
 
-#ifdef REPDL_DEBUG_HOOKS
-// Development only (not built into the library): force the number of rounds, read a row's front.
-REPDL_API void repdl_debug_sum1d_rounds(int r) { g_debug_rounds = r; }
-REPDL_API void repdl_debug_sum1d_norefine(int v) { g_debug_norefine = v; }
-REPDL_API int repdl_debug_sum1d_front(const void *workspace, int64_t n)
-{
-    const Layout l = layout(1, n);
-    Ctl c;
-    hipDeviceSynchronize();
-    hipMemcpy(&c, static_cast<const char *>(workspace) + l.ctl, sizeof(c), hipMemcpyDeviceToHost);
-    return c.front;
-}
-REPDL_API void repdl_debug_sum1d_counts(unsigned long long *c, int reset)
-{
-    hipDeviceSynchronize();
-    hipMemcpyFromSymbol(c, HIP_SYMBOL(g_dbg), sizeof(g_dbg));
-    if (reset)
-    {
-        unsigned long long z[8] = {};
-        hipMemcpyToSymbol(HIP_SYMBOL(g_dbg), z, sizeof(z));
-    }
-}
-REPDL_API void repdl_debug_sum1d_work(const void *workspace, int64_t n, int *counts)
-{
-    const Layout l = layout(1, n);
-    Work w[MAX_ROUNDS];
-    hipDeviceSynchronize();
-    hipMemcpy(w, static_cast<const char *>(workspace) + l.work, sizeof(w), hipMemcpyDeviceToHost);
-    for (int i = 0; i < MAX_ROUNDS; i++)
-        counts[i] = w[i].count + w[i].light;
-}
-#endif

@@ -25,9 +25,9 @@ def test_library_exports_every_declared_symbol():
     assert len(names) >= 17
     for n in names:
         assert hasattr(lib, n), n
-    other = {"repdl_hip_error_string", "repdl_hip_abi_version", "repdl_hip_sum1d_workspace_bytes",
-             "repdl_hip_matrix_path", "repdl_hip_init", "repdl_hip_sum1d_static_max_n"}
-    assert set(_lib.SIGNATURES) | other == set(names)
+    other = {"repdl_hip_error_string", "repdl_hip_abi_version", "repdl_hip_matrix_path", "repdl_hip_init",
+             "repdl_hip_sum1d_static_max_n", "repdl_hip_routes_taken", "repdl_hip_route_name"}
+    assert set(_lib.SIGNATURES) | set(_lib.SIZE_QUERIES) | other == set(names)
 
 
 def test_abi_version_and_error_strings():

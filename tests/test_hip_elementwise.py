@@ -62,6 +62,17 @@ def test_div_mix_and_specials():
     assert _same_bits(ops.div(a[1:1001].cuda(), b[3:1003].cuda()), oracle.div(a[1:1001], b[3:1003]))
 
 
+def test_div_tensor_by_tensor_at_full_size():
+    """The 2^28-element launch of the elementwise configuration (x / y, both from the value mix), every
+    output against the oracle and against PyTorch CPU's x.div(y), which is what RepDL's div is
+    (repdl/ops.py:98-103)."""
+    n = 1 << 28
+    a, b = gen.elementwise_mix(3, n), gen.elementwise_mix(4, n)
+    got = _ops().div(a.cuda(), b.cuda()).cpu()
+    assert _same_bits(got, oracle.div(a, b))
+    assert _same_bits(got, a.div(b))
+
+
 def test_sqrt_matches_torch_cpu_convention():
     ops = _ops()
     x = gen.elementwise_mix(15, 1 << 20)

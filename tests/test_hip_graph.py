@@ -55,3 +55,64 @@ def test_graph_replays_match_eager():
         torch.cuda.synchronize()
         for g, wnt in zip(got, want):
             assert torch.equal(g.view(torch.int32), wnt.view(torch.int32)), rep
+
+
+_FRESH_CAPTURE = r"""
+import sys, torch
+sys.path.insert(0, {root!r}); sys.path.insert(0, {root!r} + "/tests")
+import gen
+import repdl_amd
+from repdl_amd import ops
+from repdl_amd.backend import hip
+
+dev = torch.device("cuda:0")
+repdl_amd.init()                        # the device check cannot run under capture; nothing else has run
+N, IC, H, W, OC = 8, 64, 28, 28, 128
+x = torch.relu(gen.normal_like(1, N, IC, H, W)).to(dev)
+w3 = gen.normal_like(2, OC, IC, 3, 3).to(dev)       # 3x3 at stride 2: a padded copy, residues, padded rows in scratch
+go3 = gen.normal_like(3, N, OC, 14, 14).to(dev)
+w1 = gen.normal_like(4, IC, IC, 3, 3).to(dev)       # 3x3 at stride 1: guard words, the transposed kernel
+go1 = gen.normal_like(5, N, IC, H, W).to(dev)
+bias = gen.normal_like(6, OC).to(dev)
+
+def step():
+    return (ops.conv2d_bias(x, w3, bias, (2, 2), (1, 1), 1),
+            ops.conv2d_grad_input((N, IC, H, W), w3, go3, (2, 2), (1, 1)),
+            ops.conv2d_grad_kernel(x, (OC, IC, 3, 3), go3, (2, 2), (1, 1)),
+            ops.conv2d(x, w1, (1, 1), (1, 1), 1),
+            ops.conv2d_grad_input((N, IC, H, W), w1, go1, (1, 1), (1, 1)),
+            ops.conv2d_grad_kernel(x, (IC, IC, 3, 3), go1, (1, 1), (1, 1)),
+            ops.sum4d_dim023(go1.expand(N, IC, H, W).repeat(8, 1, 2, 1)))   # chains of 100352: the parallel evaluation
+
+graph = torch.cuda.CUDAGraph()
+with torch.cuda.graph(graph):           # the first call of every operator in this process
+    captured = step()
+for rep in range(3):
+    x.copy_(torch.relu(gen.normal_like(10 + rep, N, IC, H, W)).to(dev))
+    go1.copy_(gen.normal_like(20 + rep, N, IC, H, W).to(dev))
+    graph.replay()
+    torch.cuda.synchronize()
+    got = [t.clone() for t in captured]
+    want = step()                       # eager work between the replays
+    torch.cuda.synchronize()
+    for i, (g, wnt) in enumerate(zip(got, want)):
+        assert torch.equal(g.view(torch.int32), wnt.view(torch.int32)), (rep, i)
+from repdl_amd import _lib
+assert _lib.lib().repdl_hip_scratch_bytes() == 0    # the bindings bring their own scratch: the cache was never used
+print("fresh-capture ok", hip.BINDING)
+"""
+
+
+def test_convolutions_captured_in_a_fresh_process():
+    """Forward, grad-input and grad-kernel of two layers and a channel sum, captured into a graph as the first
+    calls of a new process -- no warm-up, so nothing the operators need may be allocated, freed or kept by the
+    library: their scratch comes from PyTorch's allocator through the *_ws entry points -- and replayed to the
+    eager bits."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, "-c", _FRESH_CAPTURE.format(root=root)], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert "fresh-capture ok" in proc.stdout
