@@ -293,7 +293,9 @@ def leg_entry(name, workload, bound, work, fn, steps, warmup, parity, cpu, traff
 
 LINE_LIMIT = 7000  # bytes of the printed line: harnesses that keep only the tail of stdout must still see every leg
 DETAIL_JSON = os.path.join(ROOT, "gpurun_out", "bench_detail.json")
-ALSO_UNITS = {"hbm": {"unit": "GB/s", "peak": HBM_PEAK_GBS}, "mfma": {"unit": "TFLOP/s", "peak": FP32_PEAK_TFLOPS}}
+# per bound of a secondary leg: unit and peak of its `roofline.achieved`, unit of its `cpu_baseline.value` (unless the leg names another)
+ALSO_UNITS = {"hbm": {"unit": "GB/s", "peak": HBM_PEAK_GBS, "cpu_unit": "GB/s"},
+              "mfma": {"unit": "TFLOP/s", "peak": FP32_PEAK_TFLOPS, "cpu_unit": "GFLOP/s"}}
 
 
 def compact_leg(e):
@@ -307,7 +309,9 @@ def compact_leg(e):
         out["equal"] = e["parity"].get("equal")
     c = e.get("cpu_baseline")
     if c is not None:
-        out["cpu_baseline"] = {"value": sig4(c["value"]), "unit": c["unit"], "cores": c["cores"], "kind": c["kind"], "sample": c["short"]}
+        out["cpu_baseline"] = {"value": sig4(c["value"]), "cores": c["cores"], "kind": c["kind"], "sample": c["short"]}
+        if c["unit"] != ALSO_UNITS[r["bound"]]["cpu_unit"]:
+            out["cpu_baseline"]["unit"] = c["unit"]
     return out
 
 
@@ -445,7 +449,6 @@ def main() -> int:
                      "note": kernel_note},
         "cpu_baseline": cpu_baseline,
         "parity": parity,
-        "also_settle_ms": SETTLE_MS,
         "also": [],
     }
     if traffic is None:
