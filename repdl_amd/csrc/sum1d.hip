@@ -374,17 +374,33 @@ __global__ __launch_bounds__(1024) void sum1d_prefix_kernel(const double *__rest
     bool want = false;
     double carry = 0.0;
     int par = 0;
+    // (the loads of a tile are issued one tile ahead: the loop is a chain of scans and barriers, and a
+    // tile's round trip to memory in front of each -- 65536 sums, eight tiles -- made it 86 us long)
+    double nv[PER], na[PER];
+    auto request = [&](int64_t base) {
+        const int64_t i0 = base + (int64_t)tid * PER;
+#pragma unroll
+        for (int d = 0; d < PER; d++)
+        {
+            nv[d] = i0 + d < nblk ? bsum[i0 + d] : 0.0;
+            na[d] = babs != nullptr && i0 + d < nblk ? babs[i0 + d] : 0.0;
+        }
+    };
+    request(0);
     for (int64_t base = 0; base < nblk; base += PER * 1024)
     {
         const int64_t i0 = base + (int64_t)tid * PER;
-        double v[PER];
+        double v[PER], ab[PER];
         double tot = 0.0;
 #pragma unroll
         for (int d = 0; d < PER; d++)
         {
-            v[d] = i0 + d < nblk ? bsum[i0 + d] : 0.0;
+            v[d] = nv[d];
+            ab[d] = na[d];
             tot += v[d];
         }
+        if (base + PER * 1024 < nblk) // (uniform)
+            request(base + PER * 1024);
         double inc = tot;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1)
@@ -414,7 +430,7 @@ __global__ __launch_bounds__(1024) void sum1d_prefix_kernel(const double *__rest
                 if (babs != nullptr)
                 {
                     const int64_t left = n - (i0 + d) * BLK; // elements of this block (the last one may be short)
-                    want = want || quantum_of(run).q * 32.0 * (double)(left < BLK ? left : BLK) >= babs[i0 + d];
+                    want = want || quantum_of(run).q * 32.0 * (double)(left < BLK ? left : BLK) >= ab[d];
                 }
             }
             run += v[d];
@@ -1491,9 +1507,7 @@ inline size_t round256(size_t v) { return (v + 255) & ~(size_t)255; }
 // serial single-chain kernel of sum.hip
 int repdl_sum1d_serial(const float *in, float *out, int64_t n, int average, void *stream);
 
-// Number of speculative rounds for `rows` chains of n elements (0: step 4 alone).  Rounds pay
-// from a few million elements on; chains that come in rows are short and many, and their walks
-// already run side by side.
+// Number of speculative rounds for `rows` chains of n elements (0: step 4 alone).
 static int spec_rounds(int64_t rows, int64_t n)
 {
     // Chains that come in rows: three rounds when the chains are very long and their nodes few enough
@@ -1507,8 +1521,16 @@ static int spec_rounds(int64_t rows, int64_t n)
     // longer waited for every workspace: they fill the chip that the other streams' kernels would use.)
     if (rows > 1)
         return (n >= ((int64_t)1 << 19) && rows * repdl_cdiv(repdl_cdiv(n, BLK), NODEB) <= 3200) ? 3 : 0;
-    if (n < ((int64_t)1 << 22))
+    // A single chain: two rounds from 2^18 elements on.  The lone walk of step 4 on zero-mean data takes
+    // 0.54 / 0.62 / 0.81 / 1.07 ms at 2^18 / 2^19 / 2^20 / 2^21 elements (it grows with the length, and 2^22
+    // with four rounds takes 0.36); after two rounds it is 0.20 / 0.21 / 0.21 / 0.22 ms.  Chains that drift
+    // pay the rounds' ten launches: 0.044 / 0.056 / 0.062 / 0.070 -> 0.09 / 0.08 / 0.085 / 0.09 ms.  (At 2^17
+    // elements: 0.27 -> 0.20 against 0.04 -> 0.07, and the mean of a cross_entropy over that many rows is of
+    // the drifting kind: not there.  Three rounds instead of two: 0.01 ms slower both ways.)
+    if (n < ((int64_t)1 << 18))
         return 0;
+    if (n < ((int64_t)1 << 22))
+        return 2;
     return n < ((int64_t)1 << 24) ? 4 : (n < ((int64_t)1 << 26) ? 8 : MAX_ROUNDS);
 }
 
