@@ -72,7 +72,7 @@ LEG_KERNELS = {
     "conv3x3_dgrad": {"kernels": ["conv_tapdma_prep_kernel", "conv_tapdma_kernel<1,"]},
     "conv3x3_wgrad": {"kernels": ["conv_wgrad_mfma_kernel<14, 1, 8, 32, false>"]},
     "conv1x1_fwd": {"kernels": ["mm_dma_kernel<false, false, 2, 2, 2, 2, 4"]},
-    "conv1x1_dgrad": {"kernels": ["conv_point_prep_kernel", "conv_point_kernel<1>"]},
+    "conv1x1_dgrad": {"kernels": ["conv_point_kernel<1>"]},
     "conv1x1_wgrad": {"kernels": ["conv_wgrad_mfma_kernel<14, 1, 8, 16, true>"]},
     "adam_step": {"kernels": ["adam_kernel"]},
 }
