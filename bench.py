@@ -292,7 +292,7 @@ def leg_entry(name, workload, bound, work, fn, steps, warmup, parity, cpu, traff
 
 
 LINE_LIMIT = 7000  # bytes of the printed line: harnesses that keep only the tail of stdout must still see every leg
-DETAIL_JSON = os.path.join(ROOT, "gpurun_out", "bench_detail.json")
+DETAIL_JSON = os.environ.get("REPDL_BENCH_DETAIL", "bench_detail.json")  # every leg in full (digests, notes), beside the printed line
 # per bound of a secondary leg: unit and peak of its `roofline.achieved`, unit of its `cpu_baseline.value` (unless the leg names another)
 ALSO_UNITS = {"hbm": {"unit": "GB/s", "peak": HBM_PEAK_GBS, "cpu_unit": "GB/s"},
               "mfma": {"unit": "TFLOP/s", "peak": FP32_PEAK_TFLOPS, "cpu_unit": "GFLOP/s"}}
@@ -330,7 +330,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=10)  # 77 ms of headline launches: the first tens of ms after idle are not steady state
     ap.add_argument("--quick", action="store_true", help="headline only, no secondary operators, no full parity")
-    ap.add_argument("--only", default="", help="comma list of secondary legs to run (mm1024,mm_fma,sum2d,sum2d_dim0,sum4d,sum1d,"
+    ap.add_argument("--only", default="", help="comma list of secondary legs to run (mm1024,mm64,mm_fma,sum2d,sum2d_dim0,sum4d,sum1d,"
                                                "exp,log,sqrt,div,loss,conv,linear,adam,cnn)")
     ap.add_argument("--size", type=int, default=8192, help="mm size (M=N=K); the metric is quoted at 8192")
     ap.add_argument("--copy-probe", action="store_true",
@@ -484,6 +484,23 @@ def main() -> int:
             cpu = {"value": round(2.0 * 1024 ** 3 / dt / 1e9, 3), "unit": "GFLOP/s", "cores": cores, "kind": kind, "sample": "the full product", "short": "full"}
             also.append(leg_entry("mm", "1024x1024x1024 NN, N(0,1) entries (configs[0])", "mfma", 2.0 * 1024 ** 3, f, args.steps * 4, args.warmup, par, cpu, "mm1024",
                                   short="1024^3 NN cfg0"))
+            del a_d, b_d
+
+        if want("mm64"):
+            # a Linear layer at batch 64: 64 output rows, every SIMD one chain of dependent matrix instructions
+            g = torch.Generator().manual_seed(15)
+            a_h = torch.randn(64, 4096, generator=g)
+            b_h = (torch.rand(4096, 4096, generator=g) * 2 - 1) / 64.0
+            a_d, b_d = a_h.to(dev), b_h.to(dev)
+            hold = {}
+            def f(): hold["y"] = ops.mm(a_d, b_d, False, True)
+            f()
+            dt, y_cpu = cpu_time(lambda: (refmods[0].mm(a_h, b_h, False, True) if refmods else oracle.mm(a_h, b_h, False, True)))
+            par = {"equal": sha(hold["y"]) == sha(y_cpu), "sha256_gpu": sha(hold["y"])}
+            cpu = {"value": round(2.0 * 64 * 4096 * 4096 / dt / 1e9, 3), "unit": "GFLOP/s", "cores": cores, "kind": kind, "sample": "the full product",
+                   "short": "full"}
+            also.append(leg_entry("mm", "64x4096x4096 NT (nn.Linear forward at batch 64)", "mfma", 2.0 * 64 * 4096 * 4096, f, args.steps * 4, args.warmup,
+                                  par, cpu, short="64x4096x4096 NT"))
             del a_d, b_d
 
         if want("sum2d"):
@@ -775,7 +792,8 @@ def main() -> int:
         torch.cuda.synchronize()
 
     try:
-        os.makedirs(os.path.dirname(DETAIL_JSON), exist_ok=True)
+        if os.path.dirname(DETAIL_JSON):
+            os.makedirs(os.path.dirname(DETAIL_JSON), exist_ok=True)
         with open(DETAIL_JSON, "w") as f:
             json.dump(result, f, indent=1)
             f.write("\n")
