@@ -116,3 +116,48 @@ def test_convolutions_captured_in_a_fresh_process():
     proc = subprocess.run([sys.executable, "-c", _FRESH_CAPTURE.format(root=root)], capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     assert "fresh-capture ok" in proc.stdout
+
+
+def test_training_step_captured():
+    """A whole training step of the 2-conv + 2-FC CNN -- forward, loss, backward with its side streams, the fused
+    SGD update -- captured into one graph (the operators bring their scratch from PyTorch's allocator, so nothing in
+    it allocates behind PyTorch's back) and replayed: three eager steps, the capture, three replays give the weights
+    of six eager steps, bit for bit."""
+    import models
+    import repdl_amd
+
+    dev = torch.device("cuda:0")
+    repdl_amd.init()
+    x, y = models.images(21, 64).to(dev), gen.labels(22, 64, 10).to(dev)
+    lossf = repdl_amd.nn.CrossEntropyLoss()
+
+    def make():
+        m = repdl_amd.from_torch_module(models.cnn(0)).to(dev)
+        return m, repdl_amd.optim.SGD(m.parameters(), 0.01)
+
+    def step(m, opt):
+        opt.zero_grad(set_to_none=True)
+        lossf(m(x), y).backward()
+        opt.step()
+
+    m, opt = make()
+    for _ in range(6):
+        step(m, opt)
+    want = repdl_amd.utils.get_hash(m)
+
+    m2, opt2 = make()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step(m2, opt2)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    opt2.zero_grad(set_to_none=True)
+    with torch.cuda.graph(graph):
+        lossf(m2(x), y).backward()
+        opt2.step()
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    assert repdl_amd.utils.get_hash(m2) == want
