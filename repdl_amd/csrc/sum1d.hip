@@ -304,16 +304,19 @@ __device__ __forceinline__ double quantise(float x, const Quantum &g)
 // prev == nullptr: exact sums, and the sums of the magnitudes in babs; else: sums of the elements
 // rounded to the grid of the state prev[block] predicted by the previous pass -- unless that pass
 // found the refinement pointless for this row (refine[row] == 0: nothing is read, bsum stays).
+// The first pass clears refine[row] for the prefix launch that follows it.
 __global__ __launch_bounds__(256) void sum1d_blocksum_kernel(const float *__restrict__ x, Chains c,
                                                              const double *__restrict__ prev,
                                                              double *__restrict__ bsum, double *__restrict__ babs,
-                                                             const int *__restrict__ refine, int vec)
+                                                             int *__restrict__ refine, int vec)
 {
     __shared__ double part[2][4];
     const int tid = threadIdx.x;
     const int64_t row = blockIdx.y;
     if (prev != nullptr && refine[row] == 0)
         return;
+    if (prev == nullptr && blockIdx.x == 0 && tid == 0)
+        refine[row] = 0;
     x += row * c.row_stride;
     bsum += row * c.nblk;
     float v[16];
@@ -346,106 +349,118 @@ __global__ __launch_bounds__(256) void sum1d_blocksum_kernel(const float *__rest
     }
 }
 
-// ---- step 2: exclusive prefix of the block sums (one workgroup per row) --------------------
-// Tiles of 8192 sums: a thread owns eight consecutive ones, the workgroup scans the thread totals.
+// ---- step 2: exclusive prefix of the block sums -----------------------------------------------
+// grid (tiles of 4096 sums, rows).  A workgroup first adds up everything before its tile (a plain
+// reduction, every read coalesced; the order is fixed, so the prediction is the same on every run),
+// then scans the tile: a thread owns four consecutive sums, the workgroup scans the thread totals.
+// Memory is touched in rows of 64 consecutive sums per wave (512 contiguous bytes per instruction) and
+// the rows are turned into four-per-thread through LDS, each wave in its own 2 KiB: a thread that
+// loaded and stored its own sums directly made every instruction touch 64 separate lines, and one
+// workgroup walking all the tiles of a chain of 2^28 elements one after the other took 80 us.
 // First pass (babs given): also decides whether the refinement pass is worth its read of the input,
-// refine[row] = 1 if some block enters at a state whose grid is within 2^5 of the block's mean
-// magnitude -- where elements lose bits that matter, or vanish, the chain drifts away from the exact
-// sum systematically (a sum of 2^28 values in [0,1) stalls at 2^24) and only the refined prediction
-// follows it; where the grid is far finer than the elements the rounding errors have no direction
-// and the rounds re-centre the windows anyway.  Either answer gives the same result: the prediction
-// only places the candidate windows.  Second pass (babs null): nothing to do if refine[row] == 0.
+// refine[row] = 1 (it was cleared by the block-sum launch before) if some block enters at a state
+// whose grid is within 2^5 of the block's mean magnitude -- where elements lose bits that matter, or
+// vanish, the chain drifts away from the exact sum systematically (a sum of 2^28 values in [0,1) stalls
+// at 2^24) and only the refined prediction follows it; where the grid is far finer than the elements the
+// rounding errors have no direction and the rounds re-centre the windows anyway.  Either answer gives
+// the same result: the prediction only places the candidate windows.  Second pass (babs null): nothing
+// to do if refine[row] == 0.
+constexpr int PREFIX_TILE = 4096;
+
 __global__ __launch_bounds__(1024) void sum1d_prefix_kernel(const double *__restrict__ bsum,
                                                             double *__restrict__ prefix, int64_t nblk,
                                                             const double *__restrict__ babs, int *__restrict__ refine, int64_t n)
 {
-    constexpr int PER = 8;
+    constexpr int PER = PREFIX_TILE / 1024;
+    __shared__ __attribute__((aligned(16))) double stage[16][64 * PER];
     __shared__ double wsum[2][16];
-    __shared__ int want_s;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    if (babs == nullptr && refine[blockIdx.x] == 0)
+    const int64_t row = blockIdx.y, base = (int64_t)blockIdx.x * PREFIX_TILE;
+    if (babs == nullptr && refine[row] == 0)
         return;
-    bsum += (int64_t)blockIdx.x * nblk; // one workgroup per row
-    prefix += (int64_t)blockIdx.x * nblk;
+    bsum += row * nblk;
+    prefix += row * nblk;
     if (babs != nullptr)
-        babs += (int64_t)blockIdx.x * nblk;
-    if (tid == 0)
-        want_s = 0;
-    bool want = false;
-    double carry = 0.0;
-    int par = 0;
-    // (the loads of a tile are issued one tile ahead: the loop is a chain of scans and barriers, and a
-    // tile's round trip to memory in front of each -- 65536 sums, eight tiles -- made it 86 us long)
-    double nv[PER], na[PER];
-    auto request = [&](int64_t base) {
-        const int64_t i0 = base + (int64_t)tid * PER;
+        babs += row * nblk;
+    double *const mine = stage[wave];
+    // this tile, requested before the reduction below
+    double rv[PER], ra[PER];
 #pragma unroll
-        for (int d = 0; d < PER; d++)
-        {
-            nv[d] = i0 + d < nblk ? bsum[i0 + d] : 0.0;
-            na[d] = babs != nullptr && i0 + d < nblk ? babs[i0 + d] : 0.0;
-        }
-    };
-    request(0);
-    for (int64_t base = 0; base < nblk; base += PER * 1024)
+    for (int r = 0; r < PER; r++)
     {
-        const int64_t i0 = base + (int64_t)tid * PER;
-        double v[PER], ab[PER];
-        double tot = 0.0;
-#pragma unroll
-        for (int d = 0; d < PER; d++)
-        {
-            v[d] = nv[d];
-            ab[d] = na[d];
-            tot += v[d];
-        }
-        if (base + PER * 1024 < nblk) // (uniform)
-            request(base + PER * 1024);
-        double inc = tot;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1)
-        {
-            const double o = __shfl_up(inc, off, 64);
-            if (lane >= off)
-                inc += o;
-        }
-        if (lane == 63)
-            wsum[par][wave] = inc;
-        __syncthreads(); // (the other half of wsum is not written before everyone has passed the next barrier)
-        double before = 0.0, total = 0.0;
-#pragma unroll
-        for (int w = 0; w < 16; w++)
-        {
-            const double t = wsum[par][w];
-            before += w < wave ? t : 0.0;
-            total += t;
-        }
-        double run = carry + before + (inc - tot);
-#pragma unroll
-        for (int d = 0; d < PER; d++)
-        {
-            if (i0 + d < nblk)
-            {
-                prefix[i0 + d] = run;
-                if (babs != nullptr)
-                {
-                    const int64_t left = n - (i0 + d) * BLK; // elements of this block (the last one may be short)
-                    want = want || quantum_of(run).q * 32.0 * (double)(left < BLK ? left : BLK) >= ab[d];
-                }
-            }
-            run += v[d];
-        }
-        carry += total;
-        par ^= 1;
+        const int64_t i = base + wave * (64 * PER) + r * 64 + lane;
+        rv[r] = i < nblk ? bsum[i] : 0.0;
+        ra[r] = babs != nullptr && i < nblk ? babs[i] : 0.0;
     }
-    if (babs != nullptr)
-    {
-        if (want)
-            want_s = 1; // (same value from every writer)
+    // everything before the tile
+    double part = 0.0;
+    for (int64_t i = tid; i < base; i += 1024)
+        part += bsum[i];
+    part = wave_sum(part);
+    if (lane == 0)
+        wsum[0][wave] = part;
+    // rows of 64 (register r: the wave's sum r * 64 + lane) to four consecutive per thread
+    auto to_consecutive = [&](const double(&rows)[PER], double(&own)[PER]) {
+#pragma unroll
+        for (int r = 0; r < PER; r++)
+            mine[r * 64 + lane] = rows[r];
         __syncthreads();
-        if (tid == 0)
-            refine[blockIdx.x] = want_s;
+#pragma unroll
+        for (int d = 0; d < PER; d++)
+            own[d] = mine[lane * PER + d];
+        __syncthreads();
+    };
+    const int64_t i0 = base + (int64_t)tid * PER;
+    double v[PER], ab[PER];
+    to_consecutive(rv, v); // (its barriers also publish wsum[0])
+    if (babs != nullptr)   // (uniform)
+        to_consecutive(ra, ab);
+    double carry = 0.0;
+#pragma unroll
+    for (int w = 0; w < 16; w++)
+        carry += wsum[0][w];
+    double tot = 0.0;
+#pragma unroll
+    for (int d = 0; d < PER; d++)
+        tot += v[d];
+    double inc = tot;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1)
+    {
+        const double o = __shfl_up(inc, off, 64);
+        if (lane >= off)
+            inc += o;
     }
+    if (lane == 63)
+        wsum[1][wave] = inc;
+    __syncthreads();
+    double before = 0.0;
+#pragma unroll
+    for (int w = 0; w < 16; w++)
+        before += w < wave ? wsum[1][w] : 0.0;
+    double run = carry + before + (inc - tot);
+    bool want = false;
+#pragma unroll
+    for (int d = 0; d < PER; d++)
+    {
+        mine[lane * PER + d] = run;
+        if (babs != nullptr && i0 + d < nblk)
+        {
+            const int64_t left = n - (i0 + d) * BLK; // elements of this block (the last one may be short)
+            want = want || quantum_of(run).q * 32.0 * (double)(left < BLK ? left : BLK) >= ab[d];
+        }
+        run += v[d];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < PER; r++)
+    {
+        const int64_t i = base + wave * (64 * PER) + r * 64 + lane;
+        if (i < nblk)
+            prefix[i] = mine[r * 64 + lane];
+    }
+    if (babs != nullptr && want)
+        refine[row] = 1; // (same value from every writer, in this workgroup and the others)
 }
 
 // ---- step 3: chunk and block tuples --------------------------------------------------------
@@ -1052,6 +1067,12 @@ __global__ __launch_bounds__(64) void sum1d_plan_kernel(const double *__restrict
     const int64_t n0 = sb * NPS;
     const int cnt = nnode - n0 < NPS ? (int)(nnode - n0) : NPS;
     float centre = 0.0f; // lane i: node n0 + i
+    // Later rounds chain through tables -- the approximate offsets of the super-blocks before this one in
+    // its hyper-block, then the previous round's tables of its own nodes.  All of them come into LDS first,
+    // in one round trip: read where they lie, every step of the chain was a trip to memory of its own.
+    __shared__ __attribute__((aligned(16))) float lsa[HB - 1][CAND];
+    __shared__ __attribute__((aligned(16))) uint32_t ltab[NPS][CAND];
+    __shared__ uint32_t lsb[HB], lnb[NPS];
     if (round == 0)
     {
         if (lane < cnt)
@@ -1059,26 +1080,36 @@ __global__ __launch_bounds__(64) void sum1d_plan_kernel(const double *__restrict
     }
     else
     {
+        const bool near_front = sb / HB == front / HB;
+        const int64_t jh = sb / HB * HB;
+        const int before = near_front ? 0 : (int)(sb - jh);
+#pragma unroll
+        for (int j = 0; j < HB - 1; j++)
+            if (j < before)
+                reinterpret_cast<uint4 *>(lsa[j])[lane] = reinterpret_cast<const uint4 *>(SA + (jh + j) * CAND)[lane];
+#pragma unroll
+        for (int i = 0; i < NPS; i++)
+            if (i < cnt)
+                reinterpret_cast<uint4 *>(ltab[i])[lane] = reinterpret_cast<const uint4 *>(tab_old + (n0 + i) * CAND)[lane];
+        if (lane < before)
+            lsb[lane] = sbase[jh + lane];
+        if (lane < cnt)
+            lnb[lane] = nbase_old[n0 + lane];
         // (wave-uniform chain)  The resolver left a centre for every super-block of the hyper-block
         // the front lies in, and for the first super-block of every later hyper-block; from
         // there the centre goes through the approximate offsets of the super-blocks before this one.
-        double sa;
-        if (sb / HB == front / HB)
-            sa = (double)sc[sb];
-        else
+        double sa = near_front ? (double)sc[sb] : (double)hc[sb / HB];
+        __syncthreads();
+        for (int j = 0; j < before; j++)
         {
-            sa = (double)hc[sb / HB];
-            for (int64_t j = sb / HB * HB; j < sb; j++)
-            {
-                bool hit;
-                const uint32_t idx = nearest_candidate(__float_as_uint((float)sa), sbase[j], hit);
-                sa += (double)SA[j * CAND + idx];
-            }
+            bool hit;
+            const uint32_t idx = nearest_candidate(__float_as_uint((float)sa), lsb[j], hit);
+            sa += (double)lsa[j][idx];
         }
         for (int i = 0; i < cnt; i++)
         {
             centre = lane == i ? (float)sa : centre;
-            sa = approx_step(sa, nbase_old[n0 + i], tab_old + (n0 + i) * CAND);
+            sa = approx_step(sa, lnb[i], ltab[i]);
         }
     }
     int kind = -1; // 0: keep the old table, 1: the node's own map, 2: walk
@@ -1095,7 +1126,7 @@ __global__ __launch_bounds__(64) void sum1d_plan_kernel(const double *__restrict
         const uint32_t e0 = base + (base & 1u), e1 = base + CAND - 2 + (base & 1u);
         const uint32_t o0 = base + 1 - (base & 1u), o1 = base + CAND - 1 - (base & 1u);
         const bool whole = e0 >= ln.smin0 && e1 <= ln.smax0 && o0 >= ln.smin1 && o1 <= ln.smax1 && e1 >= e0 && o1 >= o0;
-        kind = (round != 0 && nbase_old[n0 + lane] == base) ? 0 : (whole ? 1 : 2);
+        kind = (round != 0 && lnb[lane] == base) ? 0 : (whole ? 1 : 2);
         if (kind == 2)
         {
             const int gn = (int)(row * nnode + n0 + lane);
@@ -1117,7 +1148,7 @@ __global__ __launch_bounds__(64) void sum1d_plan_kernel(const double *__restrict
         {
             const int c = q * 64 + lane;
             const uint32_t st = b + (uint32_t)c;
-            tab_new[(n0 + i) * CAND + c] = k == 0 ? tab_old[(n0 + i) * CAND + c] : st + (uint32_t)((st & 1u) ? a1 : a0);
+            tab_new[(n0 + i) * CAND + c] = k == 0 ? ltab[i][c] : st + (uint32_t)((st & 1u) ? a1 : a0);
         }
     }
 }
@@ -1136,12 +1167,17 @@ __global__ __launch_bounds__(256) void sum1d_cand_walk_kernel(
     __shared__ int item_s;
     const int tid = threadIdx.x;
     const int front_count = work[round].count, count = front_count + work[round].light;
-    for (;;)
+    // A workgroup's first node is the one of its own index, the later ones come off a counter: a round
+    // with nothing (or little) left to walk costs the idle workgroups no atomic -- a thousand of them on
+    // one address were 12 us of every such round.
+    for (bool first = true;; first = false)
     {
-        if (tid == 0)
-            item_s = atomicAdd(&work[round].next, 1);
+        if (first && (int)blockIdx.x >= count) // (uniform)
+            break;
+        if (!first && tid == 0)
+            item_s = (int)gridDim.x + atomicAdd(&work[round].next, 1);
         __syncthreads();
-        const int item = item_s;
+        const int item = first ? (int)blockIdx.x : item_s;
         __syncthreads(); // (everyone has read item_s, and has finished with the LDS of the previous node)
         if (item >= count)
             break;
@@ -1227,14 +1263,26 @@ __global__ __launch_bounds__(256) void sum1d_compose_kernel(const uint32_t *__re
     SA += (row * nsup + sb) * CAND;
     SOK += (row * nsup + sb) * (CAND / 32);
     const int64_t n0 = sb * NPS;
-    const uint32_t base0 = nbase[n0];
+    const int cnt = nnode - n0 < NPS ? (int)(nnode - n0) : NPS;
+    // the tables of the super-block's nodes, brought into LDS together: the chain below is then sixteen
+    // LDS reads in a row instead of sixteen round trips to memory
+    __shared__ uint32_t ltab[NPS][CAND];
+    __shared__ uint32_t lbase[NPS];
+#pragma unroll
+    for (int i = 0; i < NPS; i++)
+        if (i < cnt)
+            ltab[i][tid] = tab[(n0 + i) * CAND + tid];
+    if (tid < cnt)
+        lbase[tid] = nbase[n0 + tid];
+    __syncthreads();
+    const uint32_t base0 = lbase[0];
     uint32_t y = base0 + (uint32_t)tid; // exact while ok
     bool ok = true;
     double sa = 0.0; // the approximate state once a window was missed
-    for (int i = 0; i < NPS && n0 + i < nnode; i++)
+    for (int i = 0; i < cnt; i++)
     {
-        const uint32_t b = nbase[n0 + i];
-        const uint32_t *t = tab + (n0 + i) * CAND;
+        const uint32_t b = lbase[i];
+        const uint32_t *t = ltab[i];
         if (ok)
         {
             const uint32_t d = y - b;
@@ -1284,19 +1332,37 @@ __global__ __launch_bounds__(256) void sum1d_compose2_kernel(const uint32_t *__r
     HA += (row * nhyp + h) * CAND;
     HOK += (row * nhyp + h) * (CAND / 32);
     const int64_t j0 = h * HB > front ? h * HB : front, j1 = (h + 1) * HB < nsup ? (h + 1) * HB : nsup;
-    const uint32_t base0 = sbase[j0];
+    const int cnt = (int)(j1 - j0);
+    // the tables of the hyper-block's super-blocks in LDS (as in sum1d_compose_kernel)
+    __shared__ uint32_t lse[HB][CAND];
+    __shared__ float lsa[HB][CAND];
+    __shared__ uint32_t lok[HB][CAND / 32];
+    __shared__ uint32_t lbase[HB];
+#pragma unroll
+    for (int i = 0; i < HB; i++)
+        if (i < cnt)
+        {
+            lse[i][tid] = SE[(j0 + i) * CAND + tid];
+            lsa[i][tid] = SA[(j0 + i) * CAND + tid];
+        }
+    if (tid < cnt * (CAND / 32))
+        lok[tid / (CAND / 32)][tid % (CAND / 32)] = SOK[j0 * (CAND / 32) + tid];
+    else if (tid >= 128 && tid < 128 + cnt)
+        lbase[tid - 128] = sbase[j0 + tid - 128];
+    __syncthreads();
+    const uint32_t base0 = lbase[0];
     uint32_t y = base0 + (uint32_t)tid; // exact while ok
     bool ok = true;
     double sa = 0.0;
-    for (int64_t j = j0; j < j1; j++)
+    for (int i = 0; i < cnt; i++)
     {
-        const uint32_t b = sbase[j];
+        const uint32_t b = lbase[i];
         if (ok)
         {
             const uint32_t d = y - b;
-            if (d < (uint32_t)CAND && ((SOK[j * (CAND / 32) + (d >> 5)] >> (d & 31u)) & 1u) != 0u)
+            if (d < (uint32_t)CAND && ((lok[i][d >> 5] >> (d & 31u)) & 1u) != 0u)
             {
-                y = SE[j * CAND + d];
+                y = lse[i][d];
                 continue;
             }
             ok = false;
@@ -1304,7 +1370,7 @@ __global__ __launch_bounds__(256) void sum1d_compose2_kernel(const uint32_t *__r
         }
         bool hit;
         const uint32_t idx = nearest_candidate(__float_as_uint((float)sa), b, hit);
-        sa += (double)SA[j * CAND + idx];
+        sa += (double)lsa[i][idx];
     }
     const double entry = (double)__uint_as_float(base0 + (uint32_t)tid);
     HE[tid] = y;
@@ -1625,15 +1691,13 @@ int repdl_sum_chains(const float *in, float *out, int64_t rows, int64_t nseg, in
     const dim3 g2((unsigned)nblk, (unsigned)rows);
     double *babs = reinterpret_cast<double *>(w + l.babs);
     int *refine = reinterpret_cast<int *>(w + l.refine);
-    REPDL_LAUNCH(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(nullptr), bsum, babs,
-                       static_cast<const int *>(refine), vec);
-    REPDL_LAUNCH(sum1d_prefix_kernel, dim3((unsigned)rows), dim3(1024), 0, s, bsum, prefix, nblk,
-                       static_cast<const double *>(babs), refine, n);
+    REPDL_LAUNCH(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(nullptr), bsum, babs, refine, vec);
+    REPDL_LAUNCH(sum1d_prefix_kernel, dim3((unsigned)repdl_cdiv(nblk, PREFIX_TILE), (unsigned)rows), dim3(1024), 0, s, bsum, prefix,
+                 nblk, static_cast<const double *>(babs), refine, n);
     // one refinement of the prediction (see quantum_of)
-    REPDL_LAUNCH(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(prefix), bsum, babs,
-                 static_cast<const int *>(refine), vec);
-    REPDL_LAUNCH(sum1d_prefix_kernel, dim3((unsigned)rows), dim3(1024), 0, s, bsum, prefix, nblk,
-                 static_cast<const double *>(nullptr), refine, n);
+    REPDL_LAUNCH(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(prefix), bsum, babs, refine, vec);
+    REPDL_LAUNCH(sum1d_prefix_kernel, dim3((unsigned)repdl_cdiv(nblk, PREFIX_TILE), (unsigned)rows), dim3(1024), 0, s, bsum, prefix,
+                 nblk, static_cast<const double *>(nullptr), refine, n);
     REPDL_LAUNCH(sum1d_tuple_kernel, g2, dim3(256), 0, s, in, c, prefix, T1, TG, T2, vec);
     REPDL_LAUNCH(sum1d_super_kernel, dim3((unsigned)repdl_cdiv(nsup, 4), (unsigned)rows), dim3(256), 0, s, T2, TN, T3, ctl,
                        work, nblk, nnode, nsup);
