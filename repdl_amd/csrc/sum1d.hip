@@ -467,7 +467,7 @@ __global__ __launch_bounds__(1024) void sum1d_prefix_kernel(const double *__rest
 __global__ __launch_bounds__(256) void sum1d_tuple_kernel(const float *__restrict__ x, Chains c,
                                                           const double *__restrict__ prefix,
                                                           Tup *__restrict__ T1, Tup *__restrict__ TG,
-                                                          Tup *__restrict__ T2, int vec)
+                                                          Tup *__restrict__ T2, int vec, int self_prefix)
 {
     __shared__ double wtot[4];
     __shared__ Tup wt[4];
@@ -481,9 +481,49 @@ __global__ __launch_bounds__(256) void sum1d_tuple_kernel(const float *__restric
     float v[16];
     load16(x, c, blk * BLK + tid * 16, vec, v);
 
+    // The state predicted at the block start.  self_prefix (one short unsegmented chain): the block
+    // adds up everything before it in binary64 itself -- at most 63 blocks, from the cache -- which
+    // saves the four launches of steps 1 and 2 where a launch is longer than its work.  (Any fixed
+    // order serves: the value only predicts.)
+    double pstart;
+    if (self_prefix)
+    {
+        const int64_t e0 = blk * BLK;
+        double p = 0.0;
+        if (vec)
+        {
+            // (e0 is a multiple of 4096: four loads in flight per thread, four partial sums)
+            double p4[4] = {0.0, 0.0, 0.0, 0.0};
+            for (int64_t i = (int64_t)tid * 4; i < e0; i += 4096)
+            {
+                float4 f[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+                    f[u] = *reinterpret_cast<const float4 *>(x + i + 1024 * u);
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+                    p4[u] += ((double)f[u].x + (double)f[u].y) + ((double)f[u].z + (double)f[u].w);
+            }
+            p = (p4[0] + p4[1]) + (p4[2] + p4[3]);
+        }
+        else
+        {
+            for (int64_t i = tid; i < e0; i += 256)
+                p += (double)x[i];
+        }
+        p = wave_sum(p);
+        if (lane == 0)
+            wtot[wave] = p;
+        __syncthreads();
+        pstart = (wtot[0] + wtot[1]) + (wtot[2] + wtot[3]);
+        __syncthreads(); // (wtot is used again below)
+    }
+    else
+        pstart = prefix[blk];
+
     // binary64 exclusive prefix over the threads of the block (elements on the grid of the
     // state predicted for the block start, as in the refined block sums)
-    const Quantum g = quantum_of(prefix[blk]);
+    const Quantum g = quantum_of(pstart);
     double d = 0.0;
     bool finite = true, allzero = true;
 #pragma unroll
@@ -505,7 +545,7 @@ __global__ __launch_bounds__(256) void sum1d_tuple_kernel(const float *__restric
     if (lane == 63)
         wtot[wave] = inc;
     __syncthreads();
-    double base = prefix[blk];
+    double base = pstart;
     for (int w = 0; w < wave; w++)
         base += wtot[w];
     const double excl = base + (inc - d);
@@ -813,7 +853,7 @@ __global__ __launch_bounds__(64) void sum1d_walk_kernel(const float *__restrict_
                                                         const Tup *__restrict__ T2,
                                                         const Tup *__restrict__ T3,
                                                         const Ctl *__restrict__ ctl, float factor,
-                                                        float *__restrict__ out, int vec)
+                                                        float *__restrict__ out, int vec, int inline_super)
 {
     __shared__ __attribute__((aligned(16))) float xd[BLK + 2 * CH]; // + what the read-ahead overshoots
     const int lane = threadIdx.x;
@@ -826,16 +866,29 @@ __global__ __launch_bounds__(64) void sum1d_walk_kernel(const float *__restrict_
     out += row;
     // Where the speculative rounds got to (super-block `first`, state there); 0 and +0.0f
     // without rounds; nothing to do if they resolved the whole chain.
-    const int64_t first = __builtin_amdgcn_readfirstlane(ctl[row].front);
+    // inline_super (a chain of one super-block, walked from its start at +0.0f): T3 and ctl have not been
+    // written -- the launch of step 3b is saved -- and the super-block's tuple is joined here.
+    const int64_t first = inline_super ? 0 : __builtin_amdgcn_readfirstlane(ctl[row].front);
     if (first >= nsup)
         return;
-    uint32_t s = __builtin_amdgcn_readfirstlane(ctl[row].s); // wave-uniform throughout
+    uint32_t s = inline_super ? 0u : __builtin_amdgcn_readfirstlane(ctl[row].s); // wave-uniform throughout
     BlockRegs pf;                                            // the block requested ahead
     int64_t pf_blk = -1;
     load_block(pf, x, c, T1, TG, 0, lane, vec); // (any valid block: the registers are then defined)
     pf_blk = 0;
     const int64_t gfirst = first & ~(int64_t)63;
-    Tup nsup_t = (gfirst + lane < nsup) ? T3[gfirst + lane] : tup_identity(HYP_ANY);
+    Tup nsup_t = tup_identity(HYP_ANY);
+    if (inline_super)
+    {
+        Tup t = lane < nblk ? T2[lane] : tup_identity(HYP_ANY);
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1)
+            t = tup_join(t, tup_shfl_down(t, off)); // lane 0: the blocks in order
+        if (lane == 0)
+            nsup_t = t;
+    }
+    else if (gfirst + lane < nsup)
+        nsup_t = T3[gfirst + lane];
     // block tuples of the super-block being tried, and of the next one
     Tup blk_next = (first * SUP + lane < nblk) ? T2[first * SUP + lane] : tup_identity(HYP_ANY);
     for (int64_t g0 = gfirst; g0 < nsup; g0 += 64)
@@ -860,6 +913,9 @@ __global__ __launch_bounds__(64) void sum1d_walk_kernel(const float *__restrict_
             if (walk_apply(s, lsh, i & 31))
                 continue;
             const WalkTup lb = walk_tup(lane_tup(blk_cur));
+            // blocks of this super-block with a chunk whose map does not even hold for the predicted state:
+            // the ones that will most likely fail as wholes, and so the ones to request ahead
+            const unsigned long long expect_fail = __ballot(blk_cur.heavy > 0);
             for (int hb = 0; hb < SUP / 32; hb++)
             {
             const WalkHalf lbh = hb ? lb.B : lb.A;
@@ -878,7 +934,10 @@ __global__ __launch_bounds__(64) void sum1d_walk_kernel(const float *__restrict_
                 const WalkTup lg = walk_tup(lane_tup(pf.tgr)), lc = walk_tup(lane_tup(pf.tch));
                 __syncthreads();
                 {
-                    const int64_t nb = blk + 1 < nblk ? blk + 1 : blk;
+                    const int bi = 32 * hb + b5;
+                    const unsigned long long later = bi < 63 ? expect_fail >> (bi + 1) : 0ull;
+                    int64_t nb = later != 0ull ? blk + 1 + __builtin_ctzll(later) : blk + 1;
+                    nb = nb < nblk ? nb : blk;
                     load_block(pf, x, c, T1, TG, nb, lane, vec);
                     pf_blk = nb;
                 }
@@ -1691,6 +1750,16 @@ int repdl_sum_chains(const float *in, float *out, int64_t rows, int64_t nseg, in
     const dim3 g2((unsigned)nblk, (unsigned)rows);
     double *babs = reinterpret_cast<double *>(w + l.babs);
     int *refine = reinterpret_cast<int *>(w + l.refine);
+    const int rounds = spec_rounds(rows, n);
+    // One short chain: two launches instead of seven (the map pass makes its own prediction, the walk joins
+    // the one super-block's tuple itself).  65536 elements: 0.040 -> 0.016 ms.
+    if (rows == 1 && nseg == 1 && rounds == 0 && nsup == 1)
+    {
+        repdl_route_note(REPDL_ROUTE_SUM_CHAINS);
+        REPDL_LAUNCH(sum1d_tuple_kernel, g2, dim3(256), 0, s, in, c, prefix, T1, TG, T2, vec, 1);
+        REPDL_LAUNCH(sum1d_walk_kernel, dim3(1), dim3(64), 0, s, in, c, T1, TG, T2, T3, ctl, factor, out, vec, 1);
+        return repdl_launch_status();
+    }
     REPDL_LAUNCH(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(nullptr), bsum, babs, refine, vec);
     REPDL_LAUNCH(sum1d_prefix_kernel, dim3((unsigned)repdl_cdiv(nblk, PREFIX_TILE), (unsigned)rows), dim3(1024), 0, s, bsum, prefix,
                  nblk, static_cast<const double *>(babs), refine, n);
@@ -1698,10 +1767,9 @@ int repdl_sum_chains(const float *in, float *out, int64_t rows, int64_t nseg, in
     REPDL_LAUNCH(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(prefix), bsum, babs, refine, vec);
     REPDL_LAUNCH(sum1d_prefix_kernel, dim3((unsigned)repdl_cdiv(nblk, PREFIX_TILE), (unsigned)rows), dim3(1024), 0, s, bsum, prefix,
                  nblk, static_cast<const double *>(nullptr), refine, n);
-    REPDL_LAUNCH(sum1d_tuple_kernel, g2, dim3(256), 0, s, in, c, prefix, T1, TG, T2, vec);
+    REPDL_LAUNCH(sum1d_tuple_kernel, g2, dim3(256), 0, s, in, c, prefix, T1, TG, T2, vec, 0);
     REPDL_LAUNCH(sum1d_super_kernel, dim3((unsigned)repdl_cdiv(nsup, 4), (unsigned)rows), dim3(256), 0, s, T2, TN, T3, ctl,
                        work, nblk, nnode, nsup);
-    const int rounds = spec_rounds(rows, n);
     repdl_route_note(rounds > 0 ? REPDL_ROUTE_SUM_CHAINS_ROUNDS : REPDL_ROUTE_SUM_CHAINS);
     if (rounds > 0)
     {
@@ -1733,7 +1801,7 @@ int repdl_sum_chains(const float *in, float *out, int64_t rows, int64_t nseg, in
         }
     }
     // whatever the rounds left (everything, without rounds), from the front
-    REPDL_LAUNCH(sum1d_walk_kernel, dim3((unsigned)rows), dim3(64), 0, s, in, c, T1, TG, T2, T3, ctl, factor, out, vec);
+    REPDL_LAUNCH(sum1d_walk_kernel, dim3((unsigned)rows), dim3(64), 0, s, in, c, T1, TG, T2, T3, ctl, factor, out, vec, 0);
     return repdl_launch_status();
 }
 
