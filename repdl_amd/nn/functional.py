@@ -42,16 +42,56 @@ def linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tenso
 
 
 _SIDE_STREAMS = {}
+_DEFER_STREAMS = {}
+_DEFERRED = {}
+_DEFER_POOL = 3  # side streams that deferred jobs rotate over (with the current stream: the four hardware queues of a process)
+defer_parameter_gradients = True  # False: every job of _side_by_side is joined where it was started
+deferred_stats = {"jobs": 0, "copies_rewritten": 0}  # (for tests: how often each path was taken)
 
 
-def _side_by_side(device: torch.device, jobs):
+def _deferrable(param: Optional[torch.Tensor]) -> bool:
+    """Whether the gradient of `param` may still be in flight on a side stream when the backward
+    function that made it returns.  It may if nothing reads it before the backward pass ends: the
+    tensor is a leaf without hooks whose .grad is empty -- autograd then keeps the gradient tensor
+    itself, or a copy that _join_deferred() makes again once the gradient is complete -- and no
+    graph is being recorded through the backward pass.  Code that reads parameter gradients DURING
+    the backward pass by other means (hooks on autograd nodes) sets defer_parameter_gradients = False."""
+    return (defer_parameter_gradients and param is not None and param.is_leaf and param.grad is None
+            and param.is_contiguous() and not torch.is_grad_enabled() and not param._backward_hooks
+            and not getattr(param, "_post_accumulate_grad_hooks", None))
+
+
+def _join_deferred(key: int) -> None:
+    """End of a backward pass: the current stream waits for the deferred jobs, and a parameter whose
+    .grad is not the job's own tensor (autograd copied it, possibly before it was complete) gets
+    the finished values."""
+    pending = _DEFERRED.pop(key, None)
+    if pending is None:
+        return
+    cur = torch.cuda.current_stream(key)
+    for st in pending["streams"]:
+        cur.wait_stream(st)
+    for param, grad in pending["grads"]:
+        if param.grad is not None and param.grad.data_ptr() != grad.data_ptr():
+            param.grad.copy_(grad)
+            deferred_stats["copies_rewritten"] += 1
+
+
+def _side_by_side(device: torch.device, jobs, defer=None, reads=(), params=None):
     """Runs independent jobs (callables returning a tensor, or None for "not needed") and
     returns their results in order.  On the GPU the first needed job runs on the current
     stream and the others on side streams of their own (default priority, made once per
     device), so that they overlap: the reductions and the grad-kernel of a backward pass are
     chains as long as the batch -- bound by the latency of one chain, busy on a fraction of
     the CUs -- and side by side they take the time of the longest instead of the sum.
-    The results are what the jobs return one after the other: the jobs are independent."""
+    The results are what the jobs return one after the other: the jobs are independent.
+
+    defer[i] (only inside a backward pass; job i makes the gradient of params[i], and the caller
+    has asked _deferrable(params[i])): the result is not waited for here but when the backward
+    pass ends (a callback queued with the autograd engine), so that the current stream goes on with
+    the next layer's backward while a grad-kernel chain of this one is still running.  Such jobs
+    take turns on a small pool of streams, and `reads` -- the tensors they read -- are kept from
+    reuse until those streams are done with them."""
     todo = [i for i, j in enumerate(jobs) if j is not None]
     out = [None] * len(jobs)
     if device.type != "cuda" or len(todo) < 2:
@@ -59,16 +99,38 @@ def _side_by_side(device: torch.device, jobs):
             out[i] = jobs[i]()
         return out
     key = device.index if device.index is not None else torch.cuda.current_device()
-    streams = _SIDE_STREAMS.setdefault(key, [])
-    while len(streams) < len(todo) - 1:
-        streams.append(torch.cuda.Stream(device=key))
     cur = torch.cuda.current_stream(key)
-    for st, i in zip(streams, todo[1:]):
+    late = [i for i in todo[1:] if defer is not None and defer[i]]
+    side = [i for i in todo[1:] if i not in late]
+    streams = _SIDE_STREAMS.setdefault(key, [])
+    while len(streams) < len(side):
+        streams.append(torch.cuda.Stream(device=key))
+    for st, i in zip(streams, side):
         st.wait_stream(cur)  # the inputs are complete
         with torch.cuda.stream(st):
             out[i] = jobs[i]()
+    if late:
+        pool = _DEFER_STREAMS.setdefault(key, {"streams": [], "next": 0})
+        while len(pool["streams"]) < _DEFER_POOL:
+            pool["streams"].append(torch.cuda.Stream(device=key))
+        pending = _DEFERRED.setdefault(key, {"streams": [], "grads": []})
+        # (one callback per call: whichever runs first joins everything that is pending, the others find nothing)
+        torch.autograd.Variable._execution_engine.queue_callback(lambda: _join_deferred(key))
+        for i in late:
+            st = pool["streams"][pool["next"] % _DEFER_POOL]
+            pool["next"] += 1
+            st.wait_stream(cur)
+            with torch.cuda.stream(st):
+                out[i] = jobs[i]()
+            for t in reads:
+                t.record_stream(st)
+            out[i].record_stream(cur)
+            if st not in pending["streams"]:
+                pending["streams"].append(st)
+            deferred_stats["jobs"] += 1
+            pending["grads"].append((params[i], out[i].detach()))  # (an alias: the result itself stays autograd's alone)
     out[todo[0]] = jobs[todo[0]]()
-    for st, i in zip(streams, todo[1:]):
+    for st, i in zip(streams, side):
         cur.wait_stream(st)  # later work on the current stream sees the result, and the inputs are
         out[i].record_stream(cur)  # not reused before the side stream is done with them
     return out
@@ -79,6 +141,7 @@ class _Conv2d(torch.autograd.Function):
     def forward(ctx, x, weight, bias, stride, padding, groups):
         ctx.save_for_backward(x, weight)
         ctx.conf = (stride, padding, groups)
+        ctx.params = (weight, bias)  # (the parameters themselves, for their .grad and hooks)
         return ops.conv2d_bias(x, weight, bias, stride=stride, padding=padding, groups=groups)
 
     @staticmethod
@@ -89,10 +152,13 @@ class _Conv2d(torch.autograd.Function):
         x, weight = ctx.saved_tensors
         need_x, need_w, need_b = ctx.needs_input_grad[:3]
         # grad-input fills the chip; grad-kernel and the bias sum are latency-bound chains: side by side
+        # (the chains of the parameters' gradients need not end before the next layer's backward starts)
         gx, gw, gb = _side_by_side(gy.device, [
             (lambda: ops.conv2d_grad_input(x.shape, weight, gy, stride, padding)) if need_x else None,
             (lambda: ops.conv2d_grad_kernel(x, weight.shape, gy, stride, padding)) if need_w else None,
-            (lambda: ops.sum4d_dim023(gy)) if need_b else None])
+            (lambda: ops.sum4d_dim023(gy)) if need_b else None],
+            defer=(False, need_x and _deferrable(ctx.params[0]), need_x and _deferrable(ctx.params[1])), reads=(x, gy),
+            params=(None,) + ctx.params)
         return gx, gw, gb, None, None, None
 
 

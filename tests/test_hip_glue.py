@@ -140,3 +140,73 @@ def test_backward_streams_repeated():
         assert torch.equal(gamma.grad, ops.sum4d_dim023(ops.div(y.detach() - pc(mean.detach()), pc(std).expand_as(y)) * go)), it
         coef = ops.div(gamma.detach(), 2 * std * std * std)
         assert torch.equal(var.grad, ops.sum4d_dim023(go * (pc(mean.detach()) - y.detach()) * pc(coef))), it
+
+
+def _two_conv_grads(defer, accumulate=False, hook=False, keep=None):
+    """Gradients of a two-layer convolution stack (the first layer's parameter gradients can be
+    deferred: its input needs a gradient too) after one or two backward passes."""
+    from repdl_amd.nn import functional as F
+
+    old = F.defer_parameter_gradients
+    F.defer_parameter_gradients = defer
+    try:
+        x = gen.relu_like(41, 8, 3, 24, 24).cuda().requires_grad_(True)
+        w1 = (gen.normal_like(42, 16, 3, 3, 3) * 0.2).cuda().requires_grad_(True)
+        b1 = gen.normal_like(43, 16).cuda().requires_grad_(True)
+        w2 = (gen.normal_like(44, 8, 16, 3, 3) * 0.1).cuda().requires_grad_(True)
+        b2 = gen.normal_like(45, 8).cuda().requires_grad_(True)
+        seen = []
+        if hook:
+            w1.register_hook(lambda g: seen.append(g.clone()))
+        go = gen.normal_like(46, 8, 8, 24, 24).cuda()
+        for _ in range(2 if accumulate else 1):
+            y = F.conv2d(torch.relu(F.conv2d(x, w1, b1, 1, 1)), w2, b2, 1, 1)
+            y.backward(go)
+        torch.cuda.synchronize()
+        out = [t.grad.clone() for t in (x, w1, b1, w2, b2)] + seen
+        if keep is not None:
+            keep.append(w1.grad)
+        return out
+    finally:
+        F.defer_parameter_gradients = old
+
+
+@pytest.mark.parametrize("accumulate,hook", [(False, False), (True, False), (False, True)])
+def test_deferred_parameter_gradients(accumulate, hook):
+    """Parameter gradients whose chains are joined only when the backward pass ends are the bits of
+    the joined-at-once ones: on the first pass (deferred), on a second pass onto existing .grad
+    (not deferred: autograd reads the gradient at once) and with a tensor hook (not deferred)."""
+    from repdl_amd.nn import functional as F
+
+    for _ in range(3):
+        a = _two_conv_grads(False, accumulate, hook)
+        before = F.deferred_stats["jobs"]
+        b = _two_conv_grads(True, accumulate, hook)
+        # weight and bias of both layers on a first pass (a second pass finds .grad filled and defers nothing);
+        # a hook on w1 takes w1 out
+        assert F.deferred_stats["jobs"] - before == (3 if hook else 4)
+        assert len(a) == len(b) and all(torch.equal(p, q) for p, q in zip(a, b))
+
+
+def test_deferred_gradient_that_autograd_copies(monkeypatch):
+    """If something else holds the gradient tensor, autograd stores a copy of it in .grad -- made
+    on the current stream while the chain may still be running on its side stream.  The end-of-pass
+    callback writes the finished values into that copy."""
+    from repdl_amd import ops
+
+    want = _two_conv_grads(False)
+    held = []
+    real = ops.conv2d_grad_kernel
+
+    def holding(*args, **kw):
+        held.append(real(*args, **kw))
+        return held[-1]
+
+    monkeypatch.setattr(ops, "conv2d_grad_kernel", holding)
+    from repdl_amd.nn import functional as F
+
+    kept, before = [], F.deferred_stats["copies_rewritten"]
+    got = _two_conv_grads(True, keep=kept)
+    assert all(torch.equal(p, q) for p, q in zip(want, got))
+    assert all(kept[0].data_ptr() != h.data_ptr() for h in held)  # .grad is a copy, not a held tensor
+    assert F.deferred_stats["copies_rewritten"] - before == 2     # both layers' weights
