@@ -67,6 +67,11 @@ _Mean4dDim023 = _mean_function(
     "Mean4dDim023Function", ops.sum4d_dim023, lambda g, s: g.unsqueeze(-1).unsqueeze(-1).expand(s))
 
 
+# the reference's class names (func.py:11, 47, 72, 98)
+ExpandFunction = _Broadcast
+Mean1dFunction, Mean2dDim0Function, Mean4dDim023Function = _Mean1d, _Mean2dDim0, _Mean4dDim023
+
+
 def mean1d(input: torch.Tensor) -> torch.Tensor:
     assert input.dim() == 1
     return _Mean1d.apply(input)

@@ -211,3 +211,34 @@ def test_readme_initial_model_hash():
     kinds = [type(m).__name__ for m in model.net]
     assert kinds.count("Conv2d") == 2 and kinds.count("Linear") == 3
     assert all(type(m).__module__.startswith("repdl_amd") for m in model.net if type(m).__name__ in ("Conv2d", "Linear"))
+
+
+def test_reference_names_resolve():
+    """Every public name of the reference's Python packages resolves under the same path here
+    (repdl/__init__.py:8-15, func.py, ops.py, optim.py, utils.py, nn/__init__.py:4-8, nn/functional.py:4-7,
+    nn/linear.py, nn/conv.py, nn/loss.py, nn/batchnorm.py)."""
+    import importlib
+
+    names = {
+        "repdl_amd": ["func", "nn", "ops", "optim", "utils", "from_torch_module"],
+        "repdl_amd.ops": ["conv2d", "conv2d_grad_input", "conv2d_grad_kernel", "cross_entropy", "div", "mm", "softmax", "sqrt",
+                          "sum1d", "sum2d_dim0", "sum2d_dim1", "sum4d_dim023"],
+        "repdl_amd.func": ["ExpandFunction", "expand_as", "Mean1dFunction", "mean1d", "Mean2dDim0Function", "mean2d_dim0",
+                           "Mean4dDim023Function", "mean4d_dim023"],
+        "repdl_amd.optim": ["Adam"],
+        "repdl_amd.utils": ["get_hash", "print_hash"],
+        "repdl_amd.nn": ["functional", "BatchNorm1d", "BatchNorm2d", "Conv2d", "Linear", "CrossEntropyLoss"],
+        "repdl_amd.nn.functional": ["batch_norm", "conv2d", "linear", "cross_entropy"],
+        "repdl_amd.nn.linear": ["LinearFunction", "linear", "Linear"],
+        "repdl_amd.nn.conv": ["Conv2dFunction", "conv2d", "Conv2d"],
+        "repdl_amd.nn.loss": ["CrossEntropyFunction", "cross_entropy", "CrossEntropyLoss"],
+        "repdl_amd.nn.batchnorm": ["BatchNormFunction", "batch_norm", "BatchNorm1d", "BatchNorm2d"],
+    }
+    for mod, attrs in names.items():
+        m = importlib.import_module(mod)
+        for a in attrs:
+            assert hasattr(m, a), (mod, a)
+    from repdl_amd.nn.linear import LinearFunction
+
+    assert issubclass(LinearFunction, torch.autograd.Function)
+    assert issubclass(repdl_amd.func.Mean1dFunction, torch.autograd.Function)
