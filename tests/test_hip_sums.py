@@ -51,6 +51,25 @@ def test_sum1d_parallel_path(name, x):
         assert got.view(torch.int32).item() == want.view(torch.int32).item() or (torch.isnan(got) and torch.isnan(want)), (name, avg)
 
 
+@pytest.mark.parametrize("n", [32768, 36865, 65536, 65537, 100_001, 131_072, 200_000, 262_143])
+def test_sum1d_one_short_chain(n):
+    """One chain shorter than 2^18 elements takes two launches (the map pass predicts the state at its own
+    block's start, the walk joins the one super-block's tuple): lengths at and off block boundaries, data that
+    drifts, changes sign and hovers near zero, pointers on and off 16-byte boundaries, sum and mean."""
+    from repdl_amd import ops
+
+    r = _rng(n)
+    kinds = {"zero_mean": r.random(n + 1) * 2 - 1, "drift": r.random(n + 1) * 10 + 2, "normal": r.standard_normal(n + 1),
+             "negative_drift": -r.random(n + 1)}
+    for name, v in kinds.items():
+        h = torch.from_numpy(v.astype(np.float32))
+        d = h.cuda()
+        for off in (0, 1):
+            for avg in (False, True):
+                got, want = ops.sum1d(d[off:], avg).cpu(), oracle.sum1d(h[off:], avg)
+                assert got.view(torch.int32).item() == want.view(torch.int32).item(), (name, off, avg)
+
+
 def test_sum1d_unaligned_and_plain_entry():
     """Unaligned input pointer, and the C entry point without a workspace (which takes
     its scratch from the stream-ordered allocator)."""
