@@ -124,8 +124,10 @@ enum RepdlRoute
     REPDL_ROUTE_MM_UNALIGNED_32,
     REPDL_ROUTE_MM_FMA,
     // conv2d / conv2d_grad_input
-    REPDL_ROUTE_CONV_PATCH_16,   // 3x3 at stride 1 from an input patch in LDS, 16-byte DMA lanes
+    REPDL_ROUTE_CONV_PATCH_16,   // 3x3 at stride 1 from an input patch in LDS, 16-byte DMA lanes, tiles of 64 pixels
     REPDL_ROUTE_CONV_PATCH_4,    // the same with 4-byte lanes
+    REPDL_ROUTE_CONV_PATCH_16_WIDE, // tiles of 128 pixels
+    REPDL_ROUTE_CONV_PATCH_4_WIDE,
     REPDL_ROUTE_CONV_POINT,      // 1x1 at stride 1: both operands streamed
     REPDL_ROUTE_CONV_POINT_MM,   // 1x1 at stride 1: a batch of matrix products per image
     REPDL_ROUTE_CONV_PADDED_64_HALF, // padded copy of the gathered operand, 64-row tiles of 64 pixels

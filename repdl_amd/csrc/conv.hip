@@ -2407,12 +2407,32 @@ int launch_conv_gemm(const float *gathered, const float *kernel, float *out, con
     const bool mfma = repdl_mfma_exact();
     // 3x3 at stride 1: the input-patch kernel (batch 64: 64 -> 64 at 56x56 0.213 -> 0.149 ms, 128 -> 128 at
     // 28x28 0.208 -> 0.143, 256 -> 256 at 14x14 0.28 -> 0.18)
+    // Tiles of 128 pixels (eight waves) or of 64 (four)?  On the wider tile the kernel operand serves twice the
+    // pixels and twice the waves share the DMA -- 3 to 12 % faster where both widths cover the image with the same
+    // waste -- but its last tile of an image wastes more: 28x28 = 784 pixels are 7 tiles of 128 or 13 of 64, and
+    // the narrow tile is 5 % faster there once the launch is large (1664 tiles); small launches take the wide tile
+    // whatever the waste (64 x 64 channels at 28x28, 832 tiles: 11 % faster), images of one narrow tile never (7x7:
+    // 63 % slower).  Measured at batch 64, forward / grad-input alike: 64 -> 64 at 56x56 0.147 -> 0.143 ms, 256 ->
+    // 256 at 14x14 0.167 -> 0.153, 64 -> 64 at 64x64 0.181 -> 0.166, 32 -> 32 at 56x56 0.089 -> 0.081.
+    const int64_t c128 = repdl_cdiv(P, 128), c64 = repdl_cdiv(P, 64);
+    const int64_t tiles64 = c64 * d.N * repdl_cdiv(MODE == MODE_FWD ? d.OC : d.IC, 64);
+    const bool wide = P > 64 && (tiles64 < 1024 || 186 * c128 < 100 * c64);
+    if (mfma && wide && tapdma::applies<MODE>(d, gathered, kernel, 128, 4))
+    {
+        repdl_route_note(REPDL_ROUTE_CONV_PATCH_16_WIDE);
+        return tapdma::launch<MODE, 4, 4>(gathered, kernel, out, d, s);
+    }
     if (mfma && tapdma::applies<MODE>(d, gathered, kernel, 64, 4))
     {
         repdl_route_note(REPDL_ROUTE_CONV_PATCH_16);
         return tapdma::launch<MODE, 2, 4>(gathered, kernel, out, d, s);
     }
     // any other width, 4 bytes per DMA lane
+    if (mfma && wide && tapdma::applies<MODE>(d, gathered, kernel, 128, 1))
+    {
+        repdl_route_note(REPDL_ROUTE_CONV_PATCH_4_WIDE);
+        return tapdma::launch<MODE, 4, 1>(gathered, kernel, out, d, s);
+    }
     if (mfma && tapdma::applies<MODE>(d, gathered, kernel, 64, 1))
     {
         repdl_route_note(REPDL_ROUTE_CONV_PATCH_4);

@@ -108,8 +108,10 @@ def test_mm_tiles(route):
 
 # route -> (which, (N, IC, H, W, OC, KH, KW, sH, sW, pH, pW), matrix path, images the oracle checks)
 CONV = {
-    "conv_patch_16": ("fwd", (2, 32, 20, 24, 64, 3, 3, 1, 1, 1, 1), True, 2),
-    "conv_patch_4": ("dgrad", (3, 64, 14, 14, 64, 3, 3, 1, 1, 1, 1), True, 3),
+    "conv_patch_16": ("fwd", (64, 128, 28, 28, 128, 3, 3, 1, 1, 1, 1), True, 1),  # (a large launch whose wide tiles would waste more)
+    "conv_patch_4": ("dgrad", (3, 64, 7, 7, 64, 3, 3, 1, 1, 1, 1), True, 3),        # (an image of one narrow tile)
+    "conv_patch_16_wide": ("fwd", (2, 32, 20, 24, 64, 3, 3, 1, 1, 1, 1), True, 2),
+    "conv_patch_4_wide": ("dgrad", (3, 64, 14, 14, 64, 3, 3, 1, 1, 1, 1), True, 3),
     "conv_point": ("fwd", (2, 32, 33, 40, 64, 1, 1, 1, 1, 0, 0), True, 2),
     "conv_point_mm": ("dgrad", (3, 128, 33, 40, 192, 1, 1, 1, 1, 0, 0), True, 3),
     "conv_padded_64_half": ("fwd", (2, 32, 19, 19, 64, 3, 3, 2, 2, 1, 1), True, 2),
