@@ -298,9 +298,10 @@ ALSO_UNITS = {"hbm": {"unit": "GB/s", "peak": HBM_PEAK_GBS, "cpu_unit": "GB/s"},
               "mfma": {"unit": "TFLOP/s", "peak": FP32_PEAK_TFLOPS, "cpu_unit": "GFLOP/s"}}
 
 
-def compact_leg(e):
+def compact_leg(e, cores=None):
     """A secondary leg as it is printed: numbers and short labels only.  `roofline.unit` / `roofline.peak` are those of
-    its bound (top-level "also_units"); digests, notes and what limits a leg go to the detail file."""
+    its bound (top-level "also_units"), `cpu_baseline.cores` is "also_units.cpu_cores" unless the leg states another;
+    digests, notes and what limits a leg go to the detail file."""
     r = e["roofline"]
     sig4 = lambda x: x if x is None else float("%.4g" % x)
     out = {"op": e["op"], "wl": e["short"], "ms": e["ms_per_step"],
@@ -309,7 +310,9 @@ def compact_leg(e):
         out["equal"] = e["parity"].get("equal")
     c = e.get("cpu_baseline")
     if c is not None:
-        out["cpu_baseline"] = {"value": sig4(c["value"]), "cores": c["cores"], "kind": c["kind"], "sample": c["short"]}
+        out["cpu_baseline"] = {"value": sig4(c["value"]), "kind": c["kind"], "sample": c["short"]}
+        if c["cores"] != cores:
+            out["cpu_baseline"]["cores"] = c["cores"]
         if c["unit"] != ALSO_UNITS[r["bound"]]["cpu_unit"]:
             out["cpu_baseline"]["unit"] = c["unit"]
     return out
@@ -318,8 +321,9 @@ def compact_leg(e):
 def compact_line(result) -> str:
     """The one printed line: the headline in full, the secondary legs compacted."""
     out = {k: v for k, v in result.items() if k != "also"}
-    out["also_units"] = ALSO_UNITS
-    out["also"] = [compact_leg(e) for e in result["also"]]
+    cores = result["cpu_baseline"]["cores"]
+    out["also_units"] = dict(ALSO_UNITS, cpu_cores=cores)
+    out["also"] = [compact_leg(e, cores) for e in result["also"]]
     return json.dumps(out, separators=(",", ":"))
 
 
@@ -783,6 +787,47 @@ def main() -> int:
                          "cpu_baseline": {"value": round(1.0 / dt, 2), "unit": "steps/s", "cores": cores, "kind": "port",
                                           "sample": "the same step through the same glue with the oracle's operators on CPU tensors",
                                           "short": "same glue on oracle"}})
+
+            # the same step captured into one graph (forward, loss, backward with its side streams, the fused
+            # update) and replayed: what a launch-bound loop costs without its launches
+            mg = repdl_amd.from_torch_module(models.cnn(0)).to(dev)
+            optg = repdl_amd.optim.SGD(mg.parameters(), 0.01)
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(3):  # (eager steps first: the first ones create optimizer state and streams)
+                    optg.zero_grad(set_to_none=True)
+                    lossf(mg(xd), yd).backward()
+                    optg.step()
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            optg.zero_grad(set_to_none=True)
+            with torch.cuda.graph(graph):
+                lossf(mg(xd), yd).backward()
+                optg.step()
+            replays = 0
+
+            def fg():
+                nonlocal replays
+                graph.replay()
+                replays += 1
+
+            wallg, _, _ = time_gpu(fg, args.steps, args.warmup, SETTLE_MS)
+            torch.cuda.synchronize()
+            me = repdl_amd.from_torch_module(models.cnn(0)).to(dev)  # the same number of eager steps
+            opte = repdl_amd.optim.SGD(me.parameters(), 0.01)
+            for _ in range(3 + replays):
+                opte.zero_grad(set_to_none=True)
+                lossf(me(xd), yd).backward()
+                opte.step()
+            also.append({"op": "cnn_step_graph", "workload": "the same training step captured into one graph and replayed",
+                         "short": "one graph replay",
+                         "value": round(1e3 / wallg, 1), "unit": "steps/s", "ms_per_step": round(wallg, 4),
+                         "roofline": {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": None, "traffic": None,
+                                      "traffic_note": "the launches of cnn_step as one graph launch"},
+                         "parity": {"equal": repdl_amd.utils.get_hash(mg) == repdl_amd.utils.get_hash(me), "replays": replays,
+                                    "sha256_weights": repdl_amd.utils.get_hash(mg)},
+                         "cpu_baseline": dict(also[-1]["cpu_baseline"], short="as cnn_step")})
 
     if args.copy_probe:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
