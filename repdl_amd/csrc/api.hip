@@ -8,7 +8,7 @@ namespace
 std::atomic<uint64_t> g_routes{0};
 static_assert(REPDL_ROUTE_COUNT <= 64, "one bit per route");
 const char *const ROUTE_NAMES[REPDL_ROUTE_COUNT] = {
-    "mm_128", "mm_128_tall", "mm_64_four_buffers", "mm_64_three_buffers", "mm_64_movers", "mm_64_quad", "mm_32", "mm_64x32",
+    "mm_128", "mm_128_tall", "mm_64_four_buffers", "mm_64_three_buffers", "mm_64_movers", "mm_64_wide_k", "mm_64_deep", "mm_64_quad", "mm_32", "mm_64x32",
     "mm_unaligned_128", "mm_unaligned_64_movers", "mm_unaligned_64", "mm_unaligned_quad", "mm_unaligned_32", "mm_fma",
     "conv_patch_16", "conv_patch_4", "conv_patch_16_wide", "conv_patch_4_wide", "conv_point", "conv_point_mm", "conv_padded_64_half", "conv_padded_64", "conv_padded_128",
     "conv_gather_64", "conv_gather_128", "conv_im2col", "dgrad_point_scatter", "dgrad_residues",

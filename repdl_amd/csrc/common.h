@@ -114,6 +114,8 @@ enum RepdlRoute
     REPDL_ROUTE_MM_64_FOUR_BUFFERS,  // 64x64, eight waves, four buffers, four moving waves
     REPDL_ROUTE_MM_64_THREE_BUFFERS, // 64x64, eight waves, three buffers
     REPDL_ROUTE_MM_64_MOVERS,        // 64x64, eight waves, three buffers, four moving waves
+    REPDL_ROUTE_MM_64_WIDE_K,        // one 64x64 tile per CU, 513-1024 terms: k-tiles of 64, three buffers, +4
+    REPDL_ROUTE_MM_64_DEEP,          // one 64x64 tile per CU, longer chains: k-tiles of 64, four buffers, operands three quads ahead, +4
     REPDL_ROUTE_MM_64_QUAD,          // 64x64, four waves of 32x32
     REPDL_ROUTE_MM_32,               // 32x32
     REPDL_ROUTE_MM_64X32,            // 64x32

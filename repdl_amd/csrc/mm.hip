@@ -689,6 +689,12 @@ int launch_dma(const float *A, const float *B, float *C, const float *cbias, con
 //     r = 1, 2: 8 waves of 16x32, k-tile 32, four buffers, +4 (1024^2 x 2048: 106 TFLOP/s, against 95 without
 //            the four, 81-83 with four waves of 32x32 or with three buffers; 2048 x 1024 x 2048: 122); chains of
 //            1024 terms and fewer are over before the fourth buffer pays: three buffers, +4 only at r = 1;
+//     r = 1: a CU's one workgroup has the whole LDS, and what it lacks is bytes in flight (16 KB per k-tile of
+//            32, two tiles under way, a microsecond from request to LDS: 32 GB/s per CU, two thirds of what the
+//            chains could take).  k-tiles of 64: three buffers from 513 to 1024 terms (1024^3 0.0246 -> 0.0237 ms), four
+//            and operands read three quads ahead beyond (1024^2 x 2048 -3 %, x 4096 -4 %, x 8192 -7 %; 768 x 1024
+//            x 1024 -18 %).  With two or more tiles per CU the same forms are 10-25 % slower than the ones above:
+//            their 96-128 KB leave room for one workgroup only.
 //     r = 3: 8 waves of 16x32, three buffers (1536 x 2048 x 2048: 127 against 125);
 //     r >= 4: 4 waves of 32x32, k-tile 16, six workgroups to a CU (2048^2 x 2048: 128 against 121);
 //   32x32, 4 waves of one 16x16 block, k-tile 64, read-ahead 7 quads, five buffers, +4: 0.445 at r = 1, 0.52 beyond;
@@ -721,7 +727,7 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
         const int64_t r = rounds(64, 64);
         const double c = (double)r * 4096.0 / (r >= 8 ? 0.92 : r >= 4 ? 0.89 : r == 3 ? 0.875 : r == 2 ? 0.84 : 0.73);
         if (c < best)
-            best = c, pick = r >= 4 ? 3 : r == 3 ? 6 : K > 1024 ? 2 : r == 1 ? 7 : 6;
+            best = c, pick = r >= 4 ? 3 : r == 3 ? 6 : r == 1 ? (K > 1024 ? 8 : K > 512 ? 9 : 7) : K > 1024 ? 2 : 6;
     }
     if (dma_applies<1, 1, 2, 2, 16>(M, N, K, transA, transB, vec4, nbatch))
     {
@@ -745,6 +751,8 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
         case 2:
         case 6:
         case 7:
+        case 8:
+        case 9:
             // one 64x64 tile per CU: eight waves that only move (1001^2 x 2049: 54 TFLOP/s on the
             // four-wave form, 87 with four movers, 96 with eight)
             if (rounds(64, 64) == 1)
@@ -791,6 +799,12 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
     case 7:
         repdl_route_note(REPDL_ROUTE_MM_64_MOVERS);
         return launch_dma<1, 2, 4, 2, 8, 1, 3, 4>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+    case 9:
+        repdl_route_note(REPDL_ROUTE_MM_64_WIDE_K);
+        return launch_dma<1, 2, 4, 2, 16, 1, 3, 4>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
+    case 8:
+        repdl_route_note(REPDL_ROUTE_MM_64_DEEP);
+        return launch_dma<1, 2, 4, 2, 16, 3, 4, 4>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);
     case 4:
         repdl_route_note(REPDL_ROUTE_MM_32);
         return launch_dma<1, 1, 2, 2, 16, 7, 5, 4>(A, B, C, cbias, rbias, M, N, K, transA, transB, nbatch, batch, s);

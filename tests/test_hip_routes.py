@@ -65,7 +65,9 @@ def _restore_matrix_path():
 MM = {
     "mm_128": (2048, 4096, 64, 0, 0),
     "mm_128_tall": (256, 512, 2048, 1, 0),       # chains four times as long as C is wide, both operands row-contiguous... see below
-    "mm_64_four_buffers": (1024, 1024, 2048, 0, 1),
+    "mm_64_four_buffers": (1024, 2048, 2048, 0, 1),
+    "mm_64_deep": (1024, 1024, 2048, 0, 1),
+    "mm_64_wide_k": (1024, 1024, 1000, 1, 0),
     "mm_64_three_buffers": (1024, 2048, 512, 0, 0),
     "mm_64_movers": (1024, 1024, 512, 1, 1),
     "mm_64_quad": (2048, 2048, 64, 0, 1),
