@@ -56,7 +56,7 @@ _S1 = ["sum1d_blocksum_kernel", "sum1d_prefix_kernel", "sum1d_tuple_kernel", "su
 LEG_KERNELS = {
     "mm": {"kernels": ["mm_dma_kernel<false, true, 4, 2, 2, 4, 4"]},
     "mm_fma": {"kernels": ["mm_kernel<false, true"]},
-    "mm1024": {"kernels": ["mm_dma_kernel<false, false, 1, 2, 4, 2, 8"]},
+    "mm1024": {"kernels": ["mm_dma_kernel<false, false, 1, 2, 4, 2, 16, 1, 3"]},
     "sum2d_dim1": {"kernels": ["rowchain_kernel<32, 128, true, false>"]},
     "sum2d_dim0": {"kernels": ["coltile_kernel<16, true, 2>"]},
     "sum4d_dim023": {"kernels": _S1, "grid": 49 * 256 * 64},
