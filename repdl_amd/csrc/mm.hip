@@ -727,7 +727,11 @@ int mm_dma_dispatch(const float *A, const float *B, float *C, const float *cbias
         const int64_t r = rounds(64, 64);
         const double c = (double)r * 4096.0 / (r >= 8 ? 0.92 : r >= 4 ? 0.89 : r == 3 ? 0.875 : r == 2 ? 0.84 : 0.73);
         if (c < best)
-            best = c, pick = r >= 4 ? 3 : r == 3 ? 6 : r == 1 ? (K > 1024 ? 8 : K > 512 ? 9 : 7) : K > 1024 ? 2 : 6;
+        {
+            const bool wide_k = r == 1 && K > 512 && dma_applies<1, 2, 4, 2, 16>(M, N, K, transA, transB, vec4, nbatch);
+            best = c;
+            pick = r >= 4 ? 3 : r == 3 ? 6 : wide_k ? (K > 1024 ? 8 : 9) : K > 1024 ? 2 : r == 1 ? 7 : 6;
+        }
     }
     if (dma_applies<1, 1, 2, 2, 16>(M, N, K, transA, transB, vec4, nbatch))
     {
