@@ -269,7 +269,7 @@ int repdl_hip_softmax(const float *in, float *out, int64_t M, int64_t N, void *s
 /* cross_entropy -- backend/cuda/cross_entropy.cpp:15-24 (bound at :31); semantics
  * backend/cpu/cross_entropy.cpp:15-24.  in is [M,N], target is [M] int64 class
  * indices in [0,N), out is one float.  workspace: M floats of device memory (the row
- * losses; their mean is repdl_hip_sum1d with average = 1, which from 32768 rows on takes
+ * losses; their mean is repdl_hip_sum1d with average = 1, which from 12288 rows on takes
  * its own scratch from the scratch cache as described there). */
 int repdl_hip_cross_entropy(const float *in, const int64_t *target, float *out, int64_t M,
                             int64_t N, float *workspace, void *stream);

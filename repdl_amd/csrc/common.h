@@ -16,8 +16,11 @@
             return REPDL_E_ARG; \
     } while (0)
 
-// Inputs at least this long take the parallel evaluation of the sequential sum.
-#define REPDL_SUM1D_MIN_PARALLEL 32768
+// Inputs at least this long (three blocks) take the parallel evaluation of the sequential sum.  The serial kernel
+// takes 3.3 us per 1000 elements whatever they are; the two launches of the parallel evaluation of one short
+// chain 0.02-0.04 ms up to 16384 elements and 0.03-0.09 up to 32767 (the more the sum hovers near zero), so the
+// two meet at 4096-6000 elements on sums that drift and at 8192-12288 on zero-mean ones.
+#define REPDL_SUM1D_MIN_PARALLEL 12288
 
 // Row and channel sums take the parallel evaluation when the chains are at least this long and
 // at most REPDL_SUM_ROWS_MAX_PARALLEL in number (few long chains are bound by the latency of one

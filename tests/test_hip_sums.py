@@ -35,8 +35,8 @@ def _cases():
     # of the way through, and at 2^22 for the smaller elements that follow a large start
     yield "stagnation", (0.25 + 0.75 * r.random(1 << 25)).astype(np.float32)
     yield "stagnation_small", np.concatenate([[2.0**22], r.random(2_000_000) * 0.25, -r.random(500_000) * 0.3]).astype(np.float32)
-    yield "just_long_enough", gen.uniform_pm1(3, 32768).numpy()
-    yield "just_too_short", gen.uniform_pm1(4, 32767).numpy()
+    yield "just_long_enough", gen.uniform_pm1(3, 12288).numpy()
+    yield "just_too_short", gen.uniform_pm1(4, 12287).numpy()
 
 
 @pytest.mark.parametrize("name,x", list(_cases()), ids=[n for n, _ in _cases()])
@@ -51,7 +51,7 @@ def test_sum1d_parallel_path(name, x):
         assert got.view(torch.int32).item() == want.view(torch.int32).item() or (torch.isnan(got) and torch.isnan(want)), (name, avg)
 
 
-@pytest.mark.parametrize("n", [32768, 36865, 65536, 65537, 100_001, 131_072, 200_000, 262_143])
+@pytest.mark.parametrize("n", [12288, 12289, 16384, 20_000, 32767, 32768, 36865, 65536, 65537, 100_001, 131_072, 200_000, 262_143])
 def test_sum1d_one_short_chain(n):
     """One chain shorter than 2^18 elements takes two launches (the map pass predicts the state at its own
     block's start, the walk joins the one super-block's tuple): lengths at and off block boundaries, data that
