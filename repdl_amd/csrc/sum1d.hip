@@ -1763,6 +1763,16 @@ int repdl_sum_chains(const float *in, float *out, int64_t rows, int64_t nseg, in
     REPDL_LAUNCH(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(nullptr), bsum, babs, refine, vec);
     REPDL_LAUNCH(sum1d_prefix_kernel, dim3((unsigned)repdl_cdiv(nblk, PREFIX_TILE), (unsigned)rows), dim3(1024), 0, s, bsum, prefix,
                  nblk, static_cast<const double *>(babs), refine, n);
+    // Chains of one super-block, walked from their start: four launches instead of seven.  The refinement is for
+    // sums that stall -- elements below half a quantum of the state, which takes 2^24 of them -- and the walk joins
+    // the one super-block's tuple itself (channel sums of [64,128,28,28]: 0.186 -> 0.181 ms, of its ReLU 0.060 -> 0.055).
+    if (rounds == 0 && nsup == 1)
+    {
+        repdl_route_note(REPDL_ROUTE_SUM_CHAINS);
+        REPDL_LAUNCH(sum1d_tuple_kernel, g2, dim3(256), 0, s, in, c, prefix, T1, TG, T2, vec, 0);
+        REPDL_LAUNCH(sum1d_walk_kernel, dim3((unsigned)rows), dim3(64), 0, s, in, c, T1, TG, T2, T3, ctl, factor, out, vec, 1);
+        return repdl_launch_status();
+    }
     // one refinement of the prediction (see quantum_of)
     REPDL_LAUNCH(sum1d_blocksum_kernel, g2, dim3(256), 0, s, in, c, static_cast<const double *>(prefix), bsum, babs, refine, vec);
     REPDL_LAUNCH(sum1d_prefix_kernel, dim3((unsigned)repdl_cdiv(nblk, PREFIX_TILE), (unsigned)rows), dim3(1024), 0, s, bsum, prefix,
