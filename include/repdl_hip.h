@@ -229,7 +229,7 @@ int repdl_hip_sum1d_static(const float *in, float *out, int64_t n, int average, 
 int repdl_hip_sum2d_dim0(const float *in, float *out, int64_t M, int64_t N, int average,
                          void *stream);
 /* sum2d_dim1 and sum4d_dim023 with few long chains (at most 512 chains of at least 49152
- * elements; for sum4d_dim023 also H*W a multiple of 16) take the same parallel evaluation,
+ * elements, or at most 64 of at least 24576; for sum4d_dim023 also H*W a multiple of 16) take the same parallel evaluation,
  * all chains at once, with about half the input's size in bytes from the scratch cache;
  * otherwise they allocate nothing. */
 int repdl_hip_sum2d_dim1(const float *in, float *out, int64_t M, int64_t N, int average,

@@ -418,7 +418,11 @@ static int launch_rowchain(const float *in, float *out, int64_t rows, int64_t ns
     // Few long chains: one lane per chain would be bound by the latency of a chain (8 to 10 clocks
     // per element whatever the data).  The parallel evaluation of sum1d.hip, all chains at once.
     const int64_t len = nseg * seglen;
-    if (rows <= REPDL_SUM_ROWS_MAX_PARALLEL && len >= REPDL_SUM_ROWS_MIN_PARALLEL &&
+    // (At most 64 chains: from half that length on.  There the walks of zero-mean chains take what one lane per
+    // chain takes -- 25088 elements 0.103 ms either way, 48000 0.161 -> 0.141 -- and chains that drift a third of it:
+    // 0.103 -> 0.041, 0.161 -> 0.039.  More chains of that length, or shorter ones, lose up to 75 % on zero-mean data.)
+    const bool long_enough = len >= REPDL_SUM_ROWS_MIN_PARALLEL || (rows <= 64 && len >= REPDL_SUM_ROWS_MIN_PARALLEL / 2);
+    if (rows <= REPDL_SUM_ROWS_MAX_PARALLEL && long_enough &&
         (nseg == 1 || (seglen % 16 == 0 && len <= REPDL_I32_MAX)))
     {
         const size_t bytes = repdl_sum_chains_workspace_bytes(rows, len);

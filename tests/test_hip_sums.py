@@ -135,7 +135,7 @@ def test_channel_sums_unaligned_pointer(shape):
 
 def _long_rows():
     """Few, long chains: row sums and channel sums that take the parallel evaluation (chains of at
-    least 49152 elements, at most 512 of them), with the data that attacks it."""
+    least 49152 elements, at most 512 of them, or at most 64 of at least 24576), with the data that attacks it."""
     r = _rng(12)
     L = 70_000
     rows = [
@@ -160,9 +160,10 @@ def test_row_sums_few_long_rows():
     assert torch.equal(torch.isnan(got), nan) and torch.equal(got[~nan].view(torch.int32), want[~nan].view(torch.int32))
     m2 = gen.scaled_normal(90, 5, 65537)  # a row length that is no multiple of 4: scalar loads
     assert torch.equal(ops.sum2d_dim1(m2.cuda()).cpu(), oracle.sum2d_dim1(m2))
-    for n in (49151, 49152, 49168):  # either side of the length at which rows change kernels
-        m4 = gen.uniform_pm1(92 + n, 3, n)
-        assert torch.equal(ops.sum2d_dim1(m4.cuda()).cpu(), oracle.sum2d_dim1(m4)), n
+    for n in (24575, 24576, 24592, 49151, 49152, 49168):  # either side of the lengths at which rows change kernels
+        for rows in (3, 65):                                 # (up to 64 chains from 24576 elements, up to 512 from 49152)
+            m4 = gen.uniform_pm1(92 + n, rows, n)
+            assert torch.equal(ops.sum2d_dim1(m4.cuda()).cpu(), oracle.sum2d_dim1(m4)), (rows, n)
     m3 = gen.uniform_pm1(91, 300, 66000)
     assert torch.equal(ops.sum2d_dim1(m3.cuda(), average=True).cpu(), oracle.sum2d_dim1(m3, average=True))
 
